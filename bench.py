@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode+matmul hot path on one MI355X.
+
+Headline (the JSON line's `value`): batch-1 decode-GEMV at the Llama-2-70B projection
+shapes.  One step = the four GEMVs (8192->10240, 8192->8192, 8192->28672, 28672->8192), each
+on the next of several distinct code buffers so that the 256 MB Infinity Cache cannot serve
+the weights; `value` is code bytes (N*K/4 per GEMV) per second over the timed region, inputs
+resident in HBM.  `roofline` is the GEMV kernel alone: code bytes per launch over the
+kernel's own duration (HIP events placed around the kernel by the library's timing hook)
+against 8 TB/s.  `prefill` and `small_batch` carry the M=2048 and M=4..32 figures;
+`cpu_baseline` is the torch CPU path on the host cores on one 8192x8192 GEMV.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--quick", action="store_true", help="skip prefill / small-batch / CPU legs")
+    ap.add_argument("--rotate-mb", type=int, default=400, help="distinct code bytes to rotate through, at least")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
+              "use --gpus 1.  DESIGN.md says how the path would shard.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import decode_matmul_amd as dmm
+    from decode_matmul_amd import capi, workload
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the operator has no CPU path", file=sys.stderr)
+        sys.exit(3)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    lib = capi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call(x, codes, grid, scale, y):
+        M, K = x.shape
+        st = lib.dmm_decode_matmul_f16(x.data_ptr(), codes.data_ptr(), grid.data_ptr(), scale, y.data_ptr(),
+                                       M, codes.shape[0], K, stream)
+        if st != 0:
+            raise capi.DmmError("dmm_decode_matmul_f16", st)
+
+    def rand_codes(N, K, copies, seed):
+        # device RNG: uniform over all 65536 code values, `copies` distinct matrices
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        return [torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=dev)
+                for _ in range(copies)]
+
+    # ---------------------------------------------------------------- headline: 70B GEMV
+    shapes = workload.LLAMA2_70B
+    step_bytes = sum(workload.code_bytes(N, K) for K, N in shapes)
+    copies = max(2, -(-args.rotate_mb * 1000000 // step_bytes))
+    probs = []
+    for i, (K, N) in enumerate(shapes):
+        x, _, grid, scale = workload.make_inputs(1, 8, K, seed=0)
+        probs.append(dict(K=K, N=N, x=x.to(dev), grid=grid.to(dev), scale=scale,
+                          codes=rand_codes(N, K, copies, 100 + i),
+                          y=torch.empty(1, N, dtype=torch.float16, device=dev)))
+
+    def step(i):
+        for p in probs:
+            call(p["x"], p["codes"][i % copies], p["grid"], p["scale"], p["y"])
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes * args.steps / wall / 1e9
+
+    # same region again with the kernel's own begin/end events
+    n_launch = args.steps * len(probs)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_launch)]
+    for a, b in ev:
+        a.record(); b.record()
+    torch.cuda.synchronize()
+    j = 0
+    for i in range(args.steps):
+        for p in probs:
+            lib.dmm_set_kernel_events(ev[j][0].cuda_event, ev[j][1].cuda_event)
+            call(p["x"], p["codes"][i % copies], p["grid"], p["scale"], p["y"])
+            j += 1
+    lib.dmm_set_kernel_events(None, None)
+    torch.cuda.synchronize()
+    per_shape = {}
+    j = 0
+    for i in range(args.steps):
+        for p in probs:
+            per_shape.setdefault((p["K"], p["N"]), []).append(ev[j][0].elapsed_time(ev[j][1]) * 1e-3)
+            j += 1
+    kern_s = sum(sum(v) for v in per_shape.values())
+    achieved = step_bytes * args.steps / kern_s / 1e9
+    shape_rows = []
+    for (K, N), v in per_shape.items():
+        avg = sum(v) / len(v)
+        gbs = workload.code_bytes(N, K) / avg / 1e9
+        shape_rows.append({"K": K, "N": N, "code_bytes": workload.code_bytes(N, K), "kernel_us": round(avg * 1e6, 3),
+                           "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
+
+    out = {
+        "metric": "batch-1 effective weight GB/s (code bytes N*K/4 per second, Llama-2-70B projection shapes)",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: batch-1 decode-GEMV, 8192->10240, 8192->8192, 8192->28672, 28672->8192",
+                   "M": 1, "code_buffers_rotated": copies, "distinct_code_MB": round(copies * step_bytes / 1e6, 1),
+                   "step": "4 GEMVs, one per shape"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "dmm::gemv_kernel", "launches": n_launch,
+                     "avg_launch_us": round(kern_s / n_launch * 1e6, 3),
+                     "algorithmic_bytes_per_launch": step_bytes / len(probs)},
+        "gemv_shapes": shape_rows,
+    }
+
+    if not args.quick:
+        out["small_batch"] = small_batch(torch, lib, capi, workload, dev, stream, rand_codes)
+        out["prefill"] = prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes)
+        out["cpu_baseline"] = cpu_baseline(torch, workload)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+def timed_kernel(torch, lib, fn, reps):
+    """Average duration (s) of the library's dominant kernel over `reps` calls of fn(i)."""
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in ev:
+        a.record(); b.record()
+    torch.cuda.synchronize()
+    for i in range(reps):
+        lib.dmm_set_kernel_events(ev[i][0].cuda_event, ev[i][1].cuda_event)
+        fn(i)
+    lib.dmm_set_kernel_events(None, None)
+    torch.cuda.synchronize()
+    t = [a.elapsed_time(b) * 1e-3 for a, b in ev]
+    return sum(t) / len(t)
+
+
+def small_batch(torch, lib, capi, workload, dev, stream, rand_codes):
+    rows = []
+    for K, N in workload.SMALL_BATCH:
+        copies = 24
+        codes = rand_codes(N, K, copies, 7)
+        for M in (4, 8, 16, 32):
+            x, _, grid, scale = workload.make_inputs(M, 8, K, seed=0)
+            x, grid = x.to(dev), grid.to(dev)
+            y = torch.empty(M, N, dtype=torch.float16, device=dev)
+
+            def fn(i):
+                st = lib.dmm_decode_matmul_f16(x.data_ptr(), codes[i % copies].data_ptr(), grid.data_ptr(), scale,
+                                               y.data_ptr(), M, N, K, stream)
+                assert st == 0, st
+            for i in range(5):
+                fn(i)
+            t = timed_kernel(torch, lib, fn, 48)
+            rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3),
+                         "GBps_code": round(workload.code_bytes(N, K) / t / 1e9, 1),
+                         "TFLOPs": round(workload.flops(M, N, K) / t / 1e12, 2)})
+    return rows
+
+
+def prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes):
+    rows = []
+    M = 2048
+    for K, N in workload.PREFILL:
+        codes = rand_codes(N, K, 2, 9)
+        x, _, grid, scale = workload.make_inputs(M, 8, K, seed=0)
+        x, grid = x.to(dev), grid.to(dev)
+        y = torch.empty(M, N, dtype=torch.float16, device=dev)
+
+        def fn(i):
+            st = lib.dmm_decode_matmul_f16(x.data_ptr(), codes[i % 2].data_ptr(), grid.data_ptr(), scale,
+                                           y.data_ptr(), M, N, K, stream)
+            assert st == 0, st
+        for i in range(3):
+            fn(i)
+        t = timed_kernel(torch, lib, fn, 20)
+        # comparison: own decode kernel -> dense half W in HBM -> library GEMM (torch.matmul)
+        for i in range(3):
+            W = dmm.decode(codes[i % 2], grid)
+            ref = torch.matmul(x, W.T)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(20):
+            W = dmm.decode(codes[i % 2], grid)
+            ref = torch.matmul(x, W.T)
+        b.record()
+        torch.cuda.synchronize()
+        t_cmp = a.elapsed_time(b) * 1e-3 / 20
+        tf = workload.flops(M, N, K) / t / 1e12
+        rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 2), "TFLOPs": round(tf, 1),
+                     "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                     "decode_then_library_gemm_us": round(t_cmp * 1e6, 2),
+                     "decode_then_library_gemm_TFLOPs": round(workload.flops(M, N, K) / t_cmp / 1e12, 1)})
+    tot_f = sum(workload.flops(M, N, K) for K, N in workload.PREFILL)
+    tot_t = sum(r["kernel_us"] for r in rows) * 1e-6
+    return {"shapes": rows,
+            "roofline": {"bound": "mfma", "achieved": round(tot_f / tot_t / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(tot_f / tot_t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                         "traffic": None, "kernel": "dmm::gemm_kernel"}}
+
+
+def cpu_baseline(torch, workload):
+    """The torch CPU path (decode to dense half, then matmul) on the host cores, on a bounded
+    sample: one batch-1 GEMV at 8192->8192 (16.8 MB of codes), median of 5."""
+    from oracle import cpu_path
+    K, N = 8192, 8192
+    x, codes, grid, scale = workload.make_inputs(1, N, K, seed=0)
+    cpu_path.time_cpu_path(x, codes, grid, scale, repeats=1)
+    dec, mm, _ = cpu_path.time_cpu_path(x, codes, grid, scale, repeats=5)
+    gbs = workload.code_bytes(N, K) / (dec + mm) / 1e9
+    return {"value": round(gbs, 4), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "one batch-1 GEMV 8192->8192 (16.8 MB of codes), median of 5; decode %.3f s + matmul %.3f s"
+                      % (dec, mm),
+            "host_cpu_count": os.cpu_count()}
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,66 @@
+"""decode_matmul_amd: decode-and-matmul for MI355X (gfx950).
+
+Drop-in for the reference's Python module (`from decode_matmul_cuda import decode_matmul`,
+/root/reference/test_decode_matmul.py:5, /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:237-239)
+in the half-precision form of the same code format:
+
+    from decode_matmul_amd import decode_matmul
+    y = decode_matmul(x, codes, grid, scale)      # x half [M,K], codes int16/uint16 [N,K/8],
+                                                  # grid half [256,8] -> y half [M,N]
+    W = decode(codes, grid)                       # dense half [N,K], bit-exact decode
+
+The functions are the compiled PyTorch operator (`_C`, host C++) over the C ABI of
+`libdmm.so` (hand-written HIP).  There is no CPU implementation: importing this package
+without the built extension raises, and calling the operator with CPU tensors raises.
+"""
+import os as _os
+
+_PKG_DIR = _os.path.dirname(_os.path.abspath(__file__))
+LIB_PATH = _os.path.join(_PKG_DIR, "libdmm.so")
+EXT_PATH = _os.path.join(_PKG_DIR, "_C.so")
+
+import torch as _torch  # noqa: E402  (loads the HIP runtime the extension links against)
+
+if not (_os.path.exists(LIB_PATH) and _os.path.exists(EXT_PATH)):
+    raise ImportError(
+        "decode_matmul_amd: native libraries are not built (%s, %s); run "
+        "`python -m decode_matmul_amd.build`" % (LIB_PATH, EXT_PATH)
+    )
+
+from . import _C  # noqa: E402
+from .capi import lib  # noqa: E402,F401
+from .codebook import (  # noqa: E402,F401
+    build_codebook_abs,
+    grid_from_codebook,
+    transpose_tile,
+    untranspose_tile,
+)
+
+__all__ = [
+    "decode_matmul",
+    "decode_matmul_path",
+    "decode",
+    "lib",
+    "build_codebook_abs",
+    "grid_from_codebook",
+    "transpose_tile",
+    "untranspose_tile",
+]
+
+
+def decode_matmul(x, codes, grid, scale):
+    """y[M,N] = half(scale * x @ decode(codes, grid).T), fp32 accumulation, on x's device and
+    the current stream, asynchronously.  Same role as the reference's `decode_matmul`
+    (decode_matmul_cuda.cu:178-234); raises RuntimeError on bad inputs like its TORCH_CHECKs."""
+    return _C.decode_matmul(x, codes, grid, float(scale))
+
+
+def decode_matmul_path(x, codes, grid, scale, path="auto"):
+    """decode_matmul through one named kernel path: "auto", "gemv", "gemm" or "generic".
+    A path asked for outside its domain raises instead of falling back."""
+    return _C.decode_matmul_path(x, codes, grid, float(scale), path)
+
+
+def decode(codes, grid):
+    """Dense half matrix W[N,K] from codes[N,K/8]; W[n, 8j+d] is dim d of codes[n, j]."""
+    return _C.decode(codes, grid)

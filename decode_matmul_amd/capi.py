@@ -1,0 +1,55 @@
+"""ctypes view of the C ABI declared in include/dmm.h (libdmm.so).
+
+This is the stub a non-PyTorch host would write; the GPU parity tests call the kernels
+through it with raw device pointers so that the boundary itself is what gets tested."""
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libdmm.so")
+
+# every symbol include/dmm.h declares: name -> (restype, argtypes)
+_P, _I64, _F = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float
+_OP = [_P, _P, _P, _F, _P, _I64, _I64, _I64, _P]
+SYMBOLS = {
+    "dmm_version": (ctypes.c_int, []),
+    "dmm_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "dmm_decode_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
+    "dmm_decode_matmul_f16": (ctypes.c_int, _OP),
+    "dmm_gemv_f16": (ctypes.c_int, _OP),
+    "dmm_gemm_f16": (ctypes.c_int, _OP),
+    "dmm_generic_f16": (ctypes.c_int, _OP),
+    "dmm_set_kernel_events": (ctypes.c_int, [_P, _P]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library with argument types set.  Raises OSError if it is not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError("libdmm.so is not built: run `python -m decode_matmul_amd.build`")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def status_string(status):
+    return lib().dmm_status_string(int(status)).decode()
+
+
+class DmmError(RuntimeError):
+    def __init__(self, what, status):
+        super().__init__("%s failed: %s (status %d)" % (what, status_string(status), status))
+        self.status = status
+
+
+def check(what, status):
+    if status != 0:
+        raise DmmError(what, status)

@@ -1,0 +1,131 @@
+// PyTorch-ROCm operator over the C ABI of libdmm.so.  Host code only: no device code is
+// compiled here, the kernels live in dmm.hip behind include/dmm.h.
+//
+// Mirrors the operator boundary of the reference,
+// /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:178-239: one module, a function
+// `decode_matmul`, inputs checked with TORCH_CHECK (-> Python RuntimeError), output
+// allocated by the op on x's device, launch on the current stream under a DeviceGuard.
+// Differences, all deliberate: half precision with a scale (x half, codes 16-bit, grid half
+// [256,8], scale float -> half); no shape demands beyond K % 8 == 0; no device
+// synchronisation and no exit() on error (a non-zero status becomes an exception); the
+// GIL is released around the launch.
+#include <torch/extension.h>
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include "dmm.h"
+
+namespace {
+
+#define DMM_CHECK_DEVICE(t) TORCH_CHECK((t).is_cuda(), #t " must be a GPU tensor")
+#define DMM_CHECK_CONTIGUOUS(t) TORCH_CHECK((t).is_contiguous(), #t " must be contiguous")
+#define DMM_CHECK_INPUT(t)       \
+    do {                         \
+        DMM_CHECK_DEVICE(t);     \
+        DMM_CHECK_CONTIGUOUS(t); \
+    } while (false)
+
+bool is_code_dtype(const torch::Tensor &t)
+{
+    return t.scalar_type() == torch::kInt16 || t.scalar_type() == torch::kUInt16;
+}
+
+void check_status(int st, const char *what)
+{
+    TORCH_CHECK(st == DMM_OK, what, " failed: ", dmm_status_string(st), " (status ", st, ")");
+}
+
+void check_codes_grid(const torch::Tensor &codes, const torch::Tensor &grid)
+{
+    DMM_CHECK_INPUT(codes);
+    DMM_CHECK_INPUT(grid);
+    TORCH_CHECK(is_code_dtype(codes), "codes must be int16 or uint16");
+    TORCH_CHECK(grid.scalar_type() == torch::kHalf, "grid must be float16");
+    TORCH_CHECK(codes.dim() == 2, "codes must be [N, K/8]");
+    TORCH_CHECK(grid.dim() == 2 && grid.size(0) == 256 && grid.size(1) == 8, "grid must be [256, 8]");
+    TORCH_CHECK(codes.device() == grid.device(), "codes and grid must be on the same device");
+}
+
+enum class Path { kAuto, kGemv, kGemm, kGeneric };
+
+torch::Tensor run(const torch::Tensor &x, const torch::Tensor &codes, const torch::Tensor &grid,
+                  double scale, Path path)
+{
+    DMM_CHECK_INPUT(x);
+    check_codes_grid(codes, grid);
+    TORCH_CHECK(x.scalar_type() == torch::kHalf, "x must be float16");
+    TORCH_CHECK(x.dim() == 2, "x must be [M, K]");
+    TORCH_CHECK(x.device() == codes.device(), "x and codes must be on the same device");
+    TORCH_CHECK(x.size(-1) == codes.size(-1) * 8, "x.size(-1) must be 8 * codes.size(-1)");
+
+    const int64_t M = x.size(-2);
+    const int64_t N = codes.size(-2);
+    const int64_t K = x.size(-1);
+
+    c10::hip::HIPGuard guard(x.device());
+    torch::Tensor y = torch::empty({M, N}, x.options().requires_grad(false));
+    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+
+    int st;
+    {
+        pybind11::gil_scoped_release nogil;
+        const void *xp = x.data_ptr(), *cp = codes.data_ptr(), *gp = grid.data_ptr();
+        void *yp = y.data_ptr();
+        const float sc = static_cast<float>(scale);
+        switch (path) {
+            case Path::kGemv: st = dmm_gemv_f16(xp, cp, gp, sc, yp, M, N, K, stream); break;
+            case Path::kGemm: st = dmm_gemm_f16(xp, cp, gp, sc, yp, M, N, K, stream); break;
+            case Path::kGeneric: st = dmm_generic_f16(xp, cp, gp, sc, yp, M, N, K, stream); break;
+            default: st = dmm_decode_matmul_f16(xp, cp, gp, sc, yp, M, N, K, stream); break;
+        }
+    }
+    check_status(st, "decode_matmul");
+    return y;
+}
+
+torch::Tensor decode_matmul(torch::Tensor x, torch::Tensor codes, torch::Tensor grid, double scale)
+{
+    return run(x, codes, grid, scale, Path::kAuto);
+}
+
+torch::Tensor decode_matmul_path(torch::Tensor x, torch::Tensor codes, torch::Tensor grid, double scale,
+                                 const std::string &path)
+{
+    Path p;
+    if (path == "auto") p = Path::kAuto;
+    else if (path == "gemv") p = Path::kGemv;
+    else if (path == "gemm") p = Path::kGemm;
+    else if (path == "generic") p = Path::kGeneric;
+    else TORCH_CHECK(false, "unknown path '", path, "' (auto, gemv, gemm, generic)");
+    return run(x, codes, grid, scale, p);
+}
+
+torch::Tensor decode(torch::Tensor codes, torch::Tensor grid)
+{
+    check_codes_grid(codes, grid);
+    const int64_t N = codes.size(0);
+    const int64_t K = codes.size(1) * 8;
+    c10::hip::HIPGuard guard(codes.device());
+    torch::Tensor W = torch::empty({N, K}, grid.options().requires_grad(false));
+    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    int st;
+    {
+        pybind11::gil_scoped_release nogil;
+        st = dmm_decode_f16(codes.data_ptr(), grid.data_ptr(), W.data_ptr(), N, K, stream);
+    }
+    check_status(st, "decode");
+    return W;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("decode_matmul", &decode_matmul, "Fused decode + matrix multiplication (half precision)",
+          pybind11::arg("x"), pybind11::arg("codes"), pybind11::arg("grid"), pybind11::arg("scale"));
+    m.def("decode_matmul_path", &decode_matmul_path, "decode_matmul through one named kernel path",
+          pybind11::arg("x"), pybind11::arg("codes"), pybind11::arg("grid"), pybind11::arg("scale"),
+          pybind11::arg("path"));
+    m.def("decode", &decode, "Decode codes [N, K/8] to the dense half matrix [N, K]",
+          pybind11::arg("codes"), pybind11::arg("grid"));
+}

@@ -1,0 +1,93 @@
+/* dmm.h - C ABI of the MI355X (gfx950) decode+matmul library, libdmm.so.
+ *
+ * This is the boundary a host binding (the PyTorch extension in
+ * decode_matmul_amd/csrc/torch_binding.cpp, a ctypes stub, cgo, ...) binds to.
+ * Plain pointers and sizes only.  Every pointer is a DEVICE pointer unless a comment
+ * says otherwise.  The library never allocates, frees or retains caller memory, never
+ * synchronises the device and never terminates the process: every entry point enqueues
+ * its kernels on the caller's stream and returns a status code.
+ *
+ * Code format (one 16-bit code per 8 consecutive weights along K), as defined by
+ * /root/reference/test_decode_matmul.py:29-55 and
+ * /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:45-65:
+ *   bits 0-7   grid row                     bits 8-14  sign flips of dims 0-6
+ *   dim 7 sign parity of bits 8-14          bit 15     set: shift -1/4, clear: +1/4
+ *   w[d] = half( (sign_d ? -grid[row][d] : grid[row][d]) + shift )   (flip, then one add)
+ *   W[n, 8*j + d] = decode(codes[n, j])[d]
+ */
+#ifndef DMM_H
+#define DMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  0 = success.  Negative = the call was rejected on the host before any
+ * launch.  Positive = a hipError_t reported by the HIP runtime for the launch. */
+enum {
+    DMM_OK = 0,
+    DMM_ERR_NULL_POINTER = -1,  /* a required pointer is NULL                          */
+    DMM_ERR_BAD_SHAPE = -2,     /* M, N or K negative, K not a multiple of 8, or a
+                                   shape constraint of the entry point is violated      */
+    DMM_ERR_MISALIGNED = -3,    /* a pointer misses the alignment the entry point asks  */
+    DMM_ERR_TOO_LARGE = -4,     /* a dimension exceeds what the launch can index        */
+    DMM_ERR_UNSUPPORTED = -5    /* explicit-path entry point called outside its domain  */
+};
+
+/* Library version, (major << 16) | minor. */
+int dmm_version(void);
+
+/* Human-readable text for a status code returned by this library (static storage). */
+const char *dmm_status_string(int status);
+
+/* Standalone decoder: codes [N, K/8] row-major -> W half [N, K] row-major.
+ * Replaces the decode half of the fused reference kernel
+ * (decode8weights, /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:45-65) in the
+ * half-precision form of the same code; it is the bit-exact gate of the library and the
+ * front half of the decode-then-dense-GEMM comparison.
+ *   codes  uint16/int16 bits, 2-byte aligned         grid  half [256,8], 2-byte aligned
+ *   W      half, 2-byte aligned (16-byte alignment of all three enables the wide path) */
+int dmm_decode_f16(const void *codes, const void *grid, void *W,
+                   int64_t N, int64_t K, void *stream);
+
+/* The operator: y[M,N] = half( scale * sum_k x[m,k] * W[n,k] ), W decoded on the fly,
+ * fp32 accumulation.  Replaces the host wrapper and kernel launch of
+ * /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:178-234 (operator
+ * `decode_matmul`), in the half-precision form: x half [M,K], codes [N,K/8], grid half
+ * [256,8], scalar scale, y half [M,N], all row-major and contiguous.  The only shape
+ * demand is K % 8 == 0 (the reference's M%8, N%16, K%2048 demands,
+ * decode_matmul_cuda.cu:195-207, do not apply).  Chooses the kernel from M, the shape and
+ * the pointer alignments; y is fully overwritten (no caller zeroing). */
+int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, float scale,
+                          void *y, int64_t M, int64_t N, int64_t K, void *stream);
+
+/* Explicit paths of the operator, for tests and measurement.  Same arguments.  Each
+ * returns DMM_ERR_UNSUPPORTED outside its domain instead of falling back:
+ *   dmm_gemv_f16     M <= 32, K % 256 == 0, N % 4 == 0, 16-byte aligned x/codes/grid,
+ *                    8-byte aligned y.  Decoded registers feed the MFMA unit directly;
+ *                    HBM-bound on the code bytes N*K/4.
+ *   dmm_gemm_f16     K % 64 == 0, 16-byte aligned x/codes/grid.  Decoded tiles staged in
+ *                    LDS, fp16 MFMA with fp32 accumulate.
+ *   dmm_generic_f16  any K % 8 == 0, 2-byte alignment: wave-per-row dot products with a
+ *                    DPP wave reduction.  The catch-all. */
+int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale,
+                 void *y, int64_t M, int64_t N, int64_t K, void *stream);
+int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale,
+                 void *y, int64_t M, int64_t N, int64_t K, void *stream);
+int dmm_generic_f16(const void *x, const void *codes, const void *grid, float scale,
+                    void *y, int64_t M, int64_t N, int64_t K, void *stream);
+
+/* Kernel timing hook for benchmarks.  While a (start, stop) pair of hipEvent_t handles is
+ * set on the calling thread, the dominant kernel of each operator call records `start`
+ * immediately before and `stop` immediately after itself on the GPU timeline, so
+ * hipEventElapsedTime(start, stop) is that kernel's own duration, as a profiler's kernel
+ * trace reports it.  Pass NULL, NULL to clear.  No counterpart in the reference, whose
+ * only timer (/root/reference/test_decode_matmul.py:8-22) brackets the whole call. */
+int dmm_set_kernel_events(void *start_event, void *stop_event);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DMM_H */

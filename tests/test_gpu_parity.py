@@ -1,0 +1,229 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI (ctypes, raw device
+pointers) and through the PyTorch operator, against the CPU oracle on identical seeded
+inputs.  Bar: decoded W bit-exact; y within rtol 1e-2 / atol 1e-2 of the fp32-accumulated
+reference; exact where the arithmetic is exact (integer bridge)."""
+import hashlib
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import decode_matmul_amd as dmm
+from decode_matmul_amd import capi, workload
+from conftest import GOLDEN_DIR, quarter_grid
+from gpu_util import DEV, assert_close_to_oracle, bits, c_decode, c_matmul
+from oracle import dmm_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    if isinstance(a, np.ndarray):
+        if a.dtype == np.uint16:
+            a = a.view(np.int16)
+        a = torch.from_numpy(np.ascontiguousarray(a))
+    return a.to(DEV)
+
+
+def finite_random_grid(seed):
+    rng = np.random.default_rng(seed)
+    b = rng.integers(0, 65536, size=(256, 8)).astype(np.uint16)
+    b[(b & 0x7C00) == 0x7C00] &= 0xBFFF          # no inf / nan
+    return b.view(np.float16)
+
+
+# ----------------------------------------------------------------- decode: bit-exact
+@pytest.mark.parametrize("grid_kind", ["quarter0", "quarter1", "e8p", "anyhalf0", "anyhalf1", "denormal"])
+def test_decode_all_65536_codes_bit_exact(grid_kind, all_codes):
+    if grid_kind.startswith("quarter"):
+        grid = quarter_grid(int(grid_kind[-1]))
+    elif grid_kind == "e8p":
+        grid = orc.grid_from_codebook(orc.build_codebook_abs())
+    elif grid_kind == "denormal":
+        grid = (np.arange(2048, dtype=np.uint16) * 3 % 1024).reshape(256, 8).view(np.float16)   # subnormal halves
+    else:
+        grid = finite_random_grid(int(grid_kind[-1]))
+    codes = all_codes.reshape(256, 256)                       # N=256 rows, K=2048
+    W = c_decode(dev(codes), dev(grid))
+    torch.cuda.synchronize()
+    want = orc.decode_f16(codes, grid)
+    assert np.array_equal(bits(W), bits(want))
+
+
+def test_decode_golden_sha256(all_codes):
+    gold = json.load(open(os.path.join(GOLDEN_DIR, "golden.json")))["decode_all_codes"]
+    grid = np.array(gold["grid_bits"], dtype=np.uint16).view(np.float16).reshape(256, 8)
+    W = c_decode(dev(all_codes.reshape(65536, 1)), dev(grid))
+    torch.cuda.synchronize()
+    b = bits(W)
+    assert hashlib.sha256(b.tobytes()).hexdigest() == gold["sha256_of_W_bits"]
+    assert b[:16].tolist() == gold["first16_rows_bits"] and b[-16:].tolist() == gold["last16_rows_bits"]
+
+
+@pytest.mark.parametrize("N,K,offset", [(1, 8, 0), (3, 8, 0), (7, 24, 0), (5, 40, 1), (33, 1000, 3), (4096, 4096, 0)])
+def test_decode_ragged_and_unaligned(N, K, offset):
+    rng = np.random.default_rng(N * 1000 + K)
+    grid = quarter_grid(2)
+    codes = rng.integers(0, 65536, size=(N, K // 8)).astype(np.uint16)
+    # an offset view makes the code pointer 2-byte aligned only -> narrow kernel
+    backing = torch.zeros(N * (K // 8) + 8, dtype=torch.int16, device=DEV)
+    view = backing[offset:offset + N * (K // 8)].view(N, K // 8)
+    view.copy_(dev(codes))
+    W = c_decode(view, dev(grid))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(W), bits(orc.decode_f16(codes, grid)))
+
+
+# ----------------------------------------------------------------- operator vs oracle
+def run_case(path, M, N, K, seed, via="c"):
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=seed)
+    ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+    if via == "c":
+        y = c_matmul(dev(x), dev(codes), dev(grid), scale, path)
+    else:
+        y = dmm.decode_matmul_path(dev(x), dev(codes), dev(grid), scale, path)
+    torch.cuda.synchronize()
+    assert y.dtype == torch.float16 and tuple(y.shape) == (M, N)
+    assert_close_to_oracle(y, ref, "%s M=%d N=%d K=%d" % (path, M, N, K))
+    return y
+
+
+def test_config0_operator():
+    # x [1,4096], codes [4096,512], seed 0: the reference-runnable configuration
+    run_case("auto", 1, 4096, 4096, 0)
+    run_case("auto", 1, 4096, 4096, 0, via="torch")
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 15, 16, 17, 32])
+@pytest.mark.parametrize("N,K", [(4, 256), (64, 512), (100, 768), (1024, 4096), (256, 11008)])
+def test_gemv_path(M, N, K):
+    run_case("gemv", M, N, K, seed=M + N)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 16, 64), (33, 128, 128), (128, 128, 4096), (200, 300, 448),
+                                   (256, 1000, 11008), (5, 7, 64), (130, 129, 192)])
+def test_gemm_path(M, N, K):
+    run_case("gemm", M, N, K, seed=M)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 8), (1, 5, 24), (3, 7, 1000), (9, 33, 4096), (2, 130, 11008)])
+def test_generic_path(M, N, K):
+    run_case("generic", M, N, K, seed=K)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 8192, 8192), (4, 11008, 4096), (32, 4096, 11008), (64, 512, 4096),
+                                   (1, 37, 24), (40, 64, 40)])
+def test_auto_dispatch_and_torch_operator(M, N, K):
+    y_c = run_case("auto", M, N, K, seed=1)
+    y_t = run_case("auto", M, N, K, seed=1, via="torch")
+    assert torch.equal(y_c, y_t)                 # same kernel either way
+
+
+def test_empty_problems():
+    grid = dev(quarter_grid(0))
+    x = torch.zeros(0, 64, dtype=torch.float16, device=DEV)
+    codes = torch.zeros(5, 8, dtype=torch.int16, device=DEV)
+    assert tuple(dmm.decode_matmul(x, codes, grid, 1.0).shape) == (0, 5)
+    x = torch.zeros(3, 64, dtype=torch.float16, device=DEV)
+    codes = torch.zeros(0, 8, dtype=torch.int16, device=DEV)
+    assert tuple(dmm.decode_matmul(x, codes, grid, 1.0).shape) == (3, 0)
+    assert tuple(dmm.decode(codes, grid).shape) == (0, 64)
+    # K = 0: the empty sum is zero
+    x = torch.zeros(3, 0, dtype=torch.float16, device=DEV)
+    codes = torch.zeros(4, 0, dtype=torch.int16, device=DEV)
+    y = dmm.decode_matmul(x, codes, grid, 1.0)
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (3, 4) and torch.all(y == 0)
+
+
+# ----------------------------------------------------------------- exact integer bridge
+@pytest.mark.parametrize("path,M,N,K", [("gemv", 8, 16, 4096), ("gemm", 8, 16, 4096), ("generic", 8, 16, 4096),
+                                         ("gemv", 1, 64, 8192), ("gemm", 64, 64, 8192)])
+def test_integer_bridge_is_exact(path, M, N, K):
+    """x integer-valued, grid = E8P bytes / 4, scale a power of two: every partial sum is a
+    multiple of 1/4 below 2^24 quarters, so fp32 accumulation in any order is exact and the
+    half output must EQUAL half(int32_result / 4 * scale), the reference's integer operator
+    (/root/reference/test_decode_matmul.py:58-71) on the same codes."""
+    rng = np.random.default_rng(K + M)
+    cb = orc.build_codebook_abs()
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    yi = orc.decode_matmul_i32(x, codes, cb)
+    scale = 2.0 ** -8
+    want = (yi.astype(np.float64) / 4 * scale).astype(np.float16)
+    y = c_matmul(dev(x.astype(np.float16)), dev(codes), dev(orc.grid_from_codebook(cb)), scale, path)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), bits(want))
+
+
+def test_reference_shape_golden_case():
+    """The reference's one validated shape, M=8 N=16 K=4096, from the committed fixture."""
+    case = np.load(os.path.join(GOLDEN_DIR, "int8_case.npz"))
+    x, codes, yi, cb = case["x"], case["codes"], case["y"], case["codebook_abs"]
+    grid = dmm.grid_from_codebook(torch.from_numpy(cb))
+    for path in ("auto", "gemv", "gemm", "generic"):
+        y = c_matmul(dev(x.astype(np.float16)), dev(codes), grid.to(DEV), 2.0 ** -8, path)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(y), bits((yi.astype(np.float64) / 4 * 2.0 ** -8).astype(np.float16))), path
+
+
+# ----------------------------------------------------------------- full benchmark sizes
+FULL = [(1, N, K) for (K, N) in workload.LLAMA2_70B + workload.LLAMA2_7B] + \
+       [(16, 11008, 4096), (32, 4096, 11008), (2048, 4096, 4096), (2048, 11008, 4096), (2048, 4096, 11008)]
+
+
+@pytest.mark.parametrize("M,N,K", FULL)
+def test_full_size_against_decode_then_fp32_matmul(M, N, K):
+    """At the benchmark's sizes: W from the decode kernel is bit-exact against the oracle's
+    numpy decode, and the fused operator matches (x.float() @ W.float().T) * scale computed
+    by the library GEMM on the GPU in fp32, within the operator's tolerance."""
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=0)
+    xd, cd, gd = dev(x), dev(codes), dev(grid)
+    W = c_decode(cd, gd)
+    y = c_matmul(xd, cd, gd, scale, "auto")
+    torch.cuda.synchronize()
+    want_W = orc.decode_f16(codes.numpy(), grid.numpy())
+    assert np.array_equal(bits(W), bits(want_W))
+    ref = (xd.float() @ W.float().T) * scale
+    assert_close_to_oracle(y, ref.cpu().numpy(), "full M=%d N=%d K=%d" % (M, N, K))
+    # linearity in x: y(2x) == 2 y(x) up to the last place (a power-of-two scaling changes
+    # no rounding except in the subnormal range)
+    y2 = c_matmul(xd * 2, cd, gd, scale, "auto")
+    torch.cuda.synchronize()
+    assert torch.allclose(y2.float(), 2 * y.float(), rtol=2e-3, atol=1e-3)
+
+
+def test_repeatable_and_stream_ordered():
+    """Same inputs -> same bits, run after run (no atomics, no races), also on a side stream
+    while the default stream is busy."""
+    x, codes, grid, scale = workload.make_inputs(4, 8192, 8192, seed=5)
+    xd, cd, gd = dev(x), dev(codes), dev(grid)
+    first = c_matmul(xd, cd, gd, scale, "auto")
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    for _ in range(5):
+        with torch.cuda.stream(side):
+            again = dmm.decode_matmul(xd, cd, gd, scale)
+        side.synchronize()
+        assert torch.equal(first, again)
+
+
+def test_kernel_event_hook_times_the_kernel():
+    x, codes, grid, scale = workload.make_inputs(1, 8192, 8192, seed=2)
+    xd, cd, gd = dev(x), dev(codes), dev(grid)
+    y0 = c_matmul(xd, cd, gd, scale)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(); stop.record()                # materialise the handles
+    torch.cuda.synchronize()
+    lib = capi.lib()
+    assert lib.dmm_set_kernel_events(start.cuda_event, stop.cuda_event) == 0
+    try:
+        y1 = c_matmul(xd, cd, gd, scale)
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(stop)
+    finally:
+        assert lib.dmm_set_kernel_events(None, None) == 0
+    assert torch.equal(y0, y1)
+    assert 0.0 < ms < 5.0

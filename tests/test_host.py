@@ -1,0 +1,127 @@
+"""Host-side checks that need no GPU: the C ABI library loads and exports every symbol the
+header declares, rejects bad arguments before launching anything, the PyTorch operator
+raises RuntimeError like the reference's TORCH_CHECKs, and the host helpers (codebook,
+tiling, workload generators) agree with the oracle."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import decode_matmul_amd as dmm
+from decode_matmul_amd import capi, workload
+from conftest import ROOT
+from oracle import dmm_oracle as orc
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "dmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dmm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = header_symbols()
+    assert "dmm_decode_matmul_f16" in names and "dmm_decode_f16" in names
+    handle = ctypes.CDLL(capi.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), n
+    assert sorted(capi.SYMBOLS) == names          # the ctypes stub covers the whole header
+    assert capi.lib().dmm_version() >= 1
+
+
+def test_status_strings():
+    lib = capi.lib()
+    for st in (0, -1, -2, -3, -4, -5):
+        assert len(lib.dmm_status_string(st)) > 0
+    assert b"shape" in lib.dmm_status_string(-2)
+
+
+def test_argument_errors_are_status_codes_not_crashes():
+    lib = capi.lib()
+    buf = (ctypes.c_uint16 * 4096)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    odd = ctypes.c_void_p(p.value + 1)
+    # K not a multiple of 8, negative sizes
+    assert lib.dmm_decode_f16(p, p, p, 4, 12, None) == -2
+    assert lib.dmm_decode_f16(p, p, p, -1, 8, None) == -2
+    assert lib.dmm_decode_matmul_f16(p, p, p, 1.0, p, 1, 4, 20, None) == -2
+    assert lib.dmm_decode_matmul_f16(p, p, p, 1.0, p, -1, 4, 16, None) == -2
+    # NULL pointers
+    assert lib.dmm_decode_f16(None, p, p, 4, 16, None) == -1
+    assert lib.dmm_decode_matmul_f16(p, p, None, 1.0, p, 1, 4, 16, None) == -1
+    assert lib.dmm_decode_matmul_f16(p, p, p, 1.0, None, 1, 4, 16, None) == -1
+    # odd addresses
+    assert lib.dmm_decode_f16(odd, p, p, 4, 16, None) == -3
+    assert lib.dmm_decode_matmul_f16(odd, p, p, 1.0, p, 1, 4, 16, None) == -3
+    # explicit paths refuse shapes outside their domain instead of falling back
+    assert lib.dmm_gemv_f16(p, p, p, 1.0, p, 1, 4, 16, None) == -5       # K % 256 != 0
+    assert lib.dmm_gemv_f16(p, p, p, 1.0, p, 64, 4, 256, None) == -5     # M too large
+    assert lib.dmm_gemm_f16(p, p, p, 1.0, p, 64, 4, 16, None) == -5      # K % 64 != 0
+    # empty problems succeed without touching the device
+    assert lib.dmm_decode_f16(None, None, None, 0, 64, None) == 0
+    assert lib.dmm_decode_matmul_f16(None, None, None, 1.0, None, 0, 4, 16, None) == 0
+    assert lib.dmm_decode_matmul_f16(None, None, None, 1.0, None, 3, 0, 16, None) == 0
+    # the timing hook wants both events or neither
+    assert lib.dmm_set_kernel_events(p, None) == -1
+    assert lib.dmm_set_kernel_events(None, None) == 0
+
+
+def test_operator_rejects_bad_inputs_with_runtime_error():
+    x = torch.zeros(1, 64, dtype=torch.float16)
+    codes = torch.zeros(4, 8, dtype=torch.int16)
+    grid = torch.zeros(256, 8, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        dmm.decode_matmul(x, codes, grid, 1.0)          # CPU tensors: there is no CPU path
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        dmm.decode(codes, grid)
+    with pytest.raises(RuntimeError):
+        dmm.decode_matmul_path(x, codes, grid, 1.0, "nonsense")
+
+
+def test_codebook_matches_oracle_and_reference_properties():
+    cb = dmm.build_codebook_abs()
+    assert cb.dtype == torch.int64 and cb.shape == (256,)
+    assert np.array_equal(cb.numpy(), orc.build_codebook_abs())
+    grid = dmm.grid_from_codebook(cb)
+    assert grid.dtype == torch.float16 and grid.shape == (256, 8)
+    assert np.array_equal(grid.numpy().view(np.uint16), orc.grid_from_codebook(cb.numpy()).view(np.uint16))
+    # first entry: all coordinates 1/2 -> every byte 2 (test_decode_matmul.py:85)
+    assert int(cb[0]) == 0x0202020202020202
+
+
+def test_transpose_tile_matches_oracle():
+    g = torch.Generator().manual_seed(1)
+    codes = torch.randint(-32768, 32768, (48, 24), generator=g, dtype=torch.int16)
+    t = dmm.transpose_tile(codes)
+    assert np.array_equal(t.numpy(), orc.transpose_tile(codes.numpy()))
+    assert torch.equal(dmm.untranspose_tile(t), codes)
+
+
+def test_workload_generators():
+    x, codes, grid, scale = workload.make_inputs(1, 4096, 4096, seed=0)
+    assert x.shape == (1, 4096) and x.dtype == torch.float16
+    assert codes.shape == (4096, 512) and codes.dtype == torch.int16
+    assert grid.shape == (256, 8) and set(grid.unique().tolist()) == set(workload.GRID_VALUES)
+    assert scale == pytest.approx(1 / 64)
+    x2, codes2, grid2, _ = workload.make_inputs(1, 4096, 4096, seed=0)
+    assert torch.equal(x, x2) and torch.equal(codes, codes2) and torch.equal(grid, grid2)
+    # codes use the full 16-bit range, both signs of the int16 view
+    assert int(codes.min()) < -30000 and int(codes.max()) > 30000
+    assert workload.code_bytes(28672, 8192) == 58720256
+    assert workload.flops(2048, 4096, 4096) == 68719476736
+
+
+def test_config0_cpu_plumbing():
+    """The CPU-runnable configuration: x [1,4096], codes [4096,512], seed 0.  No GPU here, so
+    this runs the oracle's two independent restatements against each other on it and checks
+    the decoded alphabet; the GPU run of the same configuration is in test_gpu_parity.py."""
+    x, codes, grid, scale = workload.make_inputs(1, 4096, 4096, seed=0)
+    W = orc.decode_f16(codes.numpy(), grid.numpy())
+    assert W.shape == (4096, 4096)
+    assert set(np.unique(W).tolist()) <= {v / 2 for v in range(-6, 7)}
+    y = orc.decode_matmul_f16(x.numpy(), codes.numpy(), grid.numpy(), scale)
+    ref = (x.float() @ torch.from_numpy(W).float().T) * scale
+    assert torch.allclose(torch.from_numpy(y).float(), ref, rtol=1e-2, atol=1e-2)
