@@ -442,16 +442,20 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t *__restrict__ 
 #pragma unroll
             for (int e4 = 0; e4 < 4; e4++) {
                 const int n = n0 + wn * 64 + i * 32 + 8 * e4 + 4 * kq;
-                h4_t o;
+                uint16_t o[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (half_t)(acc[i][j][4 * e4 + e] * scale);
+                for (int e = 0; e < 4; e++)
+                    o[e] = __builtin_bit_cast(uint16_t, (half_t)(acc[i][j][4 * e4 + e] * scale));
                 uint16_t *dst = y + (int64_t)m * N + n;
                 if (n_vec && n + 3 < N) {
-                    *reinterpret_cast<h4_t *>(dst) = o;
+                    u2_t v;
+                    v[0] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+                    v[1] = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+                    *reinterpret_cast<u2_t *>(dst) = v;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        if (n + e < N) dst[e] = __builtin_bit_cast(uint16_t, o[e]);
+                        if (n + e < N) dst[e] = o[e];
                 }
             }
         }

@@ -10,7 +10,7 @@
 // synchronisation and no exit() on error (a non-zero status becomes an exception); the
 // GIL is released around the launch.
 #include <torch/extension.h>
-#include <c10/hip/HIPGuard.h>
+#include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
 #include "dmm.h"
@@ -62,9 +62,9 @@ torch::Tensor run(const torch::Tensor &x, const torch::Tensor &codes, const torc
     const int64_t N = codes.size(-2);
     const int64_t K = x.size(-1);
 
-    c10::hip::HIPGuard guard(x.device());
+    c10::DeviceGuard guard(x.device());
     torch::Tensor y = torch::empty({M, N}, x.options().requires_grad(false));
-    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t stream = c10::hip::getCurrentHIPStream(x.device().index()).stream();
 
     int st;
     {
@@ -105,9 +105,9 @@ torch::Tensor decode(torch::Tensor codes, torch::Tensor grid)
     check_codes_grid(codes, grid);
     const int64_t N = codes.size(0);
     const int64_t K = codes.size(1) * 8;
-    c10::hip::HIPGuard guard(codes.device());
+    c10::DeviceGuard guard(codes.device());
     torch::Tensor W = torch::empty({N, K}, grid.options().requires_grad(false));
-    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t stream = c10::hip::getCurrentHIPStream(codes.device().index()).stream();
     int st;
     {
         pybind11::gil_scoped_release nogil;
