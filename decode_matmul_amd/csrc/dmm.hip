@@ -14,6 +14,8 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
 
 #include "dmm.h"
 
@@ -38,14 +40,11 @@ struct DecodeTables {
 
 __device__ __forceinline__ u4_t sign_row(uint32_t s7)
 {
-    uint32_t s8 = s7 | ((__builtin_popcount(s7) & 1u) << 7);
+    const uint32_t s8 = s7 | ((__builtin_popcount(s7) & 1u) << 7);
     u4_t r;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        uint32_t lo = ((s8 >> (2 * i)) & 1u) ? 0xBC00u : 0x3C00u;
-        uint32_t hi = ((s8 >> (2 * i + 1)) & 1u) ? 0xBC00u : 0x3C00u;
-        r[i] = lo | (hi << 16);
-    }
+    for (int i = 0; i < 4; i++)   // +-1.0 = 0x3C00 with the sign bit of dim 2i (low half) / 2i+1 (high half)
+        r[i] = 0x3C003C00u | (((s8 >> (2 * i)) & 1u) << 15) | (((s8 >> (2 * i + 1)) & 1u) << 31);
     return r;
 }
 
@@ -210,15 +209,121 @@ __global__ __launch_bounds__(256) void generic_kernel(const uint16_t *__restrict
 // row m = c of x, same 8 k.  Any k order works as long as A and B agree, so the 32 k of
 // MFMA number t in a step are {64*q + 8*t .. +8 : q = 0..3} rather than 32 consecutive k;
 // that is what lets the code load be one 16-byte load per lane.  For M = 1 only column 0
-// carries data, the other 15 columns cost nothing extra: the matrix unit has the
-// headroom and the kernel is bound by the code bytes coming from HBM.
+// carries data, the other 15 columns cost nothing extra: the matrix unit has the headroom.
 // Accumulator layout: lane holds rows 4*q + i (i = 0..3) of column c, i.e.
 // y[m = c][n = n0 + 4*q + i] - four consecutive halves of a row of y.
-template <int R, int W, int MT>
-struct GemvShared {
-    DecodeTables tab;
-    f4_t red[W][R * MT][kWave];
+//
+// What bounds the kernel is the LDS, not HBM: every code costs two 16-byte LDS gathers
+// (grid row, sign row) and the LDS delivers 128 bytes per clock per CU only when the 8
+// lanes it serves in one clock hit 8 different 16-byte bank groups.  Random rows collide,
+// so the tables are stored 8 times over: one unified table of 256 rows x 256 bytes, row i =
+// [grid row i, 8 copies | sign row (i & 127), 8 copies], and a lane reads copy lane%8.
+// Gathers are then conflict-free whatever the codes are, and - because the row pitch is
+// 256 - a table address is just a byte of the code word placed above the lane's copy
+// offset, one v_perm_b32: the low byte of a code addresses its grid row, the high byte
+// (7 sign bits + the shift bit, hence the 256 sign rows) its sign row at +128.
+constexpr int kGemvTableBytes = 256 * 256;
+
+// Thread tid fills table slots tid, tid + nthreads, ...: slot j is copy (j % 16) of row j / 16.
+// The grid rows it needs are fetched by gemv_fetch_grid beforehand, so that the global loads
+// are the first ones the kernel issues and nothing queues behind the code stream.
+template <int kNThreads>
+__device__ __forceinline__ void gemv_fetch_grid(u4_t (&g)[4096 / kNThreads], const void *grid, int tid)
+{
+#pragma unroll
+    for (int i = 0; i < 4096 / kNThreads; i++) g[i] = reinterpret_cast<const u4_t *>(grid)[(tid + i * kNThreads) >> 4];
+}
+
+template <int kNThreads>
+__device__ __forceinline__ void stage_gemv_tables(unsigned char *tab, const u4_t (&g)[4096 / kNThreads], int tid)
+{
+    u4_t *t = reinterpret_cast<u4_t *>(tab);
+#pragma unroll
+    for (int i = 0; i < 4096 / kNThreads; i++) {
+        const int j = tid + i * kNThreads;
+        t[j] = (j & 8) ? sign_row((uint32_t)((j >> 4) & 0x7F)) : g[i];
+    }
+}
+
+typedef __attribute__((address_space(3))) const u4_t lds_u4_t;
+
+// 32-bit LDS byte address of a pointer into shared memory
+__device__ __forceinline__ uint32_t lds_addr(const void *p)
+{
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+
+__device__ __forceinline__ u4_t lds_read16(uint32_t byte_addr)
+{
+    return *reinterpret_cast<lds_u4_t *>(byte_addr);
+}
+
+// w = g * s + d with d taken from the low (kHi = false) or high half of dd for both lanes
+template <bool kHi>
+__device__ __forceinline__ uint32_t pk_fma_bcast(uint32_t g, uint32_t s, uint32_t dd)
+{
+    uint32_t r;
+    if (kHi)
+        asm("v_pk_fma_f16 %0, %1, %2, %3 op_sel:[0,0,1] op_sel_hi:[1,1,1]" : "=v"(r) : "v"(g), "v"(s), "v"(dd));
+    else
+        asm("v_pk_fma_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,1,0]" : "=v"(r) : "v"(g), "v"(s), "v"(dd));
+    return r;
+}
+
+// One 32-bit word = two codes.  Its decode is split in two so that the LDS gathers of the
+// next word can be in flight while the packed FMAs and MFMAs of this one issue.
+struct GemvGather {
+    u4_t g0, s0, g1, s1;   // grid row / sign row of code 0, of code 1
+    uint32_t dd;           // (+-0.25 for code 0, +-0.25 for code 1) as packed halves
 };
+
+// lane_base: LDS byte address of this lane's table copy, table base + (lane % 8) * 16 (< 256)
+__device__ __forceinline__ void gemv_gather(GemvGather &o, uint32_t w, uint32_t lane_base)
+{
+    o.g0 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));          // byte 0 of w << 8 | lane_base
+    o.s0 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0500u) + 128u);
+    o.g1 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
+    o.s1 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0700u) + 128u);
+    o.dd = (w & 0x80008000u) | 0x34003400u;
+}
+
+__device__ __forceinline__ void gemv_finish(const GemvGather &o, h8_t &a0, h8_t &a1)
+{
+    u4_t r0, r1;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        r0[i] = pk_fma_bcast<false>(o.g0[i], o.s0[i], o.dd);
+        r1[i] = pk_fma_bcast<true>(o.g1[i], o.s1[i], o.dd);
+    }
+    a0 = __builtin_bit_cast(h8_t, r0);
+    a1 = __builtin_bit_cast(h8_t, r1);
+}
+
+// One 256-wide k step for R row tiles: 4R words, gathers one word ahead of the math.
+// acc[r][mt][0/1]: the even and odd codes of a word accumulate separately, so that
+// consecutive MFMAs never depend on each other.
+template <int R, int MT>
+__device__ __forceinline__ void gemv_step(const u4_t (&cw)[R], const u4_t (&xb)[MT][8], uint32_t lane_base,
+                                          f4_t (&acc)[R][MT][2])
+{
+    constexpr int kItems = 4 * R;       // item i: word t2 = i / R of row tile r = i % R
+    GemvGather buf[2];
+    gemv_gather(buf[0], cw[0][0], lane_base);
+#pragma unroll
+    for (int i = 0; i < kItems; i++) {
+        const int t2 = i / R, r = i % R;
+        if (i + 1 < kItems) gemv_gather(buf[(i + 1) & 1], cw[(i + 1) % R][(i + 1) / R], lane_base);
+        h8_t a0, a1;
+        gemv_finish(buf[i & 1], a0, a1);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            acc[r][mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                a0, __builtin_bit_cast(h8_t, xb[mt][2 * t2]), acc[r][mt][0], 0, 0, 0);
+            acc[r][mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                a1, __builtin_bit_cast(h8_t, xb[mt][2 * t2 + 1]), acc[r][mt][1], 0, 0, 0);
+        }
+    }
+}
 
 template <int R, int W, int MT>
 __global__ __launch_bounds__(64 * W) void gemv_kernel(const uint16_t *__restrict__ x,
@@ -226,8 +331,11 @@ __global__ __launch_bounds__(64 * W) void gemv_kernel(const uint16_t *__restrict
                                                       const void *__restrict__ grid, float scale,
                                                       uint16_t *__restrict__ y, int M, int N, int K)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    GemvShared<R, W, MT> &sh = *reinterpret_cast<GemvShared<R, W, MT> *>(smem_raw);
+    // the decode table, and - once every wave is done with it - the split-K partial sums
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+    typedef f4_t red_t[R * MT][kWave];
+    static_assert(sizeof(red_t) * W <= kGemvTableBytes, "partials must fit in the table's space");
+    red_t *red = reinterpret_cast<red_t *>(smem_raw);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -237,6 +345,7 @@ __global__ __launch_bounds__(64 * W) void gemv_kernel(const uint16_t *__restrict
     const int n_steps = K >> 8;  // 256 k per step
     const int64_t row_bytes = (int64_t)K >> 2;  // K/8 codes * 2 bytes
     const int row0 = blockIdx.x * (16 * R);
+    const uint32_t lane_base = lds_addr(smem_raw) + (uint32_t)(lane & 7) * 16u;
 
     // per-tile code pointers; rows past N are clamped (their results are never stored)
     const unsigned char *cptr[R];
@@ -246,85 +355,75 @@ __global__ __launch_bounds__(64 * W) void gemv_kernel(const uint16_t *__restrict
         row = row < N ? row : N - 1;
         cptr[r] = reinterpret_cast<const unsigned char *>(codes) + row * row_bytes + q * 16;
     }
-    // x pointers: lane's column c16 is row m of x (per m-tile), its quarter starts at 64*q.
-    // Columns past M read row 0: whatever they compute is never stored, and identical
-    // addresses within a quarter cost no extra bytes.
-    const unsigned char *xptr[MT];
+    // x goes through a buffer descriptor: lane's column c16 is row m of x (per m-tile), its
+    // quarter starts at 64*q.  Columns past M get an offset beyond the buffer, which the
+    // hardware answers with zeros without touching memory - for M = 1 only 4 lanes of the
+    // wave fetch anything - and there is no branch for the wait counters to lose track at.
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, M * K * 2, 0x00020000);
+    int xoff[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
-        int m = 16 * mt + c16;
-        m = m < M ? m : 0;
-        xptr[mt] = reinterpret_cast<const unsigned char *>(x) + ((int64_t)m * K + 64 * q) * 2;
+        const int m = 16 * mt + c16;
+        xoff[mt] = m < M ? (m * K + 64 * q) * 2 : 0x7F000000;
     }
 
-    // first step's code loads go out before the tables are built
-    u4_t cw[R];
-    int step = wave;
-    if (step < n_steps) {
+    auto load_codes = [&](u4_t (&cw)[R], int step) {
 #pragma unroll
-        for (int r = 0; r < R; r++) cw[r] = *reinterpret_cast<const u4_t *>(cptr[r] + (int64_t)step * 64);
-    }
-
-    stage_tables<true>(sh.tab, grid, tid, 64 * W);
-    __syncthreads();
-
-    f4_t acc[R][MT];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) acc[r][mt] = f4_t{0.f, 0.f, 0.f, 0.f};
-
-    for (; step < n_steps; step += W) {
-        // x for this step: 8 x 16 bytes per lane and m-tile (64 halves of the lane's quarter)
-        u4_t xb[MT][8];
+        for (int r = 0; r < R; r++)
+            cw[r] = __builtin_nontemporal_load(reinterpret_cast<const u4_t *>(cptr[r] + (int64_t)step * 64));
+    };
+    auto load_x = [&](u4_t (&xb)[MT][8], int step) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int t = 0; t < 8; t++)
-                xb[mt][t] = *reinterpret_cast<const u4_t *>(xptr[mt] + (int64_t)step * 512 + t * 16);
-        // next step's codes
-        u4_t cn[R];
-        const int next = step + W;
-        if (next < n_steps) {
-#pragma unroll
-            for (int r = 0; r < R; r++) cn[r] = *reinterpret_cast<const u4_t *>(cptr[r] + (int64_t)next * 64);
-        }
-#pragma unroll
-        for (int t2 = 0; t2 < 4; t2++) {
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                u4_t w0, w1;
-                decode8x2(cw[r][t2], sh.tab, w0, w1);
-                h8_t a0 = __builtin_bit_cast(h8_t, w0);
-                h8_t a1 = __builtin_bit_cast(h8_t, w1);
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        a0, __builtin_bit_cast(h8_t, xb[mt][2 * t2]), acc[r][mt], 0, 0, 0);
-                    acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        a1, __builtin_bit_cast(h8_t, xb[mt][2 * t2 + 1]), acc[r][mt], 0, 0, 0);
-                }
-            }
-        }
-        if (next < n_steps) {
-#pragma unroll
-            for (int r = 0; r < R; r++) cw[r] = cn[r];
-        }
-    }
+                xb[mt][t] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff[mt] + step * 512 + t * 16, 0, 0);
+    };
 
-    // cross-wave (split-K) reduction through LDS, then scale, round to half and store
+    // grid rows first, then the first two steps' loads; the table is built while those fly
+    u4_t gtmp[4096 / (64 * W)];
+    gemv_fetch_grid<64 * W>(gtmp, grid, tid);
+    u4_t cw0[R], cw1[R];
+    u4_t xb0[MT][8], xb1[MT][8];
+    int step = wave;
+    if (step < n_steps) { load_codes(cw0, step); load_x(xb0, step); }
+    if (step + W < n_steps) { load_codes(cw1, step + W); load_x(xb1, step + W); }
+
+    stage_gemv_tables<64 * W>(smem_raw, gtmp, tid);
+    __syncthreads();
+
+    f4_t acc[R][MT][2];
 #pragma unroll
     for (int r = 0; r < R; r++)
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) sh.red[wave][r * MT + mt][lane] = acc[r][mt];
+        for (int mt = 0; mt < MT; mt++) acc[r][mt][0] = acc[r][mt][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+
+    // two steps per trip, ping-pong between the register buffers: each buffer is refilled
+    // (for two steps ahead) right after it has been consumed
+    while (step < n_steps) {
+        gemv_step<R, MT>(cw0, xb0, lane_base, acc);
+        if (step + 2 * W < n_steps) { load_codes(cw0, step + 2 * W); load_x(xb0, step + 2 * W); }
+        if (step + W >= n_steps) break;
+        gemv_step<R, MT>(cw1, xb1, lane_base, acc);
+        if (step + 3 * W < n_steps) { load_codes(cw1, step + 3 * W); load_x(xb1, step + 3 * W); }
+        step += 2 * W;
+    }
+
+    // cross-wave (split-K) reduction through LDS, then scale, round to half and store
+    __syncthreads();   // every wave has finished reading the table
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) red[wave][r * MT + mt][lane] = acc[r][mt][0] + acc[r][mt][1];
     __syncthreads();
     for (int idx = tid; idx < R * MT * kWave; idx += 64 * W) {
         const int l = idx & 63;
         const int tile = idx >> 6;
         const int r = tile / MT, mt = tile % MT;
-        f4_t s = sh.red[0][tile][l];
+        f4_t s = red[0][tile][l];
 #pragma unroll
-        for (int w = 1; w < W; w++) s += sh.red[w][tile][l];
+        for (int w = 1; w < W; w++) s += red[w][tile][l];
         const int m = 16 * mt + (l & 15);
         const int n = row0 + 16 * r + 4 * (l >> 4);
         if (m < M && n < N) {   // N % 4 == 0, so the four rows are in range together
@@ -334,6 +433,299 @@ __global__ __launch_bounds__(64 * W) void gemv_kernel(const uint16_t *__restrict
             *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
         }
     }
+}
+
+// ------------------------------------------------------------------ streaming matrix-vector path
+// The batch-1 path proper (small M, x small enough to live in LDS).  What the kernel above
+// cannot do is keep enough code bytes in flight: HBM answers in a few microseconds under
+// load, so a CU needs on the order of 100 KB outstanding, and because vector-memory results
+// return in order, any x load queued behind the code prefetch stalls until the whole
+// prefetch has landed.  Here:
+//   * x is copied once per workgroup into LDS (row pitch 2K + 16 bytes, so the rows read
+//     together fall in different bank groups) and B operands are read from there;
+//   * the code stream is a ring of D register buffers per wave, refilled with raw buffer
+//     loads: the per-lane part of the address never changes, everything that moves (row
+//     block, k step) is in the scalar offset, and past the end that offset is out of range,
+//     which the hardware answers with zeros - no branch around any vector-memory
+//     instruction, so the wait counters stay exact and D * R loads per wave stay in flight;
+//   * workgroups are persistent (one per CU) and walk over row blocks, so the tables and x
+//     are staged once and the prefetch runs across row-block boundaries;
+//   * the LDS serves 16 lanes of a 16-byte gather per clock, so the decode tables hold 16
+//     copies of every row (row pitch 256 bytes, lane reads copy lane % 16): conflict-free for
+//     any codes.  A table address is one v_perm_b32: a byte of the code word placed above
+//     the lane's copy offset.
+// LDS map: [0, 32K) sign rows (128 x 256 B), [32K, 96K) grid rows (256 x 256 B),
+//          then 2 x (W x R x 4 x M) float4 partial sums (double-buffered per row block), then x.
+#ifdef DMM_TRACE
+// Experiment build only: per-wave timestamps kept in the last 4 KB of LDS and copied out
+// when the wave ends, so that marking does not disturb the vector-memory queue.
+__device__ unsigned long long *dmm_trace_buf = nullptr;
+__device__ int dmm_exp_mode = 0;   // 1: loads only (no decode), 2: decode only (no HBM traffic)
+#define DMM_TRACE_SLOTS 32
+#define DMM_TRACE_LDS(smem) (reinterpret_cast<unsigned long long *>((smem) + 160 * 1024 - 16 * DMM_TRACE_SLOTS * 8))
+#define DMM_TRACE_MARK(slot)                                                                         \
+    do {                                                                                             \
+        if ((threadIdx.x & 63) == 0)                                                                 \
+            DMM_TRACE_LDS(smem_raw)[(threadIdx.x >> 6) * DMM_TRACE_SLOTS + (slot)] = __builtin_amdgcn_s_memrealtime(); \
+    } while (0)
+#define DMM_TRACE_DUMP()                                                                             \
+    do {                                                                                             \
+        if (dmm_trace_buf && (threadIdx.x & 63) < DMM_TRACE_SLOTS)                                   \
+            dmm_trace_buf[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * DMM_TRACE_SLOTS + (threadIdx.x & 63)] = \
+                DMM_TRACE_LDS(smem_raw)[(threadIdx.x >> 6) * DMM_TRACE_SLOTS + (threadIdx.x & 63)];  \
+    } while (0)
+#else
+#define DMM_TRACE_MARK(slot) do { } while (0)
+#define DMM_TRACE_DUMP() do { } while (0)
+#endif
+
+constexpr int kSSignBytes = 128 * 256;
+constexpr int kSGridBytes = 256 * 256;
+constexpr int kSTablesBytes = kSSignBytes + kSGridBytes;
+
+__host__ __device__ constexpr int stream_red_bytes(int R, int W, int M) { return 2 * W * R * 4 * M * 16; }
+
+// Table staging: thread tid fetches ONE grid row (row tid % 256) and writes 4096 / kNThreads
+// of its 16 copies; the 2048 sign slots are computed, 2048 / kNThreads per thread.
+template <int kNThreads>
+__device__ __forceinline__ void stream_stage_tables(unsigned char *smem, const u4_t &grow, int tid)
+{
+    static_assert(kNThreads == 512 || kNThreads == 1024, "staging assumes 512 or 1024 threads");
+    constexpr int kCopiesPer = 4096 / kNThreads;          // copies of its row a thread writes
+    u4_t *sg = reinterpret_cast<u4_t *>(smem);
+    u4_t *gg = reinterpret_cast<u4_t *>(smem + kSSignBytes);
+    const int row = tid & 255, c0 = (tid >> 8) * kCopiesPer;
+#pragma unroll
+    for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + c0 + i] = grow;
+#pragma unroll
+    for (int i = 0; i < 2048 / kNThreads; i++) sg[tid + i * kNThreads] = sign_row((uint32_t)((tid + i * kNThreads) >> 4));
+}
+
+// (a & m) | (b & ~m) in one instruction
+__device__ __forceinline__ uint32_t bfi(uint32_t m, uint32_t a, uint32_t b)
+{
+    uint32_t r;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(r) : "s"(m), "v"(a), "v"(b));
+    return r;
+}
+
+struct StreamGather {
+    u4_t g0, s0, g1, s1;
+    uint32_t dd;
+};
+
+// lane_base = (lane % 16) * 16; the tables start at LDS address 0
+__device__ __forceinline__ void stream_gather(StreamGather &o, uint32_t w, uint32_t lane_base, uint32_t quarter_bits)
+{
+    const uint32_t w7 = w & 0x7FFF7FFFu;                 // sign-row index must not see the shift bit
+    o.g0 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u) + kSSignBytes);
+    o.s0 = lds_read16(__builtin_amdgcn_perm(w7, lane_base, 0x0C0C0500u));
+    o.g1 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u) + kSSignBytes);
+    o.s1 = lds_read16(__builtin_amdgcn_perm(w7, lane_base, 0x0C0C0700u));
+    o.dd = bfi(0x7FFF7FFFu, quarter_bits, w);            // (+-0.25, +-0.25): signs from the shift bits
+}
+
+template <bool kHi>
+__device__ __forceinline__ h8_t stream_finish(const u4_t &g, const u4_t &sg, uint32_t dd)
+{
+    u4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = pk_fma_bcast<kHi>(g[i], sg[i], dd);
+    return __builtin_bit_cast(h8_t, r);
+}
+
+// One 256-wide k step for R row tiles.  Items (word t2 of row tile r) run t2-major so that the
+// two B operands of a word pair are read from LDS once and used for all R tiles; the gathers
+// of item i+1 are issued before the math of item i.
+template <int R>
+__device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t lane_base,
+                                            uint32_t quarter_bits, f4_t (&acc)[R][2])
+{
+    constexpr int kItems = 4 * R;
+    StreamGather buf[2];
+    u4_t xb[2][2];
+    xb[0][0] = lds_read16(xaddr);
+    xb[0][1] = lds_read16(xaddr + 16);
+    stream_gather(buf[0], cw[0][0], lane_base, quarter_bits);
+#pragma unroll
+    for (int i = 0; i < kItems; i++) {
+        const int t2 = i / R, r = i % R;
+        if (i + 1 < kItems) {
+            const int nt2 = (i + 1) / R, nr = (i + 1) % R;
+            if (nr == 0) {
+                xb[nt2 & 1][0] = lds_read16(xaddr + nt2 * 32);
+                xb[nt2 & 1][1] = lds_read16(xaddr + nt2 * 32 + 16);
+            }
+            stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
+        }
+        // 4 packed FMAs, MFMA, 4 packed FMAs, MFMA: the second group and the next item's
+        // address math run in the shadow of the matrix unit
+        const StreamGather &b = buf[i & 1];
+        const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
+        acc[r][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[t2 & 1][0]), acc[r][0], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
+        acc[r][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[t2 & 1][1]), acc[r][1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+template <int R, int W, int D>
+__global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__restrict__ x,
+                                                             const uint16_t *__restrict__ codes,
+                                                             const void *__restrict__ grid, float scale,
+                                                             uint16_t *__restrict__ y, int M, int N, int K,
+                                                             int n_blocks)
+{
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
+    DMM_TRACE_MARK(0);
+    f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // [2][W][R][4 * M]
+    const int red_par = W * R * 4 * M;                                 // float4 per parity
+    unsigned char *xs = smem_raw + kSTablesBytes + stream_red_bytes(R, W, M);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int c16 = lane & 15;
+    const int q = lane >> 4;
+    const int n_steps = K >> 8;
+    const int row_bytes = K >> 2;
+    const int x_pitch = 2 * K + 16;
+    const uint32_t lane_base = (uint32_t)c16 * 16u;
+    const uint32_t quarter_bits = 0x34003400u;
+
+    // ---- prologue: this thread's grid row and its share of x first (short latency, nothing
+    // queued in front of them), then the first D items of the code stream; the tables and the
+    // LDS copy of x are built while the code loads fly ---------------------------------------
+    const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid & 255];
+    const int row_chunks = K >> 3;                     // 16-byte pieces per row of x
+    constexpr int kXPer = 4;                           // pieces of row 0 per thread fetched up front
+    u4_t xv[kXPer];
+#pragma unroll
+    for (int u = 0; u < kXPer; u++) {
+        const int c = u * 64 * W + tid;
+        xv[u] = c < row_chunks ? reinterpret_cast<const u4_t *>(x)[c] : u4_t{0u, 0u, 0u, 0u};
+    }
+
+    const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;   // k steps of this wave per row block
+    const int nb_wg = ((int)blockIdx.x < n_blocks)
+                          ? (n_blocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
+    // per-lane byte offset inside a row block (never changes) ...
+    int voff[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) voff[r] = (16 * r + c16) * row_bytes + q * 16;
+    // ... and the scalar part: row block and k step of the next item to prefetch.  Rows past N
+    // land past the end of the buffer by themselves; items past the end get an offset no
+    // buffer reaches.
+    constexpr int kOut = (int)0x80000000;
+    int pf_blk = 0, pf_j = 0;
+    auto issue = [&](u4_t (&cwd)[R]) {
+        const bool ok = pf_blk < nb_wg && n_sw > 0;
+#ifdef DMM_TRACE
+        const bool ok2 = ok && dmm_exp_mode != 2;
+#else
+        const bool ok2 = ok;
+#endif
+        const int soff = ok2 ? ((int)blockIdx.x + pf_blk * (int)gridDim.x) * (16 * R) * row_bytes + (wave + pf_j * W) * 64
+                             : kOut;
+#pragma unroll
+        for (int r = 0; r < R; r++) cwd[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], soff, 0);
+        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
+    };
+
+    u4_t cw[D][R];
+#pragma unroll
+    for (int d = 0; d < D; d++) issue(cw[d]);
+    DMM_TRACE_MARK(1);
+
+    // x -> LDS (padded pitch): the pieces of row 0 fetched above, then whatever is left
+#pragma unroll
+    for (int u = 0; u < kXPer; u++) {
+        const int c = u * 64 * W + tid;
+        if (c < row_chunks) reinterpret_cast<u4_t *>(xs)[c] = xv[u];
+    }
+    for (int c = kXPer * 64 * W + tid; c < row_chunks; c += 64 * W)
+        reinterpret_cast<u4_t *>(xs)[c] = reinterpret_cast<const u4_t *>(x)[c];
+    for (int m = 1; m < M; m++)
+        for (int c = tid; c < row_chunks; c += 64 * W)
+            reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = reinterpret_cast<const u4_t *>(x + (int64_t)m * K)[c];
+    DMM_TRACE_MARK(2);
+    stream_stage_tables<64 * W>(smem_raw, grow, tid);
+    DMM_TRACE_MARK(3);
+    __syncthreads();
+    DMM_TRACE_MARK(4);
+
+    // B operand address of this lane: row m = c16 (row 0 for columns past M), quarter q
+    const uint32_t xlane = lds_addr(xs) + (uint32_t)((c16 < M ? c16 : 0) * x_pitch + q * 128);
+
+    f4_t acc[R][2];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+
+    // publish this wave's partial sums of a finished row block, meet the other waves, and
+    // let wave r (< R) add up and store row tile r
+    auto finish_block = [&](int blk) {
+        f4_t *rp = red + (blk & 1) * red_par;
+        if (c16 < M) {
+#pragma unroll
+            for (int r = 0; r < R; r++) rp[(wave * R + r) * 4 * M + q * M + c16] = acc[r][0] + acc[r][1];
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+        if (wave < R && c16 < M) {
+            f4_t sacc = rp[(0 * R + wave) * 4 * M + q * M + c16];
+#pragma unroll
+            for (int w = 1; w < W; w++) sacc += rp[(w * R + wave) * 4 * M + q * M + c16];
+            const int n = ((int)blockIdx.x + blk * (int)gridDim.x) * (16 * R) + 16 * wave + 4 * q;
+            if (n < N) {   // N % 4 == 0, so the four rows are in range together
+                h4_t o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = (half_t)(sacc[e] * scale);
+                *reinterpret_cast<h4_t *>(y + (int64_t)c16 * N + n) = o;
+            }
+        }
+    };
+
+    if (n_sw == 0) {
+        // no k step for this wave (K shorter than the workgroup is wide): it still meets the
+        // others at every row block's barrier, contributing zeros
+        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
+        return;
+    }
+
+    const int n_items = nb_wg * n_sw;
+    int blk = 0, j = 0;
+    for (int i0 = 0; i0 < n_items; i0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (i0 + d < n_items) {
+#ifdef DMM_TRACE
+                if (i0 + d < 7) { asm volatile("" ::"v"(cw[d][0])); DMM_TRACE_MARK(8 + 2 * (i0 + d)); }
+                if (dmm_exp_mode == 1) {
+#pragma unroll
+                    for (int r = 0; r < R; r++) acc[r][0][0] += __builtin_bit_cast(float, cw[d][r][0] ^ cw[d][r][1] ^ cw[d][r][2] ^ cw[d][r][3]);
+                } else
+#endif
+                stream_step<R>(cw[d], xlane + (uint32_t)((wave + j * W) * 512), lane_base, quarter_bits, acc);
+                if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
+                if (++j >= n_sw) {
+                    j = 0;
+                    if (blk == 0) DMM_TRACE_MARK(5);
+                    finish_block(blk);
+                    if (blk == 0) DMM_TRACE_MARK(6);
+                    blk++;
+                }
+            }
+            issue(cw[d]);
+        }
+    }
+    DMM_TRACE_MARK(7);
+    DMM_TRACE_DUMP();
 }
 
 // ------------------------------------------------------------------ matrix-matrix path
@@ -492,7 +884,7 @@ int check_common(const void *x, const void *codes, const void *grid, const void 
 bool gemv_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
              int64_t K)
 {
-    return M >= 1 && M <= 32 && K >= 256 && (K & 255) == 0 && (N & 3) == 0 && aligned(x, 16) &&
+    return M >= 1 && M <= 32 && K >= 256 && (K & 255) == 0 && K <= (1 << 23) && (N & 3) == 0 && aligned(x, 16) &&
            aligned(codes, 16) && aligned(grid, 16) && aligned(y, 8);
 }
 
@@ -507,7 +899,7 @@ template <int R, int W, int MT>
 int launch_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                 int64_t N, int64_t K, hipStream_t stream)
 {
-    const size_t shmem = sizeof(GemvShared<R, W, MT>);
+    const size_t shmem = kGemvTableBytes;
     static bool attr_done = false;   // benign race: every thread sets the same value
     if (!attr_done && shmem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_kernel<R, W, MT>),
@@ -521,11 +913,95 @@ int launch_gemv(const void *x, const void *codes, const void *grid, float scale,
                   (int)K);
 }
 
+// Tuning override for experiments: DMM_GEMV_CFG="R,W,D" picks the streaming kernel instance
+// (rows per block = 16 R, W waves, D prefetched steps per wave), "R,W" the non-streaming one;
+// unset or unknown -> the default choice.
+int gemv_cfg_override()
+{
+    static int cfg = -1;
+    if (cfg < 0) {
+        cfg = 0;
+        if (const char *e = getenv("DMM_GEMV_CFG")) {
+            int r = 0, w = 0, d = 0;
+            const int n = sscanf(e, "%d,%d,%d", &r, &w, &d);
+            if (n >= 2) cfg = r * 10000 + w * 100 + (n == 3 ? d : 0);
+        }
+    }
+    return cfg;
+}
+
+int cu_count()
+{
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n = prop.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
+template <int R, int W, int D>
+int launch_gemv_stream(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                       int64_t N, int64_t K, hipStream_t stream)
+{
+#ifdef DMM_TRACE
+    const size_t shmem = 160 * 1024;
+#else
+    const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)M * (2 * K + 16);
+#endif
+    static bool attr_done = false;   // benign race: every thread sets the same value
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_stream_kernel<R, W, D>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const int64_t n_blocks = (N + 16 * R - 1) / (16 * R);
+    const int64_t wgs = n_blocks < cu_count() ? n_blocks : cu_count();
+    return launch(gemv_stream_kernel<R, W, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  (int)n_blocks);
+}
+
+// tables, partial sums and x fit in the 160 KB of LDS, and every byte offset of the code
+// matrix fits the 31 bits the buffer addressing is used with
+template <int R, int W>
+bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
+{
+    return M <= 16 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + M * (2 * K + 16) <= 160 * 1024 &&
+           N * (K >> 2) < (1LL << 31);
+}
+
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
-    if (M <= 16) return launch_gemv<2, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
-    return launch_gemv<2, 8, 2>(x, codes, grid, scale, y, M, N, K, stream);
+    if (M > 16) return launch_gemv<2, 8, 2>(x, codes, grid, scale, y, M, N, K, stream);
+#define DMM_STREAM_CASE(R, W, D)                                                                   \
+    case R * 10000 + W * 100 + D:                                                                  \
+        if (gemv_stream_ok<R, W>(M, N, K))                                                         \
+            return launch_gemv_stream<R, W, D>(x, codes, grid, scale, y, M, N, K, stream);         \
+        break;
+    switch (gemv_cfg_override()) {
+        DMM_STREAM_CASE(1, 8, 4)
+        DMM_STREAM_CASE(1, 8, 8)
+        DMM_STREAM_CASE(2, 8, 4)
+        DMM_STREAM_CASE(2, 8, 8)
+        DMM_STREAM_CASE(1, 16, 4)
+        DMM_STREAM_CASE(1, 16, 6)
+        DMM_STREAM_CASE(2, 16, 2)
+        DMM_STREAM_CASE(2, 16, 3)
+        DMM_STREAM_CASE(2, 16, 4)
+        case 10800: return launch_gemv<1, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
+        case 20800: return launch_gemv<2, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
+        case 40800: return launch_gemv<4, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
+        default: break;
+    }
+#undef DMM_STREAM_CASE
+    if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2>(x, codes, grid, scale, y, M, N, K, stream);
+    return launch_gemv<2, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
 }
 
 int run_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
@@ -562,6 +1038,17 @@ int run_generic(const void *x, const void *codes, const void *grid, float scale,
 using namespace dmm;
 
 extern "C" {
+
+#ifdef DMM_TRACE
+int dmm_debug_set_trace(void *buf)
+{
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(dmm::dmm_trace_buf), &buf, sizeof(buf));
+}
+int dmm_debug_set_mode(int mode)
+{
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(dmm::dmm_exp_mode), &mode, sizeof(mode));
+}
+#endif
 
 int dmm_version(void) { return (0 << 16) | 1; }
 
