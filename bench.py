@@ -24,6 +24,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
+# HBM bytes one GEMV launch moves, averaged over the four shapes: rocprofv3 FETCH_SIZE and
+# WRITE_SIZE per dispatch (19,134.7 KiB and 27.0 KiB), each scaled by what the same counter
+# reads for a plain 256 MiB device copy (x2.000 and x1.000).  Algorithmic code bytes: 38,797,312.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 39215000
 
 
 def parse():
@@ -33,6 +37,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="skip prefill / small-batch / CPU legs")
     ap.add_argument("--rotate-mb", type=int, default=400, help="distinct code bytes to rotate through, at least")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch 8 plain device copies of 256 MiB first (a known-size reference for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     return ap.parse_args()
 
 
@@ -68,6 +75,14 @@ def main():
         g.manual_seed(seed)
         return [torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=dev)
                 for _ in range(copies)]
+
+    if args.copy_calibration:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(8):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---------------------------------------------------------------- headline: 70B GEMV
     shapes = workload.LLAMA2_70B
@@ -141,8 +156,8 @@ def main():
                    "M": 1, "code_buffers_rotated": copies, "distinct_code_MB": round(copies * step_bytes / 1e6, 1),
                    "step": "4 GEMVs, one per shape"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "dmm::gemv_kernel", "launches": n_launch,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "dmm::gemv_stream_kernel", "launches": n_launch,
                      "avg_launch_us": round(kern_s / n_launch * 1e6, 3),
                      "algorithmic_bytes_per_launch": step_bytes / len(probs)},
         "gemv_shapes": shape_rows,
