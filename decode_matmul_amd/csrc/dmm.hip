@@ -729,111 +729,214 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 }
 
 // ------------------------------------------------------------------ matrix-matrix path
-// Block tile 128 (n) x 128 (m) x 64 (k), 4 waves as 2 x 2, each wave 64 x 64 with
-// v_mfma_f32_32x32x16_f16 (A = decoded W rows, B = x rows, fp32 accumulate).  Per k tile
-// every thread decodes four codes of one W row into LDS and copies 64 bytes of x into LDS;
-// the global loads of tile k+1 are issued before the MFMAs of tile k.
-constexpr int kGemmBN = 128, kGemmBM = 128, kGemmBK = 64;
-constexpr int kGemmLd = kGemmBK + 8;   // halves per LDS row: 144 B keeps 16-byte alignment, staggers banks
+// Block tile BN (n) x BM (m) x 64 (k) with WN x WM waves, each wave TN x TM tiles of
+// v_mfma_f32_32x32x16_f16 (A = decoded W rows, B = x rows, fp32 accumulate).  A wide n keeps
+// x re-reads down (x is fetched once per BN output columns) and a tall m amortises the decode.
+//
+// The k loop is software-pipelined three deep so that the matrix unit never waits for
+// staging: while the MFMAs of tile kt run out of LDS buffer kt%2, the same waves decode tile
+// kt+1 (whose codes and x already sit in registers) into buffer (kt+1)%2 - a quarter of that
+// work after each group of MFMAs, in the matrix unit's shadow - and the global loads of tiles
+// kt+2 .. kt+4 are in flight.  One barrier per k tile.  LDS rows are 144 bytes apart (9 bank groups),
+// so the 16 lanes the LDS serves per clock - 16 consecutive rows at the same k - hit 16
+// different groups.
+constexpr int kGemmBK = 64;
+constexpr int kGemmLd = kGemmBK + 8;   // halves per LDS row
 
-struct GemmShared {
-    DecodeTables tab;
-    uint16_t w[kGemmBN][kGemmLd];
-    uint16_t x[kGemmBM][kGemmLd];
+template <int WN, int WM, int TN, int TM>
+struct GemmCfg {
+    static constexpr int kThreads = 64 * WN * WM;
+    static constexpr int kBN = WN * TN * 32;
+    static constexpr int kBM = WM * TM * 32;
+    static constexpr int kTPR = kThreads / kBN;            // threads sharing one W row (1 or 2)
+    static constexpr int kCPT = 8 / kTPR;                  // codes per thread per k tile
+    static constexpr int kXPT = kBM * 8 / kThreads;        // 16-byte pieces of x per thread per k tile
+    static constexpr int kXTPR = 8 / kXPT;                 // threads sharing one x row
+    static_assert(kTPR == 1 || kTPR == 2, "one or two threads per W row");
+    static_assert(kXPT >= 1 && kXPT <= 8 && 8 % kXPT == 0, "x pieces per thread");
+    struct Shared {
+        DecodeTables tab;
+        uint16_t w[2][kBN][kGemmLd];
+        uint16_t x[2][kBM][kGemmLd];
+    };
 };
 
-__global__ __launch_bounds__(256) void gemm_kernel(const uint16_t *__restrict__ x,
-                                                   const uint16_t *__restrict__ codes,
-                                                   const void *__restrict__ grid, float scale,
-                                                   uint16_t *__restrict__ y, int M, int N, int K)
+// decode of one code with the packed delta taken from the low / high half of dd
+template <bool kHi>
+__device__ __forceinline__ u4_t gemm_decode(uint32_t code, uint32_t dd, const DecodeTables &t)
 {
-    __shared__ GemmShared sh;
+    const u4_t g = t.grid[code & 0xFFu];
+    const u4_t sg = t.sign[(code >> 8) & 0x7Fu];
+    u4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = pk_fma_bcast<kHi>(g[i], sg[i], dd);
+    return r;
+}
+
+template <int WN, int WM, int TN, int TM>
+__global__ __launch_bounds__(64 * WN * WM) void gemm_kernel(const uint16_t *__restrict__ x,
+                                                            const uint16_t *__restrict__ codes,
+                                                            const void *__restrict__ grid, float scale,
+                                                            uint16_t *__restrict__ y, int M, int N, int K)
+{
+    typedef GemmCfg<WN, WM, TN, TM> C;
+    extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
+    typename C::Shared &sh = *reinterpret_cast<typename C::Shared *>(gemm_smem);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wn = wave & 1, wm = wave >> 1;
-    const int n0 = blockIdx.x * kGemmBN;
-    const int m0 = blockIdx.y * kGemmBM;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave % WN, wm = wave / WN;
+    const int n0 = blockIdx.x * C::kBN;
+    const int m0 = blockIdx.y * C::kBM;
     const int k_tiles = K / kGemmBK;
     const int64_t kc = K >> 3;
 
-    stage_tables<true>(sh.tab, grid, tid, 256);
+    stage_tables<true>(sh.tab, grid, tid, C::kThreads);
 
-    // W staging: thread -> row tid/2, codes 4*(tid%2) .. +3 of the k tile (8 bytes)
-    const int w_row = tid >> 1, w_half = tid & 1;
+    // W staging: thread -> row tid / kTPR, kCPT codes of the k tile
+    const int w_row = tid / C::kTPR, w_part = tid % C::kTPR;
     int wr = n0 + w_row;
     wr = wr < N ? wr : N - 1;
-    const uint16_t *wsrc = codes + (int64_t)wr * kc + w_half * 4;
-    // x staging: thread -> row tid/2, 32 halves (64 bytes) starting at 32*(tid%2)
-    int xr = m0 + w_row;
+    const uint16_t *wsrc = codes + (int64_t)wr * kc + w_part * C::kCPT;
+    // x staging: thread -> row tid / kXTPR, kXPT pieces of 8 halves
+    const int x_row = tid / C::kXTPR, x_part = tid % C::kXTPR;
+    int xr = m0 + x_row;
     const bool x_in = xr < M;
     xr = x_in ? xr : M - 1;
-    const uint16_t *xsrc = x + (int64_t)xr * K + w_half * 32;
+    const uint16_t *xsrc = x + (int64_t)xr * K + x_part * C::kXPT * 8;
 
-    u2_t cw = *reinterpret_cast<const u2_t *>(wsrc);
-    u4_t xv[4];
+    struct Stage {
+        uint32_t cw[C::kCPT / 2];
+        u4_t xv[C::kXPT];
+    };
+    auto load_tile = [&](Stage &st, int kt) {
+        kt = kt < k_tiles ? kt : k_tiles - 1;    // past the end: reload the last tile (never used)
+        const uint32_t *wp = reinterpret_cast<const uint32_t *>(wsrc + (int64_t)kt * 8);
+        if (C::kCPT == 8) {
+            const u4_t v = *reinterpret_cast<const u4_t *>(wp);
 #pragma unroll
-    for (int i = 0; i < 4; i++) xv[i] = reinterpret_cast<const u4_t *>(xsrc)[i];
+            for (int i = 0; i < C::kCPT / 2; i++) st.cw[i] = v[i];
+        } else {
+            const u2_t v = *reinterpret_cast<const u2_t *>(wp);
+#pragma unroll
+            for (int i = 0; i < C::kCPT / 2; i++) st.cw[i] = v[i];
+        }
+#pragma unroll
+        for (int i = 0; i < C::kXPT; i++) st.xv[i] = reinterpret_cast<const u4_t *>(xsrc + (int64_t)kt * kGemmBK)[i];
+    };
+    // One quarter (q = 0..3) of a thread's staging work for LDS buffer `buf`, in two halves:
+    // the table gathers are issued before a group of MFMAs, the packed FMAs and the LDS writes
+    // run after it, in the matrix unit's shadow.
+    constexpr int kCq = C::kCPT / 4;             // codes per quarter: 1 or 2
+    struct Gathered {
+        u4_t g[kCq], sg[kCq];
+    };
+    auto stage_gather = [&](Gathered &o, const Stage &st, int q) {
+#pragma unroll
+        for (int c = 0; c < kCq; c++) {
+            const int ci = q * kCq + c;          // code index within the thread's kCPT
+            const uint32_t code = (ci & 1) ? st.cw[ci >> 1] >> 16 : st.cw[ci >> 1];
+            o.g[c] = sh.tab.grid[code & 0xFFu];
+            o.sg[c] = sh.tab.sign[(code >> 8) & 0x7Fu];
+        }
+    };
+    auto stage_finish = [&](const Gathered &o, const Stage &st, int buf, int q) {
+#pragma unroll
+        for (int c = 0; c < kCq; c++) {
+            const int ci = q * kCq + c;
+            const uint32_t dd = (st.cw[ci >> 1] & 0x80008000u) | 0x34003400u;
+            u4_t wv;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                wv[i] = (ci & 1) ? pk_fma_bcast<true>(o.g[c][i], o.sg[c][i], dd) : pk_fma_bcast<false>(o.g[c][i], o.sg[c][i], dd);
+            *reinterpret_cast<u4_t *>(&sh.w[buf][w_row][(w_part * C::kCPT + ci) * 8]) = wv;
+        }
+        const u4_t zero = u4_t{0u, 0u, 0u, 0u};
+        if (C::kXPT >= 4) {
+#pragma unroll
+            for (int i = 0; i < C::kXPT / 4; i++) {
+                const int pi = q * (C::kXPT / 4) + i;
+                *reinterpret_cast<u4_t *>(&sh.x[buf][x_row][(x_part * C::kXPT + pi) * 8]) = x_in ? st.xv[pi] : zero;
+            }
+        } else if (q < C::kXPT) {
+            *reinterpret_cast<u4_t *>(&sh.x[buf][x_row][(x_part * C::kXPT + q) * 8]) = x_in ? st.xv[q] : zero;
+        }
+    };
 
-    f16_t acc[2][2];
+    // ring of four stages: tile kt+1 is staged out of ring[(kt+1)%4] while tile kt+4 is fetched
+    // into ring[kt%4], so a global load has three tiles of MFMAs to arrive
+    Stage ring[4];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 4; i++) load_tile(ring[i], i);
+
+    f16_t acc[TN][TM];
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
     const int l32 = lane & 31, kq = lane >> 5;
     __syncthreads();   // tables ready
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        Gathered gq;
+        stage_gather(gq, ring[0], q);
+        stage_finish(gq, ring[0], 0, q);
+    }
+    __syncthreads();   // tile 0 staged
 
-    for (int kt = 0; kt < k_tiles; kt++) {
-        // registers -> LDS (decode W on the way)
-        {
-            u4_t w0, w1, w2, w3;
-            decode8x2(cw[0], sh.tab, w0, w1);
-            decode8x2(cw[1], sh.tab, w2, w3);
-            u4_t *dst = reinterpret_cast<u4_t *>(&sh.w[w_row][w_half * 32]);
-            dst[0] = w0; dst[1] = w1; dst[2] = w2; dst[3] = w3;
-            u4_t *xd = reinterpret_cast<u4_t *>(&sh.x[w_row][w_half * 32]);
-            const u4_t zero = u4_t{0u, 0u, 0u, 0u};
+    // Compute tile kt from buffer `buf` while staging tile kt+1 (registers sn) into the other
+    // buffer and fetching tile kt+4 into sf.  Operand fragments are double-buffered in
+    // registers: those of k step ks+1 are requested before the MFMAs of step ks are issued.
+    auto read_frags = [&](h8_t (&a)[TN], h8_t (&b)[TM], int buf, int ks) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) xd[i] = x_in ? xv[i] : zero;
+        for (int i = 0; i < TN; i++)
+            a[i] = *reinterpret_cast<const h8_t *>(&sh.w[buf][(wn * TN + i) * 32 + l32][ks * 16 + kq * 8]);
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+            b[j] = *reinterpret_cast<const h8_t *>(&sh.x[buf][(wm * TM + j) * 32 + l32][ks * 16 + kq * 8]);
+    };
+    auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf) {
+        const bool staging = kt + 1 < k_tiles;
+        load_tile(sf, kt + 4);
+        h8_t a[2][TN], b[2][TM];
+        read_frags(a[0], b[0], buf, 0);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            if (ks < 3) read_frags(a[(ks + 1) & 1], b[(ks + 1) & 1], buf, ks + 1);
+            Gathered gq;
+            if (staging) stage_gather(gq, sn, ks);
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int j = 0; j < TM; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
+            if (staging) stage_finish(gq, sn, buf ^ 1, ks);
+            __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();
-        if (kt + 1 < k_tiles) {
-            cw = *reinterpret_cast<const u2_t *>(wsrc + (int64_t)(kt + 1) * 8);
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                xv[i] = reinterpret_cast<const u4_t *>(xsrc + (int64_t)(kt + 1) * kGemmBK)[i];
-        }
-#pragma unroll
-        for (int ks = 0; ks < kGemmBK / 16; ks++) {
-            h8_t a[2], b[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                a[i] = *reinterpret_cast<const h8_t *>(&sh.w[wn * 64 + i * 32 + l32][ks * 16 + kq * 8]);
-                b[i] = *reinterpret_cast<const h8_t *>(&sh.x[wm * 64 + i * 32 + l32][ks * 16 + kq * 8]);
-            }
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads();
+    };
+
+    for (int kt = 0; kt < k_tiles; kt += 4) {
+        tile(kt, 0, ring[1], ring[0]);
+        if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1]);
+        if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
+        if (kt + 3 < k_tiles) tile(kt + 3, 1, ring[0], ring[3]);
     }
 
     // D layout of 32x32: element e of lane: row (n) = 8*(e/4) + 4*(lane/32) + e%4, column (m) = lane%32
     const bool n_vec = (N & 3) == 0;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < TN; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int m = m0 + wm * 64 + j * 32 + l32;
+        for (int j = 0; j < TM; j++) {
+            const int m = m0 + (wm * TM + j) * 32 + l32;
             if (m >= M) continue;
 #pragma unroll
             for (int e4 = 0; e4 < 4; e4++) {
-                const int n = n0 + wn * 64 + i * 32 + 8 * e4 + 4 * kq;
+                const int n = n0 + (wn * TN + i) * 32 + 8 * e4 + 4 * kq;
                 uint16_t o[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++)
@@ -892,7 +995,7 @@ bool gemm_ok(const void *x, const void *codes, const void *grid, const void *, i
              int64_t K)
 {
     return M >= 1 && N >= 1 && K >= 64 && (K & 63) == 0 && aligned(x, 16) && aligned(codes, 16) &&
-           aligned(grid, 16) && M <= 65535LL * kGemmBM;
+           aligned(grid, 16) && M <= 65535LL * 128;
 }
 
 template <int R, int W, int MT>
@@ -1004,12 +1107,40 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
     return launch_gemv<2, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
 }
 
+template <int WN, int WM, int TN, int TM>
+int launch_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                int64_t N, int64_t K, hipStream_t stream)
+{
+    typedef GemmCfg<WN, WM, TN, TM> C;
+    static bool attr_done = false;   // benign race: every thread sets the same value
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<WN, WM, TN, TM>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(typename C::Shared));
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    dim3 g((unsigned)((N + C::kBN - 1) / C::kBN), (unsigned)((M + C::kBM - 1) / C::kBM));
+    return launch(gemm_kernel<WN, WM, TN, TM>, g, dim3(C::kThreads), sizeof(typename C::Shared), stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
+}
+
+// Tuning override for experiments: DMM_GEMM_CFG=a|b|c|d picks the tile configuration.
 int run_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
-    dim3 g((unsigned)((N + kGemmBN - 1) / kGemmBN), (unsigned)((M + kGemmBM - 1) / kGemmBM));
-    return launch(gemm_kernel, g, dim3(256), 0, stream, (const uint16_t *)x, (const uint16_t *)codes, grid,
-                  scale, (uint16_t *)y, (int)M, (int)N, (int)K);
+    static int cfg = -1;
+    if (cfg < 0) {
+        const char *e = getenv("DMM_GEMM_CFG");
+        cfg = e ? e[0] : 'a';
+    }
+    switch (cfg) {
+        case 'b': return launch_gemm<2, 2, 4, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 256 x 128, 4 waves
+        case 'd': return launch_gemm<2, 4, 4, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 256 x 256, 8 waves
+        case 'g': return launch_gemm<2, 2, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 128 x 128, 4 waves, 2 per CU
+        case 'h': return launch_gemm<2, 2, 4, 2>(x, codes, grid, scale, y, M, N, K, stream);
+        default: break;
+    }
+    return launch_gemm<4, 2, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);                 // 256 x 128, 8 waves
 }
 
 // y = 0 when K == 0 (empty sum), any M, N.
