@@ -200,51 +200,18 @@ __global__ __launch_bounds__(256) void generic_kernel(const uint16_t *__restrict
     }
 }
 
-// ------------------------------------------------------------------ matrix-vector path (M <= 16*MT)
-// Workgroup = W waves, owns 16*R consecutive rows of W for the whole of K; the waves split
-// K in interleaved 256-wide steps.  In one step a lane (row r = lane%16 of each 16-row
-// tile, quarter q = lane/16) loads 8 consecutive codes (16 bytes) of its row, decodes them
-// one at a time and feeds each as the A operand (16 rows x 32 k: this lane supplies the 8
-// k of its quarter) of v_mfma_f32_16x16x32_f16.  The B operand is x: column c = lane%16 is
-// row m = c of x, same 8 k.  Any k order works as long as A and B agree, so the 32 k of
-// MFMA number t in a step are {64*q + 8*t .. +8 : q = 0..3} rather than 32 consecutive k;
-// that is what lets the code load be one 16-byte load per lane.  For M = 1 only column 0
-// carries data, the other 15 columns cost nothing extra: the matrix unit has the headroom.
+// ------------------------------------------------------------------ matrix-vector paths (M <= 32)
+// A workgroup owns 16*R consecutive rows of W for the whole of K; its W waves split K in
+// interleaved 256-wide steps.  In one step a lane (row r = lane%16 of each 16-row tile,
+// quarter q = lane/16) loads 8 consecutive codes (16 bytes) of its row, decodes them one at a
+// time and feeds each as the A operand (16 rows x 32 k: this lane supplies the 8 k of its
+// quarter) of v_mfma_f32_16x16x32_f16.  The B operand is x: column c = lane%16 is row m = c of
+// x, same 8 k.  Any k order works as long as A and B agree, so the 32 k of MFMA number t in a
+// step are {64*q + 8*t .. +8 : q = 0..3} rather than 32 consecutive k; that is what lets the
+// code load be one 16-byte load per lane.  For M = 1 only column 0 carries data, the other 15
+// columns cost nothing extra: the matrix unit has the headroom.
 // Accumulator layout: lane holds rows 4*q + i (i = 0..3) of column c, i.e.
 // y[m = c][n = n0 + 4*q + i] - four consecutive halves of a row of y.
-//
-// What bounds the kernel is the LDS, not HBM: every code costs two 16-byte LDS gathers
-// (grid row, sign row) and the LDS delivers 128 bytes per clock per CU only when the 8
-// lanes it serves in one clock hit 8 different 16-byte bank groups.  Random rows collide,
-// so the tables are stored 8 times over: one unified table of 256 rows x 256 bytes, row i =
-// [grid row i, 8 copies | sign row (i & 127), 8 copies], and a lane reads copy lane%8.
-// Gathers are then conflict-free whatever the codes are, and - because the row pitch is
-// 256 - a table address is just a byte of the code word placed above the lane's copy
-// offset, one v_perm_b32: the low byte of a code addresses its grid row, the high byte
-// (7 sign bits + the shift bit, hence the 256 sign rows) its sign row at +128.
-constexpr int kGemvTableBytes = 256 * 256;
-
-// Thread tid fills table slots tid, tid + nthreads, ...: slot j is copy (j % 16) of row j / 16.
-// The grid rows it needs are fetched by gemv_fetch_grid beforehand, so that the global loads
-// are the first ones the kernel issues and nothing queues behind the code stream.
-template <int kNThreads>
-__device__ __forceinline__ void gemv_fetch_grid(u4_t (&g)[4096 / kNThreads], const void *grid, int tid)
-{
-#pragma unroll
-    for (int i = 0; i < 4096 / kNThreads; i++) g[i] = reinterpret_cast<const u4_t *>(grid)[(tid + i * kNThreads) >> 4];
-}
-
-template <int kNThreads>
-__device__ __forceinline__ void stage_gemv_tables(unsigned char *tab, const u4_t (&g)[4096 / kNThreads], int tid)
-{
-    u4_t *t = reinterpret_cast<u4_t *>(tab);
-#pragma unroll
-    for (int i = 0; i < 4096 / kNThreads; i++) {
-        const int j = tid + i * kNThreads;
-        t[j] = (j & 8) ? sign_row((uint32_t)((j >> 4) & 0x7F)) : g[i];
-    }
-}
-
 typedef __attribute__((address_space(3))) const u4_t lds_u4_t;
 
 // 32-bit LDS byte address of a pointer into shared memory
@@ -268,171 +235,6 @@ __device__ __forceinline__ uint32_t pk_fma_bcast(uint32_t g, uint32_t s, uint32_
     else
         asm("v_pk_fma_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,1,0]" : "=v"(r) : "v"(g), "v"(s), "v"(dd));
     return r;
-}
-
-// One 32-bit word = two codes.  Its decode is split in two so that the LDS gathers of the
-// next word can be in flight while the packed FMAs and MFMAs of this one issue.
-struct GemvGather {
-    u4_t g0, s0, g1, s1;   // grid row / sign row of code 0, of code 1
-    uint32_t dd;           // (+-0.25 for code 0, +-0.25 for code 1) as packed halves
-};
-
-// lane_base: LDS byte address of this lane's table copy, table base + (lane % 8) * 16 (< 256)
-__device__ __forceinline__ void gemv_gather(GemvGather &o, uint32_t w, uint32_t lane_base)
-{
-    o.g0 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));          // byte 0 of w << 8 | lane_base
-    o.s0 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0500u) + 128u);
-    o.g1 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
-    o.s1 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0700u) + 128u);
-    o.dd = (w & 0x80008000u) | 0x34003400u;
-}
-
-__device__ __forceinline__ void gemv_finish(const GemvGather &o, h8_t &a0, h8_t &a1)
-{
-    u4_t r0, r1;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        r0[i] = pk_fma_bcast<false>(o.g0[i], o.s0[i], o.dd);
-        r1[i] = pk_fma_bcast<true>(o.g1[i], o.s1[i], o.dd);
-    }
-    a0 = __builtin_bit_cast(h8_t, r0);
-    a1 = __builtin_bit_cast(h8_t, r1);
-}
-
-// One 256-wide k step for R row tiles: 4R words, gathers one word ahead of the math.
-// acc[r][mt][0/1]: the even and odd codes of a word accumulate separately, so that
-// consecutive MFMAs never depend on each other.
-template <int R, int MT>
-__device__ __forceinline__ void gemv_step(const u4_t (&cw)[R], const u4_t (&xb)[MT][8], uint32_t lane_base,
-                                          f4_t (&acc)[R][MT][2])
-{
-    constexpr int kItems = 4 * R;       // item i: word t2 = i / R of row tile r = i % R
-    GemvGather buf[2];
-    gemv_gather(buf[0], cw[0][0], lane_base);
-#pragma unroll
-    for (int i = 0; i < kItems; i++) {
-        const int t2 = i / R, r = i % R;
-        if (i + 1 < kItems) gemv_gather(buf[(i + 1) & 1], cw[(i + 1) % R][(i + 1) / R], lane_base);
-        h8_t a0, a1;
-        gemv_finish(buf[i & 1], a0, a1);
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            acc[r][mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                a0, __builtin_bit_cast(h8_t, xb[mt][2 * t2]), acc[r][mt][0], 0, 0, 0);
-            acc[r][mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                a1, __builtin_bit_cast(h8_t, xb[mt][2 * t2 + 1]), acc[r][mt][1], 0, 0, 0);
-        }
-    }
-}
-
-template <int R, int W, int MT>
-__global__ __launch_bounds__(64 * W) void gemv_kernel(const uint16_t *__restrict__ x,
-                                                      const uint16_t *__restrict__ codes,
-                                                      const void *__restrict__ grid, float scale,
-                                                      uint16_t *__restrict__ y, int M, int N, int K)
-{
-    // the decode table, and - once every wave is done with it - the split-K partial sums
-    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    typedef f4_t red_t[R * MT][kWave];
-    static_assert(sizeof(red_t) * W <= kGemvTableBytes, "partials must fit in the table's space");
-    red_t *red = reinterpret_cast<red_t *>(smem_raw);
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int c16 = lane & 15;   // row within a 16-row tile (A) / column m within an m-tile (B)
-    const int q = lane >> 4;     // k quarter
-    const int n_steps = K >> 8;  // 256 k per step
-    const int64_t row_bytes = (int64_t)K >> 2;  // K/8 codes * 2 bytes
-    const int row0 = blockIdx.x * (16 * R);
-    const uint32_t lane_base = lds_addr(smem_raw) + (uint32_t)(lane & 7) * 16u;
-
-    // per-tile code pointers; rows past N are clamped (their results are never stored)
-    const unsigned char *cptr[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        int row = row0 + 16 * r + c16;
-        row = row < N ? row : N - 1;
-        cptr[r] = reinterpret_cast<const unsigned char *>(codes) + row * row_bytes + q * 16;
-    }
-    // x goes through a buffer descriptor: lane's column c16 is row m of x (per m-tile), its
-    // quarter starts at 64*q.  Columns past M get an offset beyond the buffer, which the
-    // hardware answers with zeros without touching memory - for M = 1 only 4 lanes of the
-    // wave fetch anything - and there is no branch for the wait counters to lose track at.
-    const __amdgpu_buffer_rsrc_t xrsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, M * K * 2, 0x00020000);
-    int xoff[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-        const int m = 16 * mt + c16;
-        xoff[mt] = m < M ? (m * K + 64 * q) * 2 : 0x7F000000;
-    }
-
-    auto load_codes = [&](u4_t (&cw)[R], int step) {
-#pragma unroll
-        for (int r = 0; r < R; r++)
-            cw[r] = __builtin_nontemporal_load(reinterpret_cast<const u4_t *>(cptr[r] + (int64_t)step * 64));
-    };
-    auto load_x = [&](u4_t (&xb)[MT][8], int step) {
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-            for (int t = 0; t < 8; t++)
-                xb[mt][t] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff[mt] + step * 512 + t * 16, 0, 0);
-    };
-
-    // grid rows first, then the first two steps' loads; the table is built while those fly
-    u4_t gtmp[4096 / (64 * W)];
-    gemv_fetch_grid<64 * W>(gtmp, grid, tid);
-    u4_t cw0[R], cw1[R];
-    u4_t xb0[MT][8], xb1[MT][8];
-    int step = wave;
-    if (step < n_steps) { load_codes(cw0, step); load_x(xb0, step); }
-    if (step + W < n_steps) { load_codes(cw1, step + W); load_x(xb1, step + W); }
-
-    stage_gemv_tables<64 * W>(smem_raw, gtmp, tid);
-    __syncthreads();
-
-    f4_t acc[R][MT][2];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) acc[r][mt][0] = acc[r][mt][1] = f4_t{0.f, 0.f, 0.f, 0.f};
-
-    // two steps per trip, ping-pong between the register buffers: each buffer is refilled
-    // (for two steps ahead) right after it has been consumed
-    while (step < n_steps) {
-        gemv_step<R, MT>(cw0, xb0, lane_base, acc);
-        if (step + 2 * W < n_steps) { load_codes(cw0, step + 2 * W); load_x(xb0, step + 2 * W); }
-        if (step + W >= n_steps) break;
-        gemv_step<R, MT>(cw1, xb1, lane_base, acc);
-        if (step + 3 * W < n_steps) { load_codes(cw1, step + 3 * W); load_x(xb1, step + 3 * W); }
-        step += 2 * W;
-    }
-
-    // cross-wave (split-K) reduction through LDS, then scale, round to half and store
-    __syncthreads();   // every wave has finished reading the table
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) red[wave][r * MT + mt][lane] = acc[r][mt][0] + acc[r][mt][1];
-    __syncthreads();
-    for (int idx = tid; idx < R * MT * kWave; idx += 64 * W) {
-        const int l = idx & 63;
-        const int tile = idx >> 6;
-        const int r = tile / MT, mt = tile % MT;
-        f4_t s = red[0][tile][l];
-#pragma unroll
-        for (int w = 1; w < W; w++) s += red[w][tile][l];
-        const int m = 16 * mt + (l & 15);
-        const int n = row0 + 16 * r + 4 * (l >> 4);
-        if (m < M && n < N) {   // N % 4 == 0, so the four rows are in range together
-            h4_t o;
-#pragma unroll
-            for (int i = 0; i < 4; i++) o[i] = (half_t)(s[i] * scale);
-            *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
-        }
-    }
 }
 
 // ------------------------------------------------------------------ streaming matrix-vector path
@@ -728,6 +530,176 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
     DMM_TRACE_DUMP();
 }
 
+// ------------------------------------------------------------------ small-batch matrix-vector path
+// M <= 32 when x does not fit in LDS beside the tables (M * K too large).  Same tables, same
+// decode, same persistent workgroups and split-K as the streaming kernel; the difference is
+// where B comes from: x is read from global memory (L2) into registers, one 256-wide step at
+// a time.  Because vector-memory results return in order, x and codes of a step travel as ONE
+// prefetch unit (x first, then the codes), D units deep: an x load never waits behind codes
+// that are needed later than it is.  All loads are raw buffer loads whose offset is out of
+// range past the end (zeros, no memory access), so no branch surrounds them and the wait
+// counters stay exact.  MT = number of 16-row tiles of x (M <= 16 * MT).
+template <int R, int MT>
+__device__ __forceinline__ void regx_step(const u4_t (&cw)[R], const u4_t (&xb)[MT][8], uint32_t lane_base,
+                                          uint32_t quarter_bits, f4_t (&acc)[R][MT][2])
+{
+    constexpr int kItems = 4 * R;
+    StreamGather buf[2];
+    stream_gather(buf[0], cw[0][0], lane_base, quarter_bits);
+#pragma unroll
+    for (int i = 0; i < kItems; i++) {
+        const int t2 = i / R, r = i % R;
+        if (i + 1 < kItems) stream_gather(buf[(i + 1) & 1], cw[(i + 1) % R][(i + 1) / R], lane_base, quarter_bits);
+        const StreamGather &b = buf[i & 1];
+        const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+            acc[r][mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[mt][2 * t2]), acc[r][mt][0], 0, 0, 0);
+        const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+            acc[r][mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[mt][2 * t2 + 1]), acc[r][mt][1], 0, 0, 0);
+    }
+}
+
+template <int R, int W, int MT, int D>
+__global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__restrict__ x,
+                                                           const uint16_t *__restrict__ codes,
+                                                           const void *__restrict__ grid, float scale,
+                                                           uint16_t *__restrict__ y, int M, int N, int K,
+                                                           int n_blocks)
+{
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
+    typedef f4_t red_t[W][R * MT][kWave];
+    red_t *red = reinterpret_cast<red_t *>(smem_raw + kSTablesBytes);   // red[parity]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c16 = lane & 15;
+    const int q = lane >> 4;
+    const int n_steps = K >> 8;
+    const int row_bytes = K >> 2;
+    const uint32_t lane_base = (uint32_t)c16 * 16u;
+    const uint32_t quarter_bits = 0x34003400u;
+
+    const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid & 255];
+
+    const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;
+    const int nb_wg = ((int)blockIdx.x < n_blocks)
+                          ? (n_blocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, M * K * 2, 0x00020000);
+    constexpr int kOut = (int)0x80000000;
+    int voff[R], xoff[MT];
+#pragma unroll
+    for (int r = 0; r < R; r++) voff[r] = (16 * r + c16) * row_bytes + q * 16;
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const int m = 16 * mt + c16;
+        xoff[mt] = m < M ? (m * K + 64 * q) * 2 : kOut;   // columns past M: zeros, no memory access
+    }
+
+    struct Unit {
+        u4_t cw[R];
+        u4_t xb[MT][8];
+    };
+    int pf_blk = 0, pf_j = 0;
+    auto issue = [&](Unit &u) {
+        const bool ok = pf_blk < nb_wg && n_sw > 0;
+        const int step = wave + pf_j * W;
+        const int xs_off = ok ? step * 512 : kOut;
+        const int soff = ok ? ((int)blockIdx.x + pf_blk * (int)gridDim.x) * (16 * R) * row_bytes + step * 64 : kOut;
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                u.xb[mt][t] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff[mt] + t * 16, xs_off, 0);
+#pragma unroll
+        for (int r = 0; r < R; r++) u.cw[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], soff, 0);
+        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
+    };
+
+    Unit ring[D];
+#pragma unroll
+    for (int d = 0; d < D; d++) issue(ring[d]);
+
+    // tables (sign rows need no load; grid rows from the fetch above)
+    {
+        constexpr int kPerRow = 64 * W / 128, kCopies = 16 / kPerRow;
+        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw);
+        const int srow = tid / kPerRow, sc0 = (tid % kPerRow) * kCopies;
+        const u4_t sv = sign_row((uint32_t)srow);
+#pragma unroll
+        for (int i = 0; i < kCopies; i++) sg[srow * 16 + sc0 + i] = sv;
+        constexpr int kCopiesPer = 4096 / (64 * W);
+        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes);
+        const int row = tid & 255, c0 = (tid >> 8) * kCopiesPer;
+#pragma unroll
+        for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + c0 + i] = grow;
+    }
+    __syncthreads();
+
+    f4_t acc[R][MT][2];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[r][mt][0] = acc[r][mt][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+
+    // end of a row block: partial sums to LDS (double-buffered per block), one barrier, then
+    // the first R * MT waves add up one (row tile, m tile) each and store it
+    auto finish_block = [&](int blk) {
+        const int par = blk & 1;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                red[par][wave][r * MT + mt][lane] = acc[r][mt][0] + acc[r][mt][1];
+                acc[r][mt][0] = acc[r][mt][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+            }
+        __syncthreads();
+        for (int tile = wave; tile < R * MT; tile += W) {
+            f4_t sacc = red[par][0][tile][lane];
+#pragma unroll
+            for (int w = 1; w < W; w++) sacc += red[par][w][tile][lane];
+            const int r = tile / MT, mt = tile % MT;
+            const int m = 16 * mt + c16;
+            const int n = ((int)blockIdx.x + blk * (int)gridDim.x) * (16 * R) + 16 * r + 4 * q;
+            if (m < M && n < N) {   // N % 4 == 0, so the four rows are in range together
+                h4_t o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = (half_t)(sacc[e] * scale);
+                *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
+            }
+        }
+    };
+
+    if (n_sw == 0) {
+        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
+        return;
+    }
+    const int n_items = nb_wg * n_sw;
+    int blk = 0, j = 0;
+    for (int i0 = 0; i0 < n_items; i0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (i0 + d < n_items) {
+                regx_step<R, MT>(ring[d].cw, ring[d].xb, lane_base, quarter_bits, acc);
+                if (++j >= n_sw) {
+                    j = 0;
+                    finish_block(blk);
+                    blk++;
+                }
+            }
+            issue(ring[d]);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ matrix-matrix path
 // Block tile BN (n) x BM (m) x 64 (k) with WN x WM waves, each wave TN x TM tiles of
 // v_mfma_f32_32x32x16_f16 (A = decoded W rows, B = x rows, fp32 accumulate).  A wide n keeps
@@ -987,7 +959,8 @@ int check_common(const void *x, const void *codes, const void *grid, const void 
 bool gemv_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
              int64_t K)
 {
-    return M >= 1 && M <= 32 && K >= 256 && (K & 255) == 0 && K <= (1 << 23) && (N & 3) == 0 && aligned(x, 16) &&
+    return M >= 1 && M <= 32 && K >= 256 && (K & 255) == 0 && K <= (1 << 23) && N * (K >> 2) < (1LL << 31) &&
+           (N & 3) == 0 && aligned(x, 16) &&
            aligned(codes, 16) && aligned(grid, 16) && aligned(y, 8);
 }
 
@@ -998,27 +971,8 @@ bool gemm_ok(const void *x, const void *codes, const void *grid, const void *, i
            aligned(grid, 16) && M <= 65535LL * 128;
 }
 
-template <int R, int W, int MT>
-int launch_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                int64_t N, int64_t K, hipStream_t stream)
-{
-    const size_t shmem = kGemvTableBytes;
-    static bool attr_done = false;   // benign race: every thread sets the same value
-    if (!attr_done && shmem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_kernel<R, W, MT>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        if (e != hipSuccess) return (int)e;
-        attr_done = true;
-    }
-    const int64_t blocks = (N + 16 * R - 1) / (16 * R);
-    return launch(gemv_kernel<R, W, MT>, dim3((unsigned)blocks), dim3(64 * W), shmem, stream,
-                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N,
-                  (int)K);
-}
-
-// Tuning override for experiments: DMM_GEMV_CFG="R,W,D" picks the streaming kernel instance
-// (rows per block = 16 R, W waves, D prefetched steps per wave), "R,W" the non-streaming one;
-// unset or unknown -> the default choice.
+// Tuning override for experiments: DMM_GEMV_CFG="R,W,D" picks the kernel instance (rows per
+// block = 16 R, W waves, D prefetched steps per wave); unset or unknown -> the default choice.
 int gemv_cfg_override()
 {
     static int cfg = -1;
@@ -1078,10 +1032,29 @@ bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
            N * (K >> 2) < (1LL << 31);
 }
 
+template <int R, int W, int MT, int D>
+int launch_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                     int64_t N, int64_t K, hipStream_t stream)
+{
+    const size_t shmem = (size_t)kSTablesBytes + 2 * W * R * MT * kWave * 16;
+    static bool attr_done = false;   // benign race: every thread sets the same value
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_regx_kernel<R, W, MT, D>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const int64_t n_blocks = (N + 16 * R - 1) / (16 * R);
+    const int64_t wgs = n_blocks < cu_count() ? n_blocks : cu_count();
+    return launch(gemv_regx_kernel<R, W, MT, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  (int)n_blocks);
+}
+
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
-    if (M > 16) return launch_gemv<2, 8, 2>(x, codes, grid, scale, y, M, N, K, stream);
+    if (M > 16) return launch_gemv_regx<2, 8, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);
 #define DMM_STREAM_CASE(R, W, D)                                                                   \
     case R * 10000 + W * 100 + D:                                                                  \
         if (gemv_stream_ok<R, W>(M, N, K))                                                         \
@@ -1097,14 +1070,13 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
         DMM_STREAM_CASE(2, 16, 2)
         DMM_STREAM_CASE(2, 16, 3)
         DMM_STREAM_CASE(2, 16, 4)
-        case 10800: return launch_gemv<1, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
-        case 20800: return launch_gemv<2, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
-        case 40800: return launch_gemv<4, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
+        case 20803: return launch_gemv_regx<2, 8, 1, 3>(x, codes, grid, scale, y, M, N, K, stream);
+        case 20802: return launch_gemv_regx<2, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
         default: break;
     }
 #undef DMM_STREAM_CASE
     if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2>(x, codes, grid, scale, y, M, N, K, stream);
-    return launch_gemv<2, 8, 1>(x, codes, grid, scale, y, M, N, K, stream);
+    return launch_gemv_regx<2, 8, 1, 3>(x, codes, grid, scale, y, M, N, K, stream);
 }
 
 template <int WN, int WM, int TN, int TM>
