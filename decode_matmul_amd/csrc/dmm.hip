@@ -388,7 +388,7 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: offsets derived from it live in SGPRs
     const int c16 = lane & 15;
     const int q = lane >> 4;
     const int n_steps = K >> 8;
