@@ -39,6 +39,7 @@ from .codebook import (  # noqa: E402,F401
 __all__ = [
     "decode_matmul",
     "decode_matmul_path",
+    "decode_matmul_int8",
     "decode",
     "lib",
     "build_codebook_abs",
@@ -59,6 +60,13 @@ def decode_matmul_path(x, codes, grid, scale, path="auto"):
     """decode_matmul through one named kernel path: "auto", "gemv", "gemm" or "generic".
     A path asked for outside its domain raises instead of falling back."""
     return _C.decode_matmul_path(x, codes, grid, float(scale), path)
+
+
+def decode_matmul_int8(x, weights_compressed, codebook_abs, tiled=True):
+    """The reference's operator with its own dtypes: int8 x [M,K], int16 codes [N,K/8], int64[256]
+    table -> int32 [M,N] (decode_matmul_cuda.cu:178-234).  tiled=True: codes as the reference's
+    kernel reads them (`transpose_tile`, test_decode_matmul.py:101-109); False: row-major."""
+    return _C.decode_matmul_int8(x, weights_compressed, codebook_abs, bool(tiled))
 
 
 def decode(codes, grid):

@@ -19,6 +19,7 @@ SYMBOLS = {
     "dmm_gemv_f16": (ctypes.c_int, _OP),
     "dmm_gemm_f16": (ctypes.c_int, _OP),
     "dmm_generic_f16": (ctypes.c_int, _OP),
+    "dmm_decode_matmul_i8": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, ctypes.c_int, _P]),
     "dmm_set_kernel_events": (ctypes.c_int, [_P, _P]),
 }
 

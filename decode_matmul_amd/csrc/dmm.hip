@@ -928,6 +928,80 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_kernel(const uint16_t *__re
         }
 }
 
+// ------------------------------------------------------------------ the reference's integer operator
+// out[m,n] = sum_k x[m,k] * W[n,k] in int32, W decoded to int8 from the packed int64 table
+// exactly as /root/reference/test_decode_matmul.py:29-55 (value = +-byte, then +1 or -1, kept
+// in int8).  Codes may be in the layout the reference's kernel reads
+// (/root/reference/test_decode_matmul.py:101-109: 16-row x 4-column tiles of 64 codes ordered
+// [row % 8][column % 4][row / 8]) or plain row-major.  One wave per output row, integer
+// arithmetic throughout, so the result is exact for any K (the sum wraps in int32 like the
+// reference's accumulator).  A correctness path, not a tuned one.
+__device__ __forceinline__ int64_t tiled_code_index(int64_t n, int64_t j, int64_t kc)
+{
+    return ((n >> 4) * (kc >> 2) + (j >> 2)) * 64 + (n & 7) * 8 + (j & 3) * 2 + ((n >> 3) & 1);
+}
+
+__device__ __forceinline__ int wave_sum_i32(int v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+                                                   const int64_t *__restrict__ codebook_abs,
+                                                   int32_t *__restrict__ out, int64_t M, int64_t N, int64_t K,
+                                                   int tiled)
+{
+    __shared__ uint64_t table[256];
+    table[threadIdx.x] = (uint64_t)codebook_abs[threadIdx.x];
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t kc = K >> 3;
+    constexpr int kMC = 4;
+    for (int64_t n = (int64_t)blockIdx.x * 4 + wave; n < N; n += (int64_t)gridDim.x * 4) {
+        for (int64_t m0 = 0; m0 < M; m0 += kMC) {
+            int acc[kMC] = {};
+            for (int64_t j = lane; j < kc; j += kWave) {
+                const uint32_t c = codes[tiled ? tiled_code_index(n, j, kc) : n * kc + j];
+                uint64_t abs = table[c & 0xFFu];
+                uint32_t s8 = (c >> 8) & 0x7Fu;
+                s8 |= (__builtin_popcount(s8) & 1u) << 7;
+                const int shift = (c >> 15) & 1;
+                int w[8];
+#pragma unroll
+                for (int d = 0; d < 8; d++) {
+                    int8_t v = (int8_t)(abs & 0xFFu);
+                    if ((s8 >> d) & 1u) v = (int8_t)(-v);
+                    v = (int8_t)(shift ? v - 1 : v + 1);
+                    w[d] = v;
+                    abs >>= 8;
+                }
+#pragma unroll
+                for (int mm = 0; mm < kMC; mm++) {
+                    if (m0 + mm < M) {
+                        const int8_t *xr = x + (m0 + mm) * K + j * 8;
+#pragma unroll
+                        for (int d = 0; d < 8; d++) acc[mm] += (int)xr[d] * w[d];
+                    }
+                }
+            }
+#pragma unroll
+            for (int mm = 0; mm < kMC; mm++) {
+                const int sum = wave_sum_i32(acc[mm]);
+                if (lane == 0 && m0 + mm < M) out[(m0 + mm) * N + n] = sum;
+            }
+        }
+    }
+}
+
+__global__ void zero_i32_kernel(int32_t *y, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        y[i] = 0;
+}
+
 // ------------------------------------------------------------------ host side
 thread_local hipEvent_t tls_start = nullptr;
 thread_local hipEvent_t tls_stop = nullptr;
@@ -1220,6 +1294,26 @@ int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale
     if (st != DMM_OK || M == 0 || N == 0) return st;
     if (!gemm_ok(x, codes, grid, y, M, N, K)) return DMM_ERR_UNSUPPORTED;
     return run_gemm(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
+}
+
+int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_abs, void *out, int64_t M,
+                         int64_t N, int64_t K, int tiled, void *stream)
+{
+    if (M < 0 || N < 0 || K < 0 || (K & 7)) return DMM_ERR_BAD_SHAPE;
+    if (tiled && ((N & 15) || (K & 31))) return DMM_ERR_BAD_SHAPE;   // the tile is 16 rows x 4 codes
+    if (M == 0 || N == 0) return DMM_OK;
+    if (!out || !codebook_abs) return DMM_ERR_NULL_POINTER;
+    if (K > 0 && (!x || !codes)) return DMM_ERR_NULL_POINTER;
+    if (!aligned(codes, 2) || !aligned(codebook_abs, 8) || !aligned(out, 4)) return DMM_ERR_MISALIGNED;
+    if (K == 0) {
+        const int64_t n = M * N;
+        const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+        return launch(zero_i32_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (int32_t *)out, n);
+    }
+    int64_t blocks = (N + 3) / 4;
+    if (blocks > 65535 * 16) blocks = 65535 * 16;
+    return launch(int8_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const int8_t *)x,
+                  (const uint16_t *)codes, (const int64_t *)codebook_abs, (int32_t *)out, M, N, K, tiled ? 1 : 0);
 }
 
 int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, float scale, void *y,

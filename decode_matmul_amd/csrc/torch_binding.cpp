@@ -117,6 +117,36 @@ torch::Tensor decode(torch::Tensor codes, torch::Tensor grid)
     return W;
 }
 
+// The reference's own signature: int8 x, int16 codes (tiled like its kernel reads them, or
+// row-major), int64[256] table -> int32 (decode_matmul_cuda.cu:178-234).
+torch::Tensor decode_matmul_int8(torch::Tensor x, torch::Tensor weights_compressed, torch::Tensor codebook_abs,
+                                 bool tiled)
+{
+    DMM_CHECK_INPUT(x);
+    DMM_CHECK_INPUT(weights_compressed);
+    DMM_CHECK_INPUT(codebook_abs);
+    TORCH_CHECK(x.scalar_type() == torch::kInt8, "x must be int8");
+    TORCH_CHECK(is_code_dtype(weights_compressed), "weights_compressed must be int16 or uint16");
+    TORCH_CHECK(codebook_abs.scalar_type() == torch::kInt64 && codebook_abs.numel() == 256,
+                "codebook_abs must be int64[256]");
+    TORCH_CHECK(x.dim() == 2 && weights_compressed.dim() == 2, "x must be [M, K], weights_compressed [N, K/8]");
+    TORCH_CHECK(x.size(-1) == weights_compressed.size(-1) << 3, "x.size(-1) must be 8 * weights_compressed.size(-1)");
+    TORCH_CHECK(x.device() == weights_compressed.device() && x.device() == codebook_abs.device(),
+                "all tensors must be on the same device");
+    const int64_t M = x.size(-2), N = weights_compressed.size(-2), K = x.size(-1);
+    c10::DeviceGuard guard(x.device());
+    torch::Tensor out = torch::empty({M, N}, x.options().dtype(torch::kInt32).requires_grad(false));
+    hipStream_t stream = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+    int st;
+    {
+        pybind11::gil_scoped_release nogil;
+        st = dmm_decode_matmul_i8(x.data_ptr(), weights_compressed.data_ptr(), codebook_abs.data_ptr(),
+                                  out.data_ptr(), M, N, K, tiled ? 1 : 0, stream);
+    }
+    check_status(st, "decode_matmul_int8");
+    return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
@@ -126,6 +156,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("decode_matmul_path", &decode_matmul_path, "decode_matmul through one named kernel path",
           pybind11::arg("x"), pybind11::arg("codes"), pybind11::arg("grid"), pybind11::arg("scale"),
           pybind11::arg("path"));
+    m.def("decode_matmul_int8", &decode_matmul_int8,
+          "The reference's integer operator: int8 x, int16 codes, int64[256] table -> int32",
+          pybind11::arg("x"), pybind11::arg("weights_compressed"), pybind11::arg("codebook_abs"),
+          pybind11::arg("tiled") = true);
     m.def("decode", &decode, "Decode codes [N, K/8] to the dense half matrix [N, K]",
           pybind11::arg("codes"), pybind11::arg("grid"));
 }

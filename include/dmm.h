@@ -79,6 +79,20 @@ int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale
 int dmm_generic_f16(const void *x, const void *codes, const void *grid, float scale,
                     void *y, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* The reference's operator itself, in integers:
+ *   out int32 [M,N] = x int8 [M,K]  @  decode(codes, codebook_abs) int8 [N,K] ^T
+ * Replaces `decode_matmul(x, weights_compressed, codebook_abs)` of
+ * /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:178-234 with its dtypes (int8, int16,
+ * int64 -> int32).  codebook_abs is the packed table of
+ * /root/reference/test_decode_matmul.py:74-86 (byte d of entry i = dim d, as int8).  tiled != 0:
+ * codes are in the layout the reference's kernel reads, `transpose_tile` of
+ * /root/reference/test_decode_matmul.py:101-109 (needs N % 16 == 0 and K % 32 == 0, as
+ * decode_matmul_cuda.cu:196-197 does); tiled == 0: plain row-major [N, K/8].  None of the
+ * reference's other shape demands (M % 8, K % 2048, K >= 4096) apply.  Exact integer
+ * arithmetic; `out` is fully overwritten.  A correctness path (one wave per output row). */
+int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_abs, void *out,
+                         int64_t M, int64_t N, int64_t K, int tiled, void *stream);
+
 /* Kernel timing hook for benchmarks.  While a (start, stop) pair of hipEvent_t handles is
  * set on the calling thread, the dominant kernel of each operator call records `start`
  * immediately before and `stop` immediately after itself on the GPU timeline, so

@@ -169,6 +169,70 @@ def test_reference_shape_golden_case():
         assert np.array_equal(bits(y), bits((yi.astype(np.float64) / 4 * 2.0 ** -8).astype(np.float16))), path
 
 
+# ----------------------------------------------------------------- the integer operator itself
+def c_matmul_i8(x, codes, cb, tiled):
+    M, K = x.shape
+    N = codes.shape[0]
+    out = torch.full((M, N), -12345, dtype=torch.int32, device=x.device)
+    st = capi.lib().dmm_decode_matmul_i8(x.data_ptr(), codes.data_ptr(), cb.data_ptr(), out.data_ptr(), M, N, K,
+                                         int(tiled), torch.cuda.current_stream().cuda_stream)
+    capi.check("dmm_decode_matmul_i8", st)
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 16, 4096), (1, 16, 32), (3, 48, 96), (13, 160, 2048), (5, 32, 8192)])
+def test_integer_operator_tiled_is_exact(M, N, K):
+    """int8 x, int16 codes in the reference kernel's tile order, packed int64 table -> int32,
+    equal to the reference's checker (/root/reference/test_decode_matmul.py:58-71) restated by
+    the oracle, element for element."""
+    rng = np.random.default_rng(N * 7 + K)
+    cb = orc.build_codebook_abs()
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    want = orc.decode_matmul_i32(x, codes, cb)
+    out = c_matmul_i8(dev(x), dev(orc.transpose_tile(codes)), dev(cb), True)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+    # the torch operator with the reference's own argument list gives the same tensor
+    out2 = dmm.decode_matmul_int8(dev(x), dmm.transpose_tile(dev(codes)), dev(cb))
+    assert out2.dtype == torch.int32 and torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 8), (2, 3, 32), (7, 37, 1000), (4, 5, 24)])
+def test_integer_operator_row_major_any_shape(M, N, K):
+    rng = np.random.default_rng(N * 11 + K)
+    cb = rng.integers(-2 ** 63, 2 ** 63, size=256, dtype=np.int64)       # any table, not only E8P
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    want = orc.decode_matmul_i32(x, codes, cb)
+    out = c_matmul_i8(dev(x), dev(codes), dev(cb), False)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_integer_operator_golden_cases_and_edges():
+    case = np.load(os.path.join(GOLDEN_DIR, "int8_case.npz"))
+    x, codes, yi, cb = case["x"], case["codes"], case["y"], case["codebook_abs"]
+    out = c_matmul_i8(dev(x), dev(orc.transpose_tile(codes)), dev(cb), True)
+    assert np.array_equal(out.cpu().numpy(), yi)
+    g = json.load(open(os.path.join(GOLDEN_DIR, "golden.json")))["int8_case"]
+    xs = np.array(g["x"], dtype=np.int8).reshape(g["M"], g["K"])
+    cs = np.array(g["codes"], dtype=np.int16).reshape(g["N"], g["K"] // 8)
+    out = c_matmul_i8(dev(xs), dev(cs), dev(cb), False)
+    assert out.cpu().numpy().reshape(-1).tolist() == g["y"]
+    # extremes: every product at its largest magnitude (x = -128, table byte -128 flipped stays -128)
+    cbx = np.frombuffer(bytes([0x80] * 8 * 256), dtype=np.int64).copy()
+    xe = np.full((2, 64), -128, dtype=np.int8)
+    ce = np.array([[0x0000, 0x8000, 0x7F00, 0xFFFF, 0x0100, 0x8100, 0x00FF, 0x80FF]] * 16, dtype=np.uint16).view(np.int16)
+    out = c_matmul_i8(dev(xe), dev(ce), dev(cbx), False)
+    assert np.array_equal(out.cpu().numpy(), orc.decode_matmul_i32(xe, ce, cbx))
+    # K == 0 gives zeros; M == 0 or N == 0 is a no-op
+    z = torch.full((3, 16), 7, dtype=torch.int32, device=DEV)
+    st = capi.lib().dmm_decode_matmul_i8(None, None, dev(cb).data_ptr(), z.data_ptr(), 3, 16, 0, 1, None)
+    torch.cuda.synchronize()
+    assert st == 0 and torch.all(z == 0)
+
+
 # ----------------------------------------------------------------- full benchmark sizes
 FULL = [(1, N, K) for (K, N) in workload.LLAMA2_70B + workload.LLAMA2_7B] + \
        [(16, 11008, 4096), (32, 4096, 11008), (2048, 4096, 4096), (2048, 11008, 4096), (2048, 4096, 11008)]

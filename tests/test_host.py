@@ -64,6 +64,17 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert lib.dmm_decode_f16(None, None, None, 0, 64, None) == 0
     assert lib.dmm_decode_matmul_f16(None, None, None, 1.0, None, 0, 4, 16, None) == 0
     assert lib.dmm_decode_matmul_f16(None, None, None, 1.0, None, 3, 0, 16, None) == 0
+    # the integer operator: K % 8, the tile's N % 16 and K % 32 only when tiled, NULLs, alignment
+    i8 = lib.dmm_decode_matmul_i8
+    assert i8(p, p, p, p, 1, 16, 20, 0, None) == -2
+    assert i8(p, p, p, p, 1, 8, 32, 1, None) == -2
+    assert i8(p, p, p, p, 1, 16, 48, 1, None) == -2
+    assert i8(p, p, p, p, -1, 16, 32, 0, None) == -2
+    assert i8(None, p, p, p, 1, 16, 32, 1, None) == -1
+    assert i8(p, p, p, None, 1, 16, 32, 1, None) == -1
+    assert i8(p, odd, p, p, 1, 16, 32, 1, None) == -3
+    assert i8(p, p, ctypes.c_void_p(p.value + 4), p, 1, 16, 32, 1, None) == -3
+    assert i8(None, None, None, None, 0, 16, 32, 1, None) == 0
     # the timing hook wants both events or neither
     assert lib.dmm_set_kernel_events(p, None) == -1
     assert lib.dmm_set_kernel_events(None, None) == 0
