@@ -6,6 +6,7 @@ sit next to this module so they travel with the tree.
     python -m decode_matmul_amd.build --lib      # only libdmm.so
 """
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -49,10 +50,34 @@ def hipcc_path():
 
 def build_lib(verbose=False):
     """hipcc: csrc/dmm.hip -> libdmm.so (gfx950 code object + the extern "C" entry points)."""
-    cmd = [hipcc_path()] + HIPCC_FLAGS + ["-I" + INCLUDE, "-o", LIB_PATH, os.path.join(CSRC, "dmm.hip")]
+    cmd = [hipcc_path()] + HIPCC_FLAGS + ["-Rpass-analysis=kernel-resource-usage",
+                                          "-I" + INCLUDE, "-o", LIB_PATH, os.path.join(CSRC, "dmm.hip")]
     out = _run(cmd)
-    if verbose and out.strip():
-        print(out)
+    # No kernel may spill registers to scratch memory: the kernels are sized to their register
+    # budget, and a build of the streaming kernel that spilled ran at half speed and returned
+    # wrong sums on the GPU.  The compiler's resource remarks name the offender.
+    name, spilled = None, []
+    for line in out.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line:
+            if int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0]) != 0:
+                spilled.append(name)
+    if spilled:
+        os.remove(LIB_PATH)
+        raise RuntimeError("kernels spill registers to scratch memory: %s" % ", ".join(spilled))
+    rest, skip = [], 0
+    for line in out.splitlines():   # drop the remarks and the two source-context lines after each
+        if "-Rpass-analysis=kernel-resource-usage" in line:
+            skip = 2
+        elif skip and re.match(r"^\s*\d*\s*\|", line):
+            skip -= 1
+        else:
+            skip = 0
+            rest.append(line)
+    rest = "\n".join(rest)
+    if verbose and rest.strip():
+        print(rest)
     return LIB_PATH
 
 

@@ -336,12 +336,13 @@ __device__ __forceinline__ h8_t stream_finish(const u4_t &g, const u4_t &sg, uin
     return __builtin_bit_cast(h8_t, r);
 }
 
-// One 256-wide k step for R row tiles.  Items (word t2 of row tile r) run t2-major so that the
-// two B operands of a word pair are read from LDS once and used for all R tiles; the gathers
-// of item i+1 are issued before the math of item i.
+// One 256-wide k step for the first nv (uniform, 1 <= nv <= R) of R row tiles.  Items (word
+// t2 of row tile r) run t2-major so that the two B operands of a word pair are read from LDS
+// once and used for all tiles; the gathers of item i+1 are issued before the math of item i.
+// Tiles past nv are skipped by uniform branches around their gathers and their math.
 template <int R>
 __device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t lane_base,
-                                            uint32_t quarter_bits, f4_t (&acc)[R][2])
+                                            uint32_t quarter_bits, f4_t (&acc)[R][2], int nv)
 {
     constexpr int kItems = 4 * R;
     StreamGather buf[2];
@@ -357,18 +358,22 @@ __device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr,
             if (nr == 0) {
                 xb[nt2 & 1][0] = lds_read16(xaddr + nt2 * 32);
                 xb[nt2 & 1][1] = lds_read16(xaddr + nt2 * 32 + 16);
+                stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
+            } else if (nr < nv) {
+                stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
             }
-            stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
         }
-        // 4 packed FMAs, MFMA, 4 packed FMAs, MFMA: the second group and the next item's
-        // address math run in the shadow of the matrix unit
-        const StreamGather &b = buf[i & 1];
-        const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
-        acc[r][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[t2 & 1][0]), acc[r][0], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
-        acc[r][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[t2 & 1][1]), acc[r][1], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
+        if (r == 0 || r < nv) {
+            // 4 packed FMAs, MFMA, 4 packed FMAs, MFMA: the second group and the next item's
+            // address math run in the shadow of the matrix unit
+            const StreamGather &b = buf[i & 1];
+            const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
+            acc[r][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[t2 & 1][0]), acc[r][0], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
+            acc[r][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[t2 & 1][1]), acc[r][1], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 }
 
@@ -377,8 +382,9 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
                                                              const uint16_t *__restrict__ codes,
                                                              const void *__restrict__ grid, float scale,
                                                              uint16_t *__restrict__ y, int M, int N, int K,
-                                                             int n_blocks)
+                                                             int n_tiles)
 {
+    static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
     if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     DMM_TRACE_MARK(0);
@@ -411,8 +417,11 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
     }
 
     const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;   // k steps of this wave per row block
-    const int nb_wg = ((int)blockIdx.x < n_blocks)
-                          ? (n_blocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    // this workgroup's share of the 16-row tiles: a contiguous range, equal to within one tile
+    // over the grid, walked R tiles (one row block) at a time; the last block may be partial
+    const int t0 = (int)(((int64_t)n_tiles * (int)blockIdx.x) / (int)gridDim.x);
+    const int t1 = (int)(((int64_t)n_tiles * ((int)blockIdx.x + 1)) / (int)gridDim.x);
+    const int nb_wg = (t1 - t0 + R - 1) / R;
 
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
@@ -420,7 +429,7 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
     int voff[R];
 #pragma unroll
     for (int r = 0; r < R; r++) voff[r] = (16 * r + c16) * row_bytes + q * 16;
-    // ... and the scalar part: row block and k step of the next item to prefetch.  Rows past N
+    // ... and the scalar part: first tile and k step of the next item to prefetch.  Rows past N
     // land past the end of the buffer by themselves; items past the end get an offset no
     // buffer reaches.
     constexpr int kOut = (int)0x80000000;
@@ -432,10 +441,11 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 #else
         const bool ok2 = ok;
 #endif
-        const int soff = ok2 ? ((int)blockIdx.x + pf_blk * (int)gridDim.x) * (16 * R) * row_bytes + (wave + pf_j * W) * 64
-                             : kOut;
+        const int tb = t0 + pf_blk * R;
+        const int soff = ok2 ? tb * 16 * row_bytes + (wave + pf_j * W) * 64 : kOut;
 #pragma unroll
-        for (int r = 0; r < R; r++) cwd[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], soff, 0);
+        for (int r = 0; r < R; r++)   // tiles of a partial block that belong to the next workgroup: no access
+            cwd[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], (r == 0 || tb + r < t1) ? soff : kOut, 0);
         if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
     };
 
@@ -483,8 +493,9 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
             f4_t sacc = rp[(0 * R + wave) * 4 * M + q * M + c16];
 #pragma unroll
             for (int w = 1; w < W; w++) sacc += rp[(w * R + wave) * 4 * M + q * M + c16];
-            const int n = ((int)blockIdx.x + blk * (int)gridDim.x) * (16 * R) + 16 * wave + 4 * q;
-            if (n < N) {   // N % 4 == 0, so the four rows are in range together
+            const int tile = t0 + blk * R + wave;
+            const int n = tile * 16 + 4 * q;
+            if (tile < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
                 h4_t o;
 #pragma unroll
                 for (int e = 0; e < 4; e++) o[e] = (half_t)(sacc[e] * scale);
@@ -513,7 +524,11 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
                     for (int r = 0; r < R; r++) acc[r][0][0] += __builtin_bit_cast(float, cw[d][r][0] ^ cw[d][r][1] ^ cw[d][r][2] ^ cw[d][r][3]);
                 } else
 #endif
-                stream_step<R>(cw[d], xlane + (uint32_t)((wave + j * W) * 512), lane_base, quarter_bits, acc);
+                {
+                    const uint32_t xa = xlane + (uint32_t)((wave + j * W) * 512);
+                    const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
+                    stream_step<R>(cw[d], xa, lane_base, quarter_bits, acc, nv);
+                }
                 if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
                 if (++j >= n_sw) {
                     j = 0;
@@ -541,7 +556,7 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 // counters stay exact.  MT = number of 16-row tiles of x (M <= 16 * MT).
 template <int R, int MT>
 __device__ __forceinline__ void regx_step(const u4_t (&cw)[R], const u4_t (&xb)[MT][8], uint32_t lane_base,
-                                          uint32_t quarter_bits, f4_t (&acc)[R][MT][2])
+                                          uint32_t quarter_bits, f4_t (&acc)[R][MT][2], int nv)
 {
     constexpr int kItems = 4 * R;
     StreamGather buf[2];
@@ -549,16 +564,21 @@ __device__ __forceinline__ void regx_step(const u4_t (&cw)[R], const u4_t (&xb)[
 #pragma unroll
     for (int i = 0; i < kItems; i++) {
         const int t2 = i / R, r = i % R;
-        if (i + 1 < kItems) stream_gather(buf[(i + 1) & 1], cw[(i + 1) % R][(i + 1) / R], lane_base, quarter_bits);
-        const StreamGather &b = buf[i & 1];
-        const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
+        if (i + 1 < kItems) {
+            const int nt2 = (i + 1) / R, nr = (i + 1) % R;
+            if (nr == 0 || nr < nv) stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
+        }
+        if (r == 0 || r < nv) {   // tiles past nv (uniform) belong to the next workgroup
+            const StreamGather &b = buf[i & 1];
+            const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++)
-            acc[r][mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[mt][2 * t2]), acc[r][mt][0], 0, 0, 0);
-        const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
+            for (int mt = 0; mt < MT; mt++)
+                acc[r][mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[mt][2 * t2]), acc[r][mt][0], 0, 0, 0);
+            const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++)
-            acc[r][mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[mt][2 * t2 + 1]), acc[r][mt][1], 0, 0, 0);
+            for (int mt = 0; mt < MT; mt++)
+                acc[r][mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[mt][2 * t2 + 1]), acc[r][mt][1], 0, 0, 0);
+        }
     }
 }
 
@@ -567,8 +587,9 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
                                                            const uint16_t *__restrict__ codes,
                                                            const void *__restrict__ grid, float scale,
                                                            uint16_t *__restrict__ y, int M, int N, int K,
-                                                           int n_blocks)
+                                                           int n_tiles)
 {
+    static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
     if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     typedef f4_t red_t[W][R * MT][kWave];
@@ -587,8 +608,10 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
     const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid & 255];
 
     const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;
-    const int nb_wg = ((int)blockIdx.x < n_blocks)
-                          ? (n_blocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    // contiguous, balanced range of 16-row tiles per workgroup, as in the streaming kernel
+    const int t0 = (int)(((int64_t)n_tiles * (int)blockIdx.x) / (int)gridDim.x);
+    const int t1 = (int)(((int64_t)n_tiles * ((int)blockIdx.x + 1)) / (int)gridDim.x);
+    const int nb_wg = (t1 - t0 + R - 1) / R;
 
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
@@ -613,14 +636,16 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
         const bool ok = pf_blk < nb_wg && n_sw > 0;
         const int step = wave + pf_j * W;
         const int xs_off = ok ? step * 512 : kOut;
-        const int soff = ok ? ((int)blockIdx.x + pf_blk * (int)gridDim.x) * (16 * R) * row_bytes + step * 64 : kOut;
+        const int tb = t0 + pf_blk * R;
+        const int soff = ok ? tb * 16 * row_bytes + step * 64 : kOut;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int t = 0; t < 8; t++)
                 u.xb[mt][t] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff[mt] + t * 16, xs_off, 0);
 #pragma unroll
-        for (int r = 0; r < R; r++) u.cw[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], soff, 0);
+        for (int r = 0; r < R; r++)
+            u.cw[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], (r == 0 || tb + r < t1) ? soff : kOut, 0);
         if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
     };
 
@@ -668,8 +693,9 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
             for (int w = 1; w < W; w++) sacc += red[par][w][tile][lane];
             const int r = tile / MT, mt = tile % MT;
             const int m = 16 * mt + c16;
-            const int n = ((int)blockIdx.x + blk * (int)gridDim.x) * (16 * R) + 16 * r + 4 * q;
-            if (m < M && n < N) {   // N % 4 == 0, so the four rows are in range together
+            const int rt = t0 + blk * R + r;
+            const int n = rt * 16 + 4 * q;
+            if (m < M && rt < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
                 h4_t o;
 #pragma unroll
                 for (int e = 0; e < 4; e++) o[e] = (half_t)(sacc[e] * scale);
@@ -688,7 +714,7 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
 #pragma unroll
         for (int d = 0; d < D; d++) {
             if (i0 + d < n_items) {
-                regx_step<R, MT>(ring[d].cw, ring[d].xb, lane_base, quarter_bits, acc);
+                regx_step<R, MT>(ring[d].cw, ring[d].xb, lane_base, quarter_bits, acc, t1 - (t0 + blk * R));
                 if (++j >= n_sw) {
                     j = 0;
                     finish_block(blk);
@@ -1090,11 +1116,11 @@ int launch_gemv_stream(const void *x, const void *codes, const void *grid, float
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
-    const int64_t n_blocks = (N + 16 * R - 1) / (16 * R);
-    const int64_t wgs = n_blocks < cu_count() ? n_blocks : cu_count();
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     return launch(gemv_stream_kernel<R, W, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
-                  (int)n_blocks);
+                  (int)n_tiles);
 }
 
 // tables, partial sums and x fit in the 160 KB of LDS, and every byte offset of the code
@@ -1118,11 +1144,11 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
-    const int64_t n_blocks = (N + 16 * R - 1) / (16 * R);
-    const int64_t wgs = n_blocks < cu_count() ? n_blocks : cu_count();
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     return launch(gemv_regx_kernel<R, W, MT, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
-                  (int)n_blocks);
+                  (int)n_tiles);
 }
 
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
@@ -1135,15 +1161,10 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
             return launch_gemv_stream<R, W, D>(x, codes, grid, scale, y, M, N, K, stream);         \
         break;
     switch (gemv_cfg_override()) {
-        DMM_STREAM_CASE(1, 8, 4)
-        DMM_STREAM_CASE(1, 8, 8)
         DMM_STREAM_CASE(2, 8, 4)
-        DMM_STREAM_CASE(2, 8, 8)
         DMM_STREAM_CASE(1, 16, 4)
-        DMM_STREAM_CASE(1, 16, 6)
         DMM_STREAM_CASE(2, 16, 2)
         DMM_STREAM_CASE(2, 16, 3)
-        DMM_STREAM_CASE(2, 16, 4)
         case 20803: return launch_gemv_regx<2, 8, 1, 3>(x, codes, grid, scale, y, M, N, K, stream);
         case 20802: return launch_gemv_regx<2, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
         default: break;
@@ -1170,7 +1191,7 @@ int launch_gemm(const void *x, const void *codes, const void *grid, float scale,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
 }
 
-// Tuning override for experiments: DMM_GEMM_CFG=a|b|c|d picks the tile configuration.
+// Tuning override for experiments: DMM_GEMM_CFG=a|b|g picks the tile configuration.
 int run_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
@@ -1181,9 +1202,7 @@ int run_gemm(const void *x, const void *codes, const void *grid, float scale, vo
     }
     switch (cfg) {
         case 'b': return launch_gemm<2, 2, 4, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 256 x 128, 4 waves
-        case 'd': return launch_gemm<2, 4, 4, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 256 x 256, 8 waves
         case 'g': return launch_gemm<2, 2, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 128 x 128, 4 waves, 2 per CU
-        case 'h': return launch_gemm<2, 2, 4, 2>(x, codes, grid, scale, y, M, N, K, stream);
         default: break;
     }
     return launch_gemm<4, 2, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);                 // 256 x 128, 8 waves
