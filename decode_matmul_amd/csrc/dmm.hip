@@ -298,7 +298,7 @@ __device__ __forceinline__ void stream_stage_tables(unsigned char *smem, const u
     u4_t *gg = reinterpret_cast<u4_t *>(smem + kSSignBytes);
     const int row = tid & 255, c0 = (tid >> 8) * kCopiesPer;
 #pragma unroll
-    for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + c0 + i] = grow;
+    for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + ((c0 + i + tid) & 15)] = grow;   // 16 lanes, 16 bank groups
 #pragma unroll
     for (int i = 0; i < 2048 / kNThreads; i++) sg[tid + i * kNThreads] = sign_row((uint32_t)((tid + i * kNThreads) >> 4));
 }
@@ -660,12 +660,12 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
         const int srow = tid / kPerRow, sc0 = (tid % kPerRow) * kCopies;
         const u4_t sv = sign_row((uint32_t)srow);
 #pragma unroll
-        for (int i = 0; i < kCopies; i++) sg[srow * 16 + sc0 + i] = sv;
+        for (int i = 0; i < kCopies; i++) sg[srow * 16 + ((sc0 + i + srow) & 15)] = sv;   // 16 lanes, 16 bank groups
         constexpr int kCopiesPer = 4096 / (64 * W);
         u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes);
         const int row = tid & 255, c0 = (tid >> 8) * kCopiesPer;
 #pragma unroll
-        for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + c0 + i] = grow;
+        for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + ((c0 + i + tid) & 15)] = grow;   // 16 lanes, 16 bank groups
     }
     __syncthreads();
 
