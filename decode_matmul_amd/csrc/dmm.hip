@@ -303,6 +303,20 @@ __device__ __forceinline__ void stream_stage_tables(unsigned char *smem, const u
     for (int i = 0; i < 2048 / kNThreads; i++) sg[tid + i * kNThreads] = sign_row((uint32_t)((tid + i * kNThreads) >> 4));
 }
 
+// Sum over each row of 16 lanes, result in lane 15 of the row (all 64 lanes must be active).
+template <int kCtrl>
+__device__ __forceinline__ float dpp_shr_add(float v)
+{
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float row_sum16(float v)
+{
+    v = dpp_shr_add<0x118>(v);   // row_shr:8, lanes shifted in from outside the row read 0
+    v = dpp_shr_add<0x114>(v);   // row_shr:4
+    v = dpp_shr_add<0x112>(v);   // row_shr:2
+    return dpp_shr_add<0x111>(v);   // row_shr:1
+}
+
 // (a & m) | (b & ~m) in one instruction
 __device__ __forceinline__ uint32_t bfi(uint32_t m, uint32_t a, uint32_t b)
 {
@@ -478,8 +492,8 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
 
-    // publish this wave's partial sums of a finished row block, meet the other waves, and
-    // let wave r (< R) add up and store row tile r
+    // publish this wave's partial sums of a finished row block, meet the other waves, add up
+    // and store
     auto finish_block = [&](int blk) {
         f4_t *rp = red + (blk & 1) * red_par;
         if (c16 < M) {
@@ -489,17 +503,22 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
         __syncthreads();
-        if (wave < R && c16 < M) {
-            f4_t sacc = rp[(0 * R + wave) * 4 * M + q * M + c16];
+        // (row tile r, x row m) pairs go round the waves; lane (w = lane % 16, quarter lane / 16)
+        // fetches ONE partial sum, wave w's, and the 16 of a row of lanes are added with DPP
+        // shifts: a single LDS round trip instead of a chain of W dependent ones
+        for (int p = wave; p < R * M; p += W) {
+            const int r = M == 1 ? p : p / M, m = p - r * M;
+            f4_t v = f4_t{0.f, 0.f, 0.f, 0.f};
+            if (c16 < W) v = rp[(c16 * R + r) * 4 * M + q * M + m];
 #pragma unroll
-            for (int w = 1; w < W; w++) sacc += rp[(w * R + wave) * 4 * M + q * M + c16];
-            const int tile = t0 + blk * R + wave;
+            for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
+            const int tile = t0 + blk * R + r;
             const int n = tile * 16 + 4 * q;
-            if (tile < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
+            if (c16 == 15 && tile < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
                 h4_t o;
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (half_t)(sacc[e] * scale);
-                *reinterpret_cast<h4_t *>(y + (int64_t)c16 * N + n) = o;
+                for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
+                *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
             }
         }
     };
