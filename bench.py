@@ -36,6 +36,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="skip prefill / small-batch / CPU legs")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the M = 2048 leg and print its object (for profiling the matrix-matrix kernel)")
     ap.add_argument("--rotate-mb", type=int, default=400, help="distinct code bytes to rotate through, at least")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch 8 plain device copies of 256 MiB first (a known-size reference for scaling "
@@ -83,6 +85,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes)}))
+        return
 
     # ---------------------------------------------------------------- headline: 70B GEMV
     shapes = workload.LLAMA2_70B

@@ -973,6 +973,219 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_kernel(const uint16_t *__re
         }
 }
 
+// ------------------------------------------------------------------ matrix-matrix path, weights in registers
+// Block tile 256 (n) x 128 (m) x 64 (k), four waves, each wave 64 rows of W (two 32-row tiles)
+// against all 128 rows of x (four 32-row tiles): 8 accumulators of v_mfma_f32_32x32x16_f16.
+//
+// The LDS is the scarce resource of the staged kernel above (table gathers with bank
+// conflicts, W tile written and read back, operand fragments read by every wave).  Here
+//   * a wave decodes ITS 64 rows straight into A-operand registers - a lane's 8 bytes of a
+//     row are the 4 codes it feeds to the 4 MFMA k steps of the tile, any k order works as
+//     long as A and B agree - so W never touches the LDS and no decode is done twice;
+//   * the tables are the conflict-free 16-copy ones of the matrix-vector kernels (256-byte
+//     row pitch, lane reads copy lane % 16, address = one v_perm_b32);
+//   * only x goes through the LDS (coalesced global loads, rows 144 bytes apart, double
+//     buffered, one barrier per k tile), read as B fragments once per wave and k step.
+// Per k tile and wave: 32 MFMAs (1024 matrix-unit clocks) against 36 LDS instructions and
+// about 64 VALU operations, so the matrix unit is the bound.  Tile kt+1 is decoded and its x
+// written while the MFMAs of tile kt run; global loads are four tiles ahead.
+// w = g * s + d, d = low (kHi false) or high half of dd for both lanes, as plain vector code:
+// the compiler folds the broadcast into the op_sel bits and its scheduler sees a VALU
+// instruction (it cannot classify inline assembly)
+template <bool kHi>
+__device__ __forceinline__ h8_t gemm_finish(const u4_t &g, const u4_t &sg, uint32_t dd)
+{
+    const h2_t dv = as_h2(dd);
+    const h2_t d = kHi ? h2_t{dv[1], dv[1]} : h2_t{dv[0], dv[0]};
+    u4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = as_u32(__builtin_elementwise_fma(as_h2(g[i]), as_h2(sg[i]), d));
+    return __builtin_bit_cast(h8_t, r);
+}
+
+constexpr int kGrBN = 256, kGrBM = 128, kGrBK = 64, kGrLd = kGrBK + 8;
+constexpr int kGrTN = 2, kGrTM = 4;
+constexpr int kGrSmemBytes = kSTablesBytes + 2 * kGrBM * kGrLd * 2;
+
+__global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restrict__ x,
+                                                       const uint16_t *__restrict__ codes,
+                                                       const void *__restrict__ grid, float scale,
+                                                       uint16_t *__restrict__ y, int M, int N, int K)
+{
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, kq = lane >> 5;
+    const uint32_t lane_base = (uint32_t)(lane & 15) * 16u;
+    const uint32_t quarter_bits = 0x34003400u;
+    const int n0 = blockIdx.x * kGrBN;
+    const int m0 = blockIdx.y * kGrBM;
+    const int k_tiles = K / kGrBK;
+    const int row_bytes = K >> 2;
+    constexpr int kOut = (int)0x80000000;
+
+    // tables: thread tid owns grid row tid (16 copies) and 8 of the 2048 sign slots
+    {
+        const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid];
+        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes);
+        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw);
+#pragma unroll
+        for (int i = 0; i < 8; i++) sg[tid + i * 256] = sign_row((uint32_t)((tid + i * 256) >> 4));
+#pragma unroll
+        for (int i = 0; i < 16; i++) gg[tid * 16 + ((i + tid) & 15)] = grow;   // 16 lanes, 16 bank groups
+    }
+
+    // global sources.  Codes: lane (row l32 of tile i, half kq) reads 8 bytes = codes 4 kq .. 4 kq + 3
+    // of the k tile.  x: thread (row tid / 2, half tid % 2) reads 64 bytes.  Both as raw buffer
+    // loads: rows past N / M and tiles past K get zeros without a memory access.
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, (int)((int64_t)M * K * 2), 0x00020000);
+    int cvoff[kGrTN];
+#pragma unroll
+    for (int i = 0; i < kGrTN; i++) {
+        const int n = n0 + wave * 64 + i * 32 + l32;
+        cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
+    }
+    const int x_row = tid >> 1, x_half = tid & 1;
+    const int xvoff = m0 + x_row < M ? ((m0 + x_row) * K + x_half * 32) * 2 : kOut;
+
+    struct Stage {
+        u2_t cw[kGrTN];
+        u4_t xv[4];
+    };
+    auto load_tile = [&](Stage &st, int kt) {
+        const int coff = kt < k_tiles ? kt * 16 : kOut;
+        const int xoff = kt < k_tiles ? kt * 128 : kOut;
+#pragma unroll
+        for (int i = 0; i < kGrTN; i++) st.cw[i] = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
+#pragma unroll
+        for (int p = 0; p < 4; p++) st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff + p * 16, xoff, 0);
+    };
+    unsigned char *xs = smem_raw + kSTablesBytes;                       // [2][kGrBM][kGrLd] halves
+    const uint32_t xs_w = lds_addr(xs) + (uint32_t)(x_row * kGrLd + x_half * 32) * 2u;       // this thread's write slot
+    const uint32_t xs_r = lds_addr(xs) + (uint32_t)(l32 * kGrLd + kq * 32) * 2u;             // this lane's B fragments
+    constexpr uint32_t kXBuf = kGrBM * kGrLd * 2;
+
+    Stage ring[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) load_tile(ring[i], i);
+
+    f16_t acc[kGrTN][kGrTM];
+#pragma unroll
+    for (int i = 0; i < kGrTN; i++)
+#pragma unroll
+        for (int j = 0; j < kGrTM; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    // A fragments of one k tile: [tile i][k step s], a decoded code each
+    u4_t afr[2][kGrTN][4];
+    auto x_store = [&](const Stage &st, int buf, int p) {
+        *reinterpret_cast<u4_t *>(xs + (xs_w - lds_addr(xs)) + buf * kXBuf + p * 16) = st.xv[p];
+    };
+    // The decode runs as a stream of units, one per k step: unit u of a tile is word u / 2 of
+    // row tile u % 2 (two codes = two k steps of that row tile).  A step gathers the table
+    // rows of its unit and finishes (packed FMAs) the unit gathered one step earlier, so no
+    // step waits for its own gathers.
+    StreamGather g[2];
+    auto unit_gather = [&](StreamGather &o, const Stage &st, int u) {
+        stream_gather(o, st.cw[u & 1][u >> 1], lane_base, quarter_bits);
+    };
+    auto unit_finish = [&](const StreamGather &o, int abuf, int u) {
+        afr[abuf][u & 1][2 * (u >> 1)] = __builtin_bit_cast(u4_t, gemm_finish<false>(o.g0, o.s0, o.dd));
+        afr[abuf][u & 1][2 * (u >> 1) + 1] = __builtin_bit_cast(u4_t, gemm_finish<true>(o.g1, o.s1, o.dd));
+    };
+
+    __syncthreads();   // tables ready
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        unit_gather(g[u & 1], ring[0], u);
+        if (u < 3) unit_finish(g[u & 1], 0, u);   // unit 3 is finished by the first step of the loop
+    }
+#pragma unroll
+    for (int p = 0; p < 4; p++) x_store(ring[0], 0, p);
+    __syncthreads();   // x tile 0 staged
+
+    auto read_b = [&](u4_t (&b)[kGrTM], int buf, int s) {
+#pragma unroll
+        for (int j = 0; j < kGrTM; j++) b[j] = lds_read16(xs_r + buf * kXBuf + (uint32_t)(j * 32 * kGrLd * 2 + s * 16));
+    };
+    // MFMAs of tile kt (A = afr[buf], B from x buffer buf) while tile kt+1 (registers sn) is
+    // decoded into afr[buf ^ 1] and its x written to buffer buf ^ 1, and tile kt+4 is fetched
+    // into sf.  Past the last tile sn holds zeros (out-of-range loads): decoding and storing
+    // them is harmless and keeps every step one straight line of code, which the scheduling
+    // hints below then weave into "one MFMA, one LDS read, two VALU" groups: with one wave per
+    // SIMD nothing else hides the non-matrix instructions.
+    auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf) {
+        load_tile(sf, kt + 4);
+        u4_t b[2][kGrTM];
+        read_b(b[0], buf, 0);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            // unit 3 of the CURRENT tile was gathered in the last step of the previous tile
+            unit_finish(g[(s + 1) & 1], s == 0 ? buf : buf ^ 1, (s + 3) & 3);
+            unit_gather(g[s & 1], sn, s);
+            if (s < 3) read_b(b[(s + 1) & 1], buf, s + 1);
+#pragma unroll
+            for (int i = 0; i < kGrTN; i++)
+#pragma unroll
+                for (int j = 0; j < kGrTM; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, afr[buf][i][s]),
+                                                                       __builtin_bit_cast(h8_t, b[s & 1][j]), acc[i][j], 0, 0, 0);
+            x_store(sn, buf ^ 1, s);
+#pragma unroll
+            for (int r = 0; r < 8; r++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+                __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);   // VALU
+            }
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);       // LDS write
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+    };
+
+    for (int kt = 0; kt < k_tiles; kt += 4) {
+        tile(kt, 0, ring[1], ring[0]);
+        if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1]);
+        if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
+        if (kt + 3 < k_tiles) tile(kt + 3, 1, ring[0], ring[3]);
+    }
+
+    // D layout of 32x32: element e of lane: row (n) = 8*(e/4) + 4*(lane/32) + e%4, column (m) = lane%32
+    const bool n_vec = (N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < kGrTN; i++)
+#pragma unroll
+        for (int j = 0; j < kGrTM; j++) {
+            const int m = m0 + j * 32 + l32;
+            if (m >= M) continue;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; e4++) {
+                const int n = n0 + wave * 64 + i * 32 + 8 * e4 + 4 * kq;
+                uint16_t o[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    o[e] = __builtin_bit_cast(uint16_t, (half_t)(acc[i][j][4 * e4 + e] * scale));
+                uint16_t *dst = y + (int64_t)m * N + n;
+                if (n_vec && n + 3 < N) {
+                    u2_t v;
+                    v[0] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+                    v[1] = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+                    *reinterpret_cast<u2_t *>(dst) = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < N) dst[e] = o[e];
+                }
+            }
+        }
+}
+
 // ------------------------------------------------------------------ the reference's integer operator
 // out[m,n] = sum_k x[m,k] * W[n,k] in int32, W decoded to int8 from the packed int64 table
 // exactly as /root/reference/test_decode_matmul.py:29-55 (value = +-byte, then +1 or -1, kept
@@ -1210,15 +1423,38 @@ int launch_gemm(const void *x, const void *codes, const void *grid, float scale,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
 }
 
-// Tuning override for experiments: DMM_GEMM_CFG=a|b|g picks the tile configuration.
+int launch_gemm_reg(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                    int64_t N, int64_t K, hipStream_t stream)
+{
+    static bool attr_done = false;   // benign race: every thread sets the same value
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_reg_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kGrSmemBytes);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    dim3 g((unsigned)((N + kGrBN - 1) / kGrBN), (unsigned)((M + kGrBM - 1) / kGrBM));
+    return launch(gemm_reg_kernel, g, dim3(256), kGrSmemBytes, stream, (const uint16_t *)x, (const uint16_t *)codes,
+                  grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
+}
+
+// the register-operand kernel addresses codes and x through 31-bit buffer offsets
+bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
+{
+    return N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31);
+}
+
+// Tuning override for experiments: DMM_GEMM_CFG=a|b|g picks a tile configuration of the
+// LDS-staged kernel, r (the default where its offsets fit) the register-operand kernel.
 int run_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
     static int cfg = -1;
     if (cfg < 0) {
         const char *e = getenv("DMM_GEMM_CFG");
-        cfg = e ? e[0] : 'a';
+        cfg = e ? e[0] : 0;
     }
+    if ((cfg == 'r' || cfg == 0) && gemm_reg_ok(M, N, K)) return launch_gemm_reg(x, codes, grid, scale, y, M, N, K, stream);
     switch (cfg) {
         case 'b': return launch_gemm<2, 2, 4, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 256 x 128, 4 waves
         case 'g': return launch_gemm<2, 2, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 128 x 128, 4 waves, 2 per CU
