@@ -1020,8 +1020,10 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     const int l32 = lane & 31, kq = lane >> 5;
     const uint32_t lane_base = (uint32_t)(lane & 15) * 16u;
     const uint32_t quarter_bits = 0x34003400u;
-    const int n0 = blockIdx.x * kGrBN;
-    const int m0 = blockIdx.y * kGrBM;
+    // Workgroups go to the 8 XCDs round robin by linear id, so with m fastest the workgroups
+    // of one XCD share a few x row blocks (which then stay in that XCD's L2) and stream the codes.
+    const int m0 = blockIdx.x * kGrBM;
+    const int n0 = blockIdx.y * kGrBN;
     const int k_tiles = K / kGrBK;
     const int row_bytes = K >> 2;
     constexpr int kOut = (int)0x80000000;
@@ -1038,7 +1040,8 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     }
 
     // global sources.  Codes: lane (row l32 of tile i, half kq) reads 8 bytes = codes 4 kq .. 4 kq + 3
-    // of the k tile.  x: thread (row tid / 2, half tid % 2) reads 64 bytes.  Both as raw buffer
+    // of the k tile.  x: load p of thread tid is piece tid % 8 (16 bytes) of row 32 p + tid / 8, so
+    // that 8 lanes cover one 128-byte line.  Both as raw buffer
     // loads: rows past N / M and tiles past K get zeros without a memory access.
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
@@ -1050,8 +1053,13 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         const int n = n0 + wave * 64 + i * 32 + l32;
         cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
     }
-    const int x_row = tid >> 1, x_half = tid & 1;
-    const int xvoff = m0 + x_row < M ? ((m0 + x_row) * K + x_half * 32) * 2 : kOut;
+    const int x_row = tid >> 3, x_piece = tid & 7;
+    int xvoff[4];
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const int m = m0 + 32 * p + x_row;
+        xvoff[p] = m < M ? (m * K + x_piece * 8) * 2 : kOut;
+    }
 
     struct Stage {
         u2_t cw[kGrTN];
@@ -1063,10 +1071,10 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
 #pragma unroll
         for (int i = 0; i < kGrTN; i++) st.cw[i] = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
 #pragma unroll
-        for (int p = 0; p < 4; p++) st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff + p * 16, xoff, 0);
+        for (int p = 0; p < 4; p++) st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
     };
     unsigned char *xs = smem_raw + kSTablesBytes;                       // [2][kGrBM][kGrLd] halves
-    const uint32_t xs_w = lds_addr(xs) + (uint32_t)(x_row * kGrLd + x_half * 32) * 2u;       // this thread's write slot
+    const uint32_t xs_w = lds_addr(xs) + (uint32_t)(x_row * kGrLd + x_piece * 8) * 2u;       // this thread's write slot (p = 0)
     const uint32_t xs_r = lds_addr(xs) + (uint32_t)(l32 * kGrLd + kq * 32) * 2u;             // this lane's B fragments
     constexpr uint32_t kXBuf = kGrBM * kGrLd * 2;
 
@@ -1085,7 +1093,7 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     // A fragments of one k tile: [tile i][k step s], a decoded code each
     u4_t afr[2][kGrTN][4];
     auto x_store = [&](const Stage &st, int buf, int p) {
-        *reinterpret_cast<u4_t *>(xs + (xs_w - lds_addr(xs)) + buf * kXBuf + p * 16) = st.xv[p];
+        *reinterpret_cast<u4_t *>(xs + (xs_w - lds_addr(xs)) + buf * kXBuf + p * (32 * kGrLd * 2)) = st.xv[p];
     };
     // The decode runs as a stream of units, one per k step: unit u of a tile is word u / 2 of
     // row tile u % 2 (two codes = two k steps of that row tile).  A step gathers the table
@@ -1433,7 +1441,7 @@ int launch_gemm_reg(const void *x, const void *codes, const void *grid, float sc
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
-    dim3 g((unsigned)((N + kGrBN - 1) / kGrBN), (unsigned)((M + kGrBM - 1) / kGrBM));
+    dim3 g((unsigned)((M + kGrBM - 1) / kGrBM), (unsigned)((N + kGrBN - 1) / kGrBN));
     return launch(gemm_reg_kernel, g, dim3(256), kGrSmemBytes, stream, (const uint16_t *)x, (const uint16_t *)codes,
                   grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
 }
@@ -1441,7 +1449,7 @@ int launch_gemm_reg(const void *x, const void *codes, const void *grid, float sc
 // the register-operand kernel addresses codes and x through 31-bit buffer offsets
 bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
 {
-    return N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31);
+    return N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31) && N <= 65535LL * kGrBN;
 }
 
 // Tuning override for experiments: DMM_GEMM_CFG=a|b|g picks a tile configuration of the
