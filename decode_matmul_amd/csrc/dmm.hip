@@ -1065,13 +1065,19 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         u2_t cw[kGrTN];
         u4_t xv[4];
     };
-    auto load_tile = [&](Stage &st, int kt) {
+    auto load_codes = [&](Stage &st, int kt) {
         const int coff = kt < k_tiles ? kt * 16 : kOut;
-        const int xoff = kt < k_tiles ? kt * 128 : kOut;
 #pragma unroll
         for (int i = 0; i < kGrTN; i++) st.cw[i] = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
+    };
+    auto load_x = [&](Stage &st, int kt, int p) {
+        const int xoff = kt < k_tiles ? kt * 128 : kOut;
+        st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
+    };
+    auto load_tile = [&](Stage &st, int kt) {
+        load_codes(st, kt);
 #pragma unroll
-        for (int p = 0; p < 4; p++) st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
+        for (int p = 0; p < 4; p++) load_x(st, kt, p);
     };
     unsigned char *xs = smem_raw + kSTablesBytes;                       // [2][kGrBM][kGrLd] halves
     const uint32_t xs_w = lds_addr(xs) + (uint32_t)(x_row * kGrLd + x_piece * 8) * 2u;       // this thread's write slot (p = 0)
@@ -1129,11 +1135,16 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     // hints below then weave into "one MFMA, one LDS read, two VALU" groups: with one wave per
     // SIMD nothing else hides the non-matrix instructions.
     auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf) {
-        load_tile(sf, kt + 4);
         u4_t b[2][kGrTM];
         read_b(b[0], buf, 0);
 #pragma unroll
         for (int s = 0; s < 4; s++) {
+            // the six global loads of tile kt+4, two per step, woven between the MFMAs too
+            if (s == 0) load_codes(sf, kt + 4);
+            if (s == 1 || s == 2) {
+                load_x(sf, kt + 4, 2 * s - 2);
+                load_x(sf, kt + 4, 2 * s - 1);
+            }
             // unit 3 of the CURRENT tile was gathered in the last step of the previous tile
             unit_finish(g[(s + 1) & 1], s == 0 ? buf : buf ^ 1, (s + 3) & 3);
             unit_gather(g[s & 1], sn, s);
@@ -1150,6 +1161,7 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
                 __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);   // VALU
+                if (s < 3 && (r == 1 || r == 4)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
             }
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);       // LDS write
             __builtin_amdgcn_sched_barrier(0);
