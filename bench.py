@@ -25,9 +25,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 # HBM bytes one GEMV launch moves, averaged over the four shapes: rocprofv3 FETCH_SIZE and
-# WRITE_SIZE per dispatch (19,134.7 KiB and 27.0 KiB), each scaled by what the same counter
+# WRITE_SIZE per dispatch (19,132.8 KiB and 28.7 KiB), each scaled by what the same counter
 # reads for a plain 256 MiB device copy (x2.000 and x1.000).  Algorithmic code bytes: 38,797,312.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 39215000
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 39213000
 
 
 def parse():
@@ -255,7 +255,7 @@ def prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes):
     return {"shapes": rows,
             "roofline": {"bound": "mfma", "achieved": round(tot_f / tot_t / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": round(tot_f / tot_t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                         "traffic": None, "kernel": "dmm::gemm_kernel"}}
+                         "traffic": None, "kernel": "dmm::gemm_reg_kernel"}}
 
 
 def cpu_baseline(torch, workload):

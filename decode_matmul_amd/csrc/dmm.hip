@@ -396,7 +396,7 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
                                                              const uint16_t *__restrict__ codes,
                                                              const void *__restrict__ grid, float scale,
                                                              uint16_t *__restrict__ y, int M, int N, int K,
-                                                             int n_tiles)
+                                                             int tiles_q, int tiles_r)
 {
     static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
@@ -431,10 +431,11 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
     }
 
     const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;   // k steps of this wave per row block
-    // this workgroup's share of the 16-row tiles: a contiguous range, equal to within one tile
-    // over the grid, walked R tiles (one row block) at a time; the last block may be partial
-    const int t0 = (int)(((int64_t)n_tiles * (int)blockIdx.x) / (int)gridDim.x);
-    const int t1 = (int)(((int64_t)n_tiles * ((int)blockIdx.x + 1)) / (int)gridDim.x);
+    // this workgroup's share of the 16-row tiles: a contiguous range, tiles_q tiles plus one
+    // more for the first tiles_r workgroups (quotient and remainder of tiles / workgroups, from
+    // the host), walked R tiles (one row block) at a time; the last block may be partial
+    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
+    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
     const int nb_wg = (t1 - t0 + R - 1) / R;
 
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -606,7 +607,7 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
                                                            const uint16_t *__restrict__ codes,
                                                            const void *__restrict__ grid, float scale,
                                                            uint16_t *__restrict__ y, int M, int N, int K,
-                                                           int n_tiles)
+                                                           int tiles_q, int tiles_r)
 {
     static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
@@ -628,8 +629,8 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
 
     const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;
     // contiguous, balanced range of 16-row tiles per workgroup, as in the streaming kernel
-    const int t0 = (int)(((int64_t)n_tiles * (int)blockIdx.x) / (int)gridDim.x);
-    const int t1 = (int)(((int64_t)n_tiles * ((int)blockIdx.x + 1)) / (int)gridDim.x);
+    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
+    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
     const int nb_wg = (t1 - t0 + R - 1) / R;
 
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -1372,7 +1373,7 @@ int launch_gemv_stream(const void *x, const void *codes, const void *grid, float
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     return launch(gemv_stream_kernel<R, W, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
-                  (int)n_tiles);
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
 
 // tables, partial sums and x fit in the 160 KB of LDS, and every byte offset of the code
@@ -1400,7 +1401,7 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     return launch(gemv_regx_kernel<R, W, MT, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
-                  (int)n_tiles);
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
 
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
