@@ -170,6 +170,7 @@ def main():
     }
 
     if not args.quick:
+        out["gemv_7b_shapes"] = gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes)
         out["small_batch"] = small_batch(torch, lib, capi, workload, dev, stream, rand_codes)
         out["prefill"] = prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes)
         out["cpu_baseline"] = cpu_baseline(torch, workload)
@@ -191,6 +192,38 @@ def timed_kernel(torch, lib, fn, reps):
     torch.cuda.synchronize()
     t = [a.elapsed_time(b) * 1e-3 for a, b in ev]
     return sum(t) / len(t)
+
+
+def gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes):
+    """configs[1]: batch-1 GEMV at the Llama-2-7B projection shapes, 30 code buffers in rotation
+    per shape (> 256 MB except 4096 -> 4096: 126 MB)."""
+    rows = []
+    for K, N in workload.LLAMA2_7B:
+        copies = 30
+        codes = rand_codes(N, K, copies, 7)
+        x, _, grid, scale = workload.make_inputs(1, 8, K, seed=0)
+        x, grid = x.to(dev), grid.to(dev)
+        y = torch.empty(1, N, dtype=torch.float16, device=dev)
+
+        def fn(i):
+            st = lib.dmm_decode_matmul_f16(x.data_ptr(), codes[i % copies].data_ptr(), grid.data_ptr(), scale,
+                                           y.data_ptr(), 1, N, K, stream)
+            assert st == 0, st
+        for i in range(5):
+            fn(i)
+        # these kernels run 5-7 us, close to the ~4 us floor of an event pair around one kernel,
+        # so time 120 back-to-back launches as one region instead (launch gaps included)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(120):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        t = a.elapsed_time(b) * 1e-3 / 120
+        gbs = workload.code_bytes(N, K) / t / 1e9
+        rows.append({"K": K, "N": N, "code_bytes": workload.code_bytes(N, K), "us_per_launch": round(t * 1e6, 3),
+                     "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
+    return rows
 
 
 def small_batch(torch, lib, capi, workload, dev, stream, rand_codes):

@@ -274,6 +274,45 @@ def test_repeatable_and_stream_ordered():
         assert torch.equal(first, again)
 
 
+def test_graph_capture_and_replay():
+    """The entry points only enqueue kernels (no allocation, no synchronisation), so a decode
+    step can be captured in a HIP graph.  Every replay is checked against the eager result,
+    with eager work and synchronisations between the replays, after x has been changed in
+    place (a replay must read the current contents of its buffers)."""
+    shapes = [(1, 1024, 4096), (1, 4096, 1024), (8, 512, 2048), (160, 384, 512)]
+    probs = []
+    for i, (M, N, K) in enumerate(shapes):
+        x, codes, grid, scale = workload.make_inputs(M, N, K, seed=40 + i)
+        probs.append([dev(x), dev(codes), dev(grid), scale, torch.empty(M, N, dtype=torch.float16, device=DEV)])
+    W = torch.empty(shapes[0][1], shapes[0][2], dtype=torch.float16, device=DEV)
+
+    def step():
+        for xd, cd, gd, scale, y in probs:
+            c_matmul(xd, cd, gd, scale, "auto", out=y)
+        c_decode(probs[0][1], probs[0][2], out=W)
+
+    step()                                   # warm-up outside the capture (kernel attributes are set here)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        for p in probs:
+            p[0].mul_(-0.5 if rep else 1.0)  # eager work between replays, changes the input
+        torch.cuda.synchronize()
+        for p in probs:
+            p[4].fill_(float("nan"))
+        W.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [p[4].clone() for p in probs] + [W.clone()]
+        step()                               # eager, same buffers
+        torch.cuda.synchronize()
+        want = [p[4] for p in probs] + [W]
+        for g, w in zip(got, want):
+            assert torch.equal(g, w), rep
+
+
 def test_kernel_event_hook_times_the_kernel():
     x, codes, grid, scale = workload.make_inputs(1, 8192, 8192, seed=2)
     xd, cd, gd = dev(x), dev(codes), dev(grid)
