@@ -259,6 +259,54 @@ def test_full_size_against_decode_then_fp32_matmul(M, N, K):
     assert torch.allclose(y2.float(), 2 * y.float(), rtol=2e-3, atol=1e-3)
 
 
+# ----------------------------------------------------------------- maximum sizes
+def _sampled_rows_check(M, N, K, path, seed):
+    """A code matrix too large to decode whole: run the operator on all of it, then check a
+    sample of output columns (first, last and random rows of W, i.e. the lowest and highest
+    byte offsets) against the oracle on just those rows."""
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    codes = torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=DEV)
+    x, _, grid, scale = workload.make_inputs(M, 8, K, seed=seed)
+    y = c_matmul(dev(x), codes, dev(grid), scale, path)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(seed)
+    rows = np.unique(np.concatenate([np.arange(40), np.arange(N - 72, N), rng.integers(0, N, size=64)]))
+    sub = codes[torch.from_numpy(rows).to(DEV)].cpu().numpy()
+    want = orc.matmul_f32(x.numpy(), orc.decode_f16(sub, grid.numpy()), scale)
+    got = y[:, torch.from_numpy(rows).to(DEV)]
+    assert_close_to_oracle(got, want, "%s M=%d N=%d K=%d sampled rows" % (path, M, N, K))
+    assert not torch.isnan(y).any()
+    del codes, y
+    torch.cuda.empty_cache()
+
+
+def test_code_matrix_just_below_2_gib_streams():
+    """N * K / 4 = 2^31 - 512 KiB: the largest code matrix the kernels with 31-bit buffer
+    offsets address."""
+    _sampled_rows_check(1, 524160, 16384, "gemv", 71)      # streaming kernel
+    _sampled_rows_check(20, 524160, 16384, "gemv", 74)     # small-batch kernel
+    _sampled_rows_check(40, 524160, 16384, "gemm", 75)     # register-operand matrix-matrix kernel
+
+
+def test_code_matrix_above_2_gib_takes_the_64_bit_path():
+    """N * K / 4 just above 2^31 bytes: the dispatcher must leave the kernels with 31-bit
+    offsets (the explicit matrix-vector entry point refuses) and still be right."""
+    M, N, K = 3, 524544, 16384
+    p = ctypes_null_call_gemv(M, N, K)
+    assert p == -5
+    _sampled_rows_check(M, N, K, "auto", 72)
+    _sampled_rows_check(40, N, K, "gemm", 73)
+
+
+def ctypes_null_call_gemv(M, N, K):
+    """Status of dmm_gemv_f16 for a shape, with dummy (never dereferenced: the call is refused
+    on the host) but aligned non-null pointers."""
+    buf = torch.empty(64, dtype=torch.float16, device=DEV)
+    ptr = buf.data_ptr()
+    return capi.lib().dmm_gemv_f16(ptr, ptr, ptr, 1.0, ptr, M, N, K, None)
+
+
 def test_repeatable_and_stream_ordered():
     """Same inputs -> same bits, run after run (no atomics, no races), also on a side stream
     while the default stream is busy."""
