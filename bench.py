@@ -36,6 +36,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="skip prefill / small-batch / CPU legs")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the M = 2048 leg and print its object (for profiling the matrix-matrix kernel)")
     ap.add_argument("--rotate-mb", type=int, default=400, help="distinct code bytes to rotate through, at least")
@@ -105,12 +106,38 @@ def main():
         for p in probs:
             call(p["x"], p["codes"][i % copies], p["grid"], p["scale"], p["y"])
 
+    # One HIP graph per code-buffer set (a step = its four launches), so that the timed loop
+    # costs the host one graph launch per step: with four ctypes calls per 56 us step the loop
+    # sits close to being bound by the host, and a busy host core then shows up in `value`.
+    run_step = step
+    launch_mode = "eager"
+    if not args.no_graph:
+        try:
+            for i in range(copies):
+                step(i)                      # kernel attributes are set outside the capture
+            torch.cuda.synchronize()
+            graphs = []
+            for c in range(copies):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    cap = torch.cuda.current_stream().cuda_stream
+                    for p in probs:
+                        st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][c].data_ptr(), p["grid"].data_ptr(),
+                                                       p["scale"], p["y"].data_ptr(), 1, p["N"], p["K"], cap)
+                        if st != 0:
+                            raise capi.DmmError("dmm_decode_matmul_f16", st)
+                graphs.append(g)
+            run_step = lambda i: graphs[i % copies].replay()
+            launch_mode = "hip graph, one replay per step"
+        except Exception as e:   # capture unavailable: time the eager loop
+            print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
+            run_step = step
     for i in range(args.warmup):
-        step(i)
+        run_step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(i)
+        run_step(i)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
@@ -160,7 +187,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "configs[2]: batch-1 decode-GEMV, 8192->10240, 8192->8192, 8192->28672, 28672->8192",
                    "M": 1, "code_buffers_rotated": copies, "distinct_code_MB": round(copies * step_bytes / 1e6, 1),
-                   "step": "4 GEMVs, one per shape"},
+                   "step": "4 GEMVs, one per shape", "launch": launch_mode},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "dmm::gemv_stream_kernel", "launches": n_launch,
@@ -235,15 +262,18 @@ def small_batch(torch, lib, capi, workload, dev, stream, rand_codes):
             x, _, grid, scale = workload.make_inputs(M, 8, K, seed=0)
             x, grid = x.to(dev), grid.to(dev)
             y = torch.empty(M, N, dtype=torch.float16, device=dev)
+            # the operator's workspace (split-K partial sums for short x; 0 bytes = none used)
+            ws_bytes = lib.dmm_workspace_bytes(M, N, K)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
 
             def fn(i):
-                st = lib.dmm_decode_matmul_f16(x.data_ptr(), codes[i % copies].data_ptr(), grid.data_ptr(), scale,
-                                               y.data_ptr(), M, N, K, stream)
+                st = lib.dmm_decode_matmul_ws_f16(x.data_ptr(), codes[i % copies].data_ptr(), grid.data_ptr(), scale,
+                                                  y.data_ptr(), M, N, K, ws.data_ptr(), ws_bytes, stream)
                 assert st == 0, st
             for i in range(5):
                 fn(i)
-            t = timed_kernel(torch, lib, fn, 48)
-            rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3),
+            t = timed_kernel(torch, lib, fn, 48)     # spans both kernels when the call splits K
+            rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3), "workspace_MB": round(ws_bytes / 1e6, 1),
                          "GBps_code": round(workload.code_bytes(N, K) / t / 1e9, 1),
                          "TFLOPs": round(workload.flops(M, N, K) / t / 1e12, 2)})
     return rows

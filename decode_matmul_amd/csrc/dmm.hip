@@ -1004,15 +1004,22 @@ __device__ __forceinline__ h8_t gemm_finish(const u4_t &g, const u4_t &sg, uint3
     return __builtin_bit_cast(h8_t, r);
 }
 
-constexpr int kGrBN = 256, kGrBM = 128, kGrBK = 64, kGrLd = kGrBK + 8;
-constexpr int kGrTN = 2, kGrTM = 4;
-constexpr int kGrSmemBytes = kSTablesBytes + 2 * kGrBM * kGrLd * 2;
+constexpr int kGrBN = 256, kGrBK = 64, kGrLd = kGrBK + 8;
+constexpr int kGrTN = 2;
+__host__ __device__ constexpr int gr_smem_bytes(int TM) { return kSTablesBytes + 2 * (32 * TM) * kGrLd * 2; }
 
+// TM = 32-row tiles of x per workgroup (block tile 256 x 32 TM): 4 for prefill, 2 and 1 for
+// shorter x.  kSplit: blockIdx.z picks a contiguous share of the k tiles and the block writes
+// fp32 partial sums to part[z][M][N] instead of y (summed, scaled and rounded by
+// splitk_reduce_kernel), so that short x still fills the chip with workgroups.
+template <int TM, bool kSplit>
 __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restrict__ x,
                                                        const uint16_t *__restrict__ codes,
                                                        const void *__restrict__ grid, float scale,
-                                                       uint16_t *__restrict__ y, int M, int N, int K)
+                                                       uint16_t *__restrict__ y, float *__restrict__ part,
+                                                       int M, int N, int K, int splits)
 {
+    constexpr int kBM = 32 * TM;
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
     if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     const int tid = threadIdx.x;
@@ -1023,11 +1030,17 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     const uint32_t quarter_bits = 0x34003400u;
     // Workgroups go to the 8 XCDs round robin by linear id, so with m fastest the workgroups
     // of one XCD share a few x row blocks (which then stay in that XCD's L2) and stream the codes.
-    const int m0 = blockIdx.x * kGrBM;
+    const int m0 = blockIdx.x * kBM;
     const int n0 = blockIdx.y * kGrBN;
-    const int k_tiles = K / kGrBK;
     const int row_bytes = K >> 2;
     constexpr int kOut = (int)0x80000000;
+    // this block's k tiles: [kt_lo, kt_lo + k_tiles)
+    int kt_lo = 0, k_tiles = K / kGrBK;
+    if (kSplit) {
+        const int z = blockIdx.z, tq = k_tiles / splits, tr = k_tiles % splits;
+        kt_lo = z * tq + (z < tr ? z : tr);
+        k_tiles = tq + (z < tr ? 1 : 0);
+    }
 
     // tables: thread tid owns grid row tid (16 copies) and 8 of the 2048 sign slots
     {
@@ -1043,7 +1056,7 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     // global sources.  Codes: lane (row l32 of tile i, half kq) reads 8 bytes = codes 4 kq .. 4 kq + 3
     // of the k tile.  x: load p of thread tid is piece tid % 8 (16 bytes) of row 32 p + tid / 8, so
     // that 8 lanes cover one 128-byte line.  Both as raw buffer
-    // loads: rows past N / M and tiles past K get zeros without a memory access.
+    // loads: rows past N / M and tiles past the end get zeros without a memory access.
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
     const __amdgpu_buffer_rsrc_t xrsrc =
@@ -1055,52 +1068,52 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
     }
     const int x_row = tid >> 3, x_piece = tid & 7;
-    int xvoff[4];
+    int xvoff[TM];
 #pragma unroll
-    for (int p = 0; p < 4; p++) {
+    for (int p = 0; p < TM; p++) {
         const int m = m0 + 32 * p + x_row;
         xvoff[p] = m < M ? (m * K + x_piece * 8) * 2 : kOut;
     }
 
     struct Stage {
         u2_t cw[kGrTN];
-        u4_t xv[4];
+        u4_t xv[TM];
     };
-    auto load_codes = [&](Stage &st, int kt) {
-        const int coff = kt < k_tiles ? kt * 16 : kOut;
+    auto load_codes = [&](Stage &st, int kt) {   // kt counts this block's tiles
+        const int coff = kt < k_tiles ? (kt_lo + kt) * 16 : kOut;
 #pragma unroll
         for (int i = 0; i < kGrTN; i++) st.cw[i] = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
     };
     auto load_x = [&](Stage &st, int kt, int p) {
-        const int xoff = kt < k_tiles ? kt * 128 : kOut;
+        const int xoff = kt < k_tiles ? (kt_lo + kt) * 128 : kOut;
         st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
     };
     auto load_tile = [&](Stage &st, int kt) {
         load_codes(st, kt);
 #pragma unroll
-        for (int p = 0; p < 4; p++) load_x(st, kt, p);
+        for (int p = 0; p < TM; p++) load_x(st, kt, p);
     };
-    unsigned char *xs = smem_raw + kSTablesBytes;                       // [2][kGrBM][kGrLd] halves
-    const uint32_t xs_w = lds_addr(xs) + (uint32_t)(x_row * kGrLd + x_piece * 8) * 2u;       // this thread's write slot (p = 0)
+    unsigned char *xs = smem_raw + kSTablesBytes;                       // [2][kBM][kGrLd] halves
+    const uint32_t xs_w = (uint32_t)(x_row * kGrLd + x_piece * 8) * 2u;                      // this thread's write slot (p = 0)
     const uint32_t xs_r = lds_addr(xs) + (uint32_t)(l32 * kGrLd + kq * 32) * 2u;             // this lane's B fragments
-    constexpr uint32_t kXBuf = kGrBM * kGrLd * 2;
+    constexpr uint32_t kXBuf = kBM * kGrLd * 2;
 
     Stage ring[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) load_tile(ring[i], i);
 
-    f16_t acc[kGrTN][kGrTM];
+    f16_t acc[kGrTN][TM];
 #pragma unroll
     for (int i = 0; i < kGrTN; i++)
 #pragma unroll
-        for (int j = 0; j < kGrTM; j++)
+        for (int j = 0; j < TM; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
     // A fragments of one k tile: [tile i][k step s], a decoded code each
     u4_t afr[2][kGrTN][4];
     auto x_store = [&](const Stage &st, int buf, int p) {
-        *reinterpret_cast<u4_t *>(xs + (xs_w - lds_addr(xs)) + buf * kXBuf + p * (32 * kGrLd * 2)) = st.xv[p];
+        *reinterpret_cast<u4_t *>(xs + xs_w + buf * kXBuf + p * (32 * kGrLd * 2)) = st.xv[p];
     };
     // The decode runs as a stream of units, one per k step: unit u of a tile is word u / 2 of
     // row tile u % 2 (two codes = two k steps of that row tile).  A step gathers the table
@@ -1122,30 +1135,34 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         if (u < 3) unit_finish(g[u & 1], 0, u);   // unit 3 is finished by the first step of the loop
     }
 #pragma unroll
-    for (int p = 0; p < 4; p++) x_store(ring[0], 0, p);
+    for (int p = 0; p < TM; p++) x_store(ring[0], 0, p);
     __syncthreads();   // x tile 0 staged
 
-    auto read_b = [&](u4_t (&b)[kGrTM], int buf, int s) {
+    auto read_b = [&](u4_t (&b)[TM], int buf, int s) {
 #pragma unroll
-        for (int j = 0; j < kGrTM; j++) b[j] = lds_read16(xs_r + buf * kXBuf + (uint32_t)(j * 32 * kGrLd * 2 + s * 16));
+        for (int j = 0; j < TM; j++) b[j] = lds_read16(xs_r + buf * kXBuf + (uint32_t)(j * 32 * kGrLd * 2 + s * 16));
     };
     // MFMAs of tile kt (A = afr[buf], B from x buffer buf) while tile kt+1 (registers sn) is
     // decoded into afr[buf ^ 1] and its x written to buffer buf ^ 1, and tile kt+4 is fetched
     // into sf.  Past the last tile sn holds zeros (out-of-range loads): decoding and storing
     // them is harmless and keeps every step one straight line of code, which the scheduling
-    // hints below then weave into "one MFMA, one LDS read, two VALU" groups: with one wave per
+    // hints below then weave into groups of one MFMA, LDS reads and VALU: with one wave per
     // SIMD nothing else hides the non-matrix instructions.
+    constexpr int kMfma = kGrTN * TM;                       // MFMAs per k step
+    constexpr int kDsPer = (TM + 4 + kMfma - 1) / kMfma;    // LDS reads per MFMA group
+    constexpr int kValuPer = (24 + kMfma - 1) / kMfma;      // VALU per MFMA group
     auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf) {
-        u4_t b[2][kGrTM];
+        u4_t b[2][TM];
         read_b(b[0], buf, 0);
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            // the six global loads of tile kt+4, two per step, woven between the MFMAs too
+            // the global loads of tile kt+4 spread over the steps, woven between the MFMAs too
             if (s == 0) load_codes(sf, kt + 4);
-            if (s == 1 || s == 2) {
+            if (TM == 4 && (s == 1 || s == 2)) {
                 load_x(sf, kt + 4, 2 * s - 2);
                 load_x(sf, kt + 4, 2 * s - 1);
             }
+            if (TM < 4 && s >= 1 && s <= TM) load_x(sf, kt + 4, s - 1);
             // unit 3 of the CURRENT tile was gathered in the last step of the previous tile
             unit_finish(g[(s + 1) & 1], s == 0 ? buf : buf ^ 1, (s + 3) & 3);
             unit_gather(g[s & 1], sn, s);
@@ -1153,18 +1170,18 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
 #pragma unroll
             for (int i = 0; i < kGrTN; i++)
 #pragma unroll
-                for (int j = 0; j < kGrTM; j++)
+                for (int j = 0; j < TM; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, afr[buf][i][s]),
                                                                        __builtin_bit_cast(h8_t, b[s & 1][j]), acc[i][j], 0, 0, 0);
-            x_store(sn, buf ^ 1, s);
+            if (s < TM) x_store(sn, buf ^ 1, s);
 #pragma unroll
-            for (int r = 0; r < 8; r++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
-                __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);   // VALU
-                if (s < 3 && (r == 1 || r == 4)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
+            for (int r = 0; r < kMfma; r++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, kDsPer, 0);     // LDS reads
+                __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0);   // VALU
+                if (s < 3 && (r == 1 || r == kMfma / 2)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
             }
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);       // LDS write
+            if (s < TM) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS write
             __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();
@@ -1182,12 +1199,24 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
 #pragma unroll
     for (int i = 0; i < kGrTN; i++)
 #pragma unroll
-        for (int j = 0; j < kGrTM; j++) {
+        for (int j = 0; j < TM; j++) {
             const int m = m0 + j * 32 + l32;
             if (m >= M) continue;
 #pragma unroll
             for (int e4 = 0; e4 < 4; e4++) {
                 const int n = n0 + wave * 64 + i * 32 + 8 * e4 + 4 * kq;
+                if (kSplit) {
+                    float *dst = part + ((int64_t)blockIdx.z * M + m) * N + n;
+                    if (n_vec && n + 3 < N) {
+                        *reinterpret_cast<f4_t *>(dst) =
+                            f4_t{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (n + e < N) dst[e] = acc[i][j][4 * e4 + e];
+                    }
+                    continue;
+                }
                 uint16_t o[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++)
@@ -1205,6 +1234,31 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
                 }
             }
         }
+}
+
+// y = half(scale * sum_z part[z]) over M * N elements; the order of the sum is fixed, so the
+// result does not depend on how the blocks were scheduled.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ part, uint16_t *__restrict__ y,
+                                                            int64_t mn, int splits, float scale)
+{
+    const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i4 >= mn) return;
+    if (i4 + 3 < mn && (mn & 3) == 0) {
+        f4_t sacc = *reinterpret_cast<const f4_t *>(part + i4);
+        for (int z = 1; z < splits; z++) sacc += *reinterpret_cast<const f4_t *>(part + (int64_t)z * mn + i4);
+        u2_t v;
+        v[0] = (uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sacc[0] * scale)) |
+               ((uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sacc[1] * scale)) << 16);
+        v[1] = (uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sacc[2] * scale)) |
+               ((uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sacc[3] * scale)) << 16);
+        *reinterpret_cast<u2_t *>(y + i4) = v;
+    } else {
+        for (int64_t i = i4; i < mn && i < i4 + 4; i++) {
+            float sacc = part[i];
+            for (int z = 1; z < splits; z++) sacc += part[(int64_t)z * mn + i];
+            y[i] = __builtin_bit_cast(uint16_t, (half_t)(sacc * scale));
+        }
+    }
 }
 
 // ------------------------------------------------------------------ the reference's integer operator
@@ -1285,11 +1339,14 @@ __global__ void zero_i32_kernel(int32_t *y, int64_t n)
 thread_local hipEvent_t tls_start = nullptr;
 thread_local hipEvent_t tls_stop = nullptr;
 
-template <typename Kern, typename... Args>
+// kFirst / kLast: whether this launch opens / closes the span the timing events bracket (an
+// operator call that takes two kernels records start before the first and stop after the second)
+template <bool kFirst = true, bool kLast = true, typename Kern, typename... Args>
 int launch(Kern kernel, dim3 grid, dim3 block, size_t shmem, hipStream_t stream, Args... args)
 {
     if (tls_start && tls_stop)
-        hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, tls_start, tls_stop, 0, args...);
+        hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, kFirst ? tls_start : nullptr,
+                              kLast ? tls_stop : nullptr, 0, args...);
     else
         hipLaunchKernelGGL(kernel, grid, block, shmem, stream, args...);
     return (int)hipGetLastError();
@@ -1444,25 +1501,92 @@ int launch_gemm(const void *x, const void *codes, const void *grid, float scale,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
 }
 
-int launch_gemm_reg(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                    int64_t N, int64_t K, hipStream_t stream)
+template <int TM, bool kSplit>
+int launch_gemm_reg_tm(const void *x, const void *codes, const void *grid, float scale, void *y, float *part,
+                       int64_t M, int64_t N, int64_t K, int splits, hipStream_t stream)
 {
     static bool attr_done = false;   // benign race: every thread sets the same value
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_reg_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kGrSmemBytes);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_reg_kernel<TM, kSplit>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, gr_smem_bytes(TM));
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
-    dim3 g((unsigned)((M + kGrBM - 1) / kGrBM), (unsigned)((N + kGrBN - 1) / kGrBN));
-    return launch(gemm_reg_kernel, g, dim3(256), kGrSmemBytes, stream, (const uint16_t *)x, (const uint16_t *)codes,
-                  grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
+    dim3 g((unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)((N + kGrBN - 1) / kGrBN), (unsigned)splits);
+    return launch<true, !kSplit>(gemm_reg_kernel<TM, kSplit>, g, dim3(256), gr_smem_bytes(TM), stream,
+                                 (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, part, (int)M,
+                                 (int)N, (int)K, splits);
+}
+
+// rows of x per block: 32, 64 or 128
+inline int gemm_reg_tm(int64_t M) { return M <= 32 ? 1 : M <= 64 ? 2 : 4; }
+
+int launch_gemm_reg(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                    int64_t N, int64_t K, hipStream_t stream)
+{
+    switch (gemm_reg_tm(M)) {
+        case 1: return launch_gemm_reg_tm<1, false>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+        case 2: return launch_gemm_reg_tm<2, false>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+        default: return launch_gemm_reg_tm<4, false>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+    }
+}
+
+// How many ways to split K so that the blocks about fill the chip: as many as fit the CU count
+// without starting a second round, each with at least 4 k tiles, and no more than the
+// workspace holds partial sums for.  1 = no split.
+int splitk_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes)
+{
+    const int tm = gemm_reg_tm(M);
+    const int64_t tiles = ((M + 32 * tm - 1) / (32 * tm)) * ((N + kGrBN - 1) / kGrBN);
+    int64_t splits = cu_count() / tiles;
+    const int64_t k_tiles = K / kGrBK;
+    if (splits > k_tiles / 4) splits = k_tiles / 4;
+    if (splits > 64) splits = 64;
+    const int64_t per_split = M * N * 4;
+    if (per_split > 0 && splits * per_split > workspace_bytes) splits = workspace_bytes / per_split;
+    return splits < 2 ? 1 : (int)splits;
+}
+
+int launch_gemm_splitk(const void *x, const void *codes, const void *grid, float scale, void *y, void *workspace,
+                       int splits, int64_t M, int64_t N, int64_t K, hipStream_t stream)
+{
+    float *part = reinterpret_cast<float *>(workspace);
+    int st;
+    switch (gemm_reg_tm(M)) {
+        case 1: st = launch_gemm_reg_tm<1, true>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+        case 2: st = launch_gemm_reg_tm<2, true>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+        default: st = launch_gemm_reg_tm<4, true>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+    }
+    if (st != 0) return st;
+    const int64_t mn = M * N;
+    const int64_t blocks = (mn + 1023) / 1024;
+    return launch<false, true>(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const float *)part,
+                               (uint16_t *)y, mn, splits, scale);
 }
 
 // the register-operand kernel addresses codes and x through 31-bit buffer offsets
 bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
 {
     return N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31) && N <= 65535LL * kGrBN;
+}
+
+// Smallest M that takes the split-K path when a workspace is given (up to M = 16 the
+// matrix-vector kernels are as fast or faster).  DMM_SPLITK_MIN_M overrides for experiments.
+int splitk_min_m()
+{
+    static int v = -1;
+    if (v < 0) {
+        const char *e = getenv("DMM_SPLITK_MIN_M");
+        v = e ? atoi(e) : 17;
+        if (v < 1) v = 1;
+    }
+    return v;
+}
+
+bool splitk_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
+               int64_t K)
+{
+    return M >= splitk_min_m() && gemm_ok(x, codes, grid, y, M, N, K) && gemm_reg_ok(M, N, K) && aligned(y, 8);
 }
 
 // Tuning override for experiments: DMM_GEMM_CFG=a|b|g picks a tile configuration of the
@@ -1609,6 +1733,30 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
     if (blocks > 65535 * 16) blocks = 65535 * 16;
     return launch(int8_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const int8_t *)x,
                   (const uint16_t *)codes, (const int64_t *)codebook_abs, (int32_t *)out, M, N, K, tiled ? 1 : 0);
+}
+
+int64_t dmm_workspace_bytes(int64_t M, int64_t N, int64_t K)
+{
+    if (M < 1 || N < 1 || K < kGrBK || (K & 63) || M < splitk_min_m() || M > 65535LL * 128 || !gemm_reg_ok(M, N, K))
+        return 0;
+    const int splits = splitk_plan(M, N, K, INT64_MAX);
+    return splits >= 2 ? (int64_t)splits * M * N * 4 : 0;
+}
+
+int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid, float scale, void *y,
+                             int64_t M, int64_t N, int64_t K, void *workspace, int64_t workspace_bytes,
+                             void *stream)
+{
+    int st = check_common(x, codes, grid, y, M, N, K);
+    if (st != DMM_OK || M == 0 || N == 0) return st;
+    if (workspace_bytes < 0) return DMM_ERR_BAD_SHAPE;
+    if (workspace && workspace_bytes > 0 && !aligned(workspace, 16)) return DMM_ERR_MISALIGNED;
+    if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K)) {
+        const int splits = splitk_plan(M, N, K, workspace_bytes);
+        if (splits >= 2)
+            return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, (hipStream_t)stream);
+    }
+    return dmm_decode_matmul_f16(x, codes, grid, scale, y, M, N, K, stream);
 }
 
 int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, float scale, void *y,

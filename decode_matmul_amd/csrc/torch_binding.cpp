@@ -65,6 +65,11 @@ torch::Tensor run(const torch::Tensor &x, const torch::Tensor &codes, const torc
     c10::DeviceGuard guard(x.device());
     torch::Tensor y = torch::empty({M, N}, x.options().requires_grad(false));
     hipStream_t stream = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+    // split-K workspace for short x, from torch's caching allocator: stream-ordered, so calls
+    // on different streams never share one
+    torch::Tensor workspace;
+    const int64_t ws_bytes = path == Path::kAuto ? dmm_workspace_bytes(M, N, K) : 0;
+    if (ws_bytes > 0) workspace = torch::empty({ws_bytes}, x.options().dtype(torch::kUInt8).requires_grad(false));
 
     int st;
     {
@@ -76,7 +81,10 @@ torch::Tensor run(const torch::Tensor &x, const torch::Tensor &codes, const torc
             case Path::kGemv: st = dmm_gemv_f16(xp, cp, gp, sc, yp, M, N, K, stream); break;
             case Path::kGemm: st = dmm_gemm_f16(xp, cp, gp, sc, yp, M, N, K, stream); break;
             case Path::kGeneric: st = dmm_generic_f16(xp, cp, gp, sc, yp, M, N, K, stream); break;
-            default: st = dmm_decode_matmul_f16(xp, cp, gp, sc, yp, M, N, K, stream); break;
+            default:
+                st = dmm_decode_matmul_ws_f16(xp, cp, gp, sc, yp, M, N, K, ws_bytes > 0 ? workspace.data_ptr() : nullptr,
+                                              ws_bytes, stream);
+                break;
         }
     }
     check_status(st, "decode_matmul");

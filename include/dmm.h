@@ -63,6 +63,24 @@ int dmm_decode_f16(const void *codes, const void *grid, void *W,
 int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, float scale,
                           void *y, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* The operator with a caller-provided workspace.  No counterpart in the reference (its one
+ * kernel accumulates split-K partial sums with atomics into the zero-initialised output,
+ * /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:95,172,210-215, which an fp16 output
+ * cannot take).  When x is short (17 <= M, up to a few hundred rows) one block per output
+ * tile leaves most of the chip idle; with a workspace the K dimension is split over several
+ * blocks per tile, each writes fp32 partial sums to the workspace and a second small kernel
+ * adds them in a fixed order (results stay bit-reproducible), scales and rounds into y.
+ *   dmm_workspace_bytes  the size that lets the call split as far as it would like to
+ *                        (0: this shape never uses a workspace); any smaller size is legal
+ *                        and only limits the split.
+ *   workspace            device memory, 16-byte aligned, owned by the caller; it must not be
+ *                        used by another call that may run at the same time (other stream).
+ *                        NULL or workspace_bytes == 0: identical to dmm_decode_matmul_f16. */
+int64_t dmm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid, float scale,
+                             void *y, int64_t M, int64_t N, int64_t K, void *workspace,
+                             int64_t workspace_bytes, void *stream);
+
 /* Explicit paths of the operator, for tests and measurement.  Same arguments.  Each
  * returns DMM_ERR_UNSUPPORTED outside its domain instead of falling back:
  *   dmm_gemv_f16     M <= 32, K % 256 == 0, N % 4 == 0, 16-byte aligned x/codes/grid,

@@ -118,7 +118,12 @@ def test_generic_path(M, N, K):
 def test_auto_dispatch_and_torch_operator(M, N, K):
     y_c = run_case("auto", M, N, K, seed=1)
     y_t = run_case("auto", M, N, K, seed=1, via="torch")
-    assert torch.equal(y_c, y_t)                 # same kernel either way
+    if capi.lib().dmm_workspace_bytes(M, N, K) == 0:
+        assert torch.equal(y_c, y_t)             # same kernel either way
+    else:                                        # the operator brings a workspace: compare like with like
+        x, codes, grid, scale = workload.make_inputs(M, N, K, seed=1)
+        y_w, _ = c_matmul_ws(dev(x), dev(codes), dev(grid), scale)
+        assert torch.equal(y_w, y_t)
 
 
 def test_empty_problems():
@@ -257,6 +262,58 @@ def test_full_size_against_decode_then_fp32_matmul(M, N, K):
     y2 = c_matmul(xd * 2, cd, gd, scale, "auto")
     torch.cuda.synchronize()
     assert torch.allclose(y2.float(), 2 * y.float(), rtol=2e-3, atol=1e-3)
+
+
+# ----------------------------------------------------------------- split-K with a workspace
+def c_matmul_ws(x, codes, grid, scale, ws_bytes=None):
+    M, K = x.shape
+    N = codes.shape[0]
+    want = capi.lib().dmm_workspace_bytes(M, N, K)
+    nbytes = want if ws_bytes is None else ws_bytes
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    y = torch.full((M, N), float("nan"), dtype=torch.float16, device=x.device)
+    st = capi.lib().dmm_decode_matmul_ws_f16(x.data_ptr(), codes.data_ptr(), grid.data_ptr(), float(scale),
+                                             y.data_ptr(), M, N, K, ws.data_ptr(), nbytes,
+                                             torch.cuda.current_stream().cuda_stream)
+    capi.check("dmm_decode_matmul_ws_f16", st)
+    return y, want
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 512, 1024), (32, 1000, 2048), (33, 514, 4096), (64, 256, 8192),
+                                   (100, 771, 1088), (200, 2048, 2048), (48, 4096, 512)])
+def test_split_k_workspace_path(M, N, K):
+    """Short x with a workspace: K is split over several blocks per tile, fp32 partial sums
+    are added in a fixed order.  Same tolerance as every other path, same bits run after run,
+    also with a workspace too small for the preferred split, and the PyTorch operator (which
+    brings its own workspace) returns the same tensor."""
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=M + N)
+    xd, cd, gd = dev(x), dev(codes), dev(grid)
+    ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+    y, want = c_matmul_ws(xd, cd, gd, scale)
+    torch.cuda.synchronize()
+    assert want >= 2 * M * N * 4, "this shape is meant to split"
+    assert_close_to_oracle(y, ref, "split-K M=%d N=%d K=%d" % (M, N, K))
+    y2, _ = c_matmul_ws(xd, cd, gd, scale)
+    assert torch.equal(y, y2)
+    y3, _ = c_matmul_ws(xd, cd, gd, scale, ws_bytes=2 * M * N * 4 + 64)     # room for two splits only
+    assert_close_to_oracle(y3, ref, "split-K, small workspace")
+    y4, _ = c_matmul_ws(xd, cd, gd, scale, ws_bytes=M * N * 4)              # too small to split: plain path
+    assert_close_to_oracle(y4, ref, "split-K, workspace too small")
+    assert torch.equal(dmm.decode_matmul(xd, cd, gd, scale), y)
+
+
+def test_split_k_integer_bridge_is_exact():
+    rng = np.random.default_rng(5)
+    M, N, K = 40, 256, 8192
+    cb = orc.build_codebook_abs()
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    yi = orc.decode_matmul_i32(x, codes, cb)
+    scale = 2.0 ** -8
+    want = (yi.astype(np.float64) / 4 * scale).astype(np.float16)
+    y, wsb = c_matmul_ws(dev(x.astype(np.float16)), dev(codes), dev(orc.grid_from_codebook(cb)), scale)
+    torch.cuda.synchronize()
+    assert wsb > 0 and np.array_equal(bits(y), bits(want))
 
 
 # ----------------------------------------------------------------- maximum sizes

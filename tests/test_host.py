@@ -75,6 +75,18 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert i8(p, odd, p, p, 1, 16, 32, 1, None) == -3
     assert i8(p, p, ctypes.c_void_p(p.value + 4), p, 1, 16, 32, 1, None) == -3
     assert i8(None, None, None, None, 0, 16, 32, 1, None) == 0
+    # the workspace variant: size query, misaligned or negative workspace, NULL workspace = plain call
+    assert lib.dmm_workspace_bytes(1, 4096, 4096) == 0            # batch 1 never splits
+    assert lib.dmm_workspace_bytes(2048, 4096, 4096) == 0         # enough tiles already
+    assert lib.dmm_workspace_bytes(32, 11008, 4096) % (32 * 11008 * 4) == 0
+    assert lib.dmm_workspace_bytes(32, 11008, 4096) >= 2 * 32 * 11008 * 4
+    assert lib.dmm_workspace_bytes(32, 11008, 4100) == 0          # K % 64 != 0: no MFMA kernel
+    assert lib.dmm_workspace_bytes(-1, 8, 64) == 0
+    wsf = lib.dmm_decode_matmul_ws_f16
+    assert wsf(p, p, p, 1.0, p, 32, 4, 20, p, 1024, None) == -2
+    assert wsf(p, p, p, 1.0, p, 32, 4, 64, ctypes.c_void_p(p.value + 4), 1024, None) == -3
+    assert wsf(p, p, p, 1.0, p, 32, 4, 64, p, -5, None) == -2
+    assert wsf(None, None, None, 1.0, None, 0, 4, 64, None, 0, None) == 0
     # the timing hook wants both events or neither
     assert lib.dmm_set_kernel_events(p, None) == -1
     assert lib.dmm_set_kernel_events(None, None) == 0
