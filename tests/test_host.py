@@ -148,3 +148,25 @@ def test_config0_cpu_plumbing():
     y = orc.decode_matmul_f16(x.numpy(), codes.numpy(), grid.numpy(), scale)
     ref = (x.float() @ torch.from_numpy(W).float().T) * scale
     assert torch.allclose(torch.from_numpy(y).float(), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_bench_refuses_more_than_one_gpu_and_needs_a_gpu():
+    """bench.py --gpus N with N > 1 exits with a message (this build is one GPU only); on a
+    machine without a GPU it says so instead of falling back to a CPU path."""
+    import subprocess
+    import sys
+    bench = os.path.join(ROOT, "bench.py")
+    r = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, bench, "--quick", "--steps", "1", "--warmup", "0"],
+                           capture_output=True, text=True, timeout=300)
+        assert r.returncode == 3 and "no GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_graft_entry_has_build_and_smoke():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("graft_entry", os.path.join(ROOT, "__graft_entry__.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert callable(mod.build) and callable(mod.smoke)
