@@ -288,19 +288,25 @@ constexpr int kSTablesBytes = kSSignBytes + kSGridBytes;
 __host__ __device__ constexpr int stream_red_bytes(int R, int W, int M) { return 2 * W * R * 4 * M * 16; }
 
 // Table staging: thread tid fetches ONE grid row (row tid % 256) and writes 4096 / kNThreads
-// of its 16 copies; the 2048 sign slots are computed, 2048 / kNThreads per thread.
+// of its 16 copies (stream_stage_grid); the 2048 sign slots are computed, 2048 / kNThreads per
+// thread (stream_stage_signs: needs no load, so it runs while the loads are in flight).
 template <int kNThreads>
-__device__ __forceinline__ void stream_stage_tables(unsigned char *smem, const u4_t &grow, int tid)
+__device__ __forceinline__ void stream_stage_signs(unsigned char *smem, int tid)
+{
+    u4_t *sg = reinterpret_cast<u4_t *>(smem);
+#pragma unroll
+    for (int i = 0; i < 2048 / kNThreads; i++) sg[tid + i * kNThreads] = sign_row((uint32_t)((tid + i * kNThreads) >> 4));
+}
+
+template <int kNThreads>
+__device__ __forceinline__ void stream_stage_grid(unsigned char *smem, const u4_t &grow, int tid)
 {
     static_assert(kNThreads == 512 || kNThreads == 1024, "staging assumes 512 or 1024 threads");
     constexpr int kCopiesPer = 4096 / kNThreads;          // copies of its row a thread writes
-    u4_t *sg = reinterpret_cast<u4_t *>(smem);
     u4_t *gg = reinterpret_cast<u4_t *>(smem + kSSignBytes);
     const int row = tid & 255, c0 = (tid >> 8) * kCopiesPer;
 #pragma unroll
     for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + ((c0 + i + tid) & 15)] = grow;   // 16 lanes, 16 bank groups
-#pragma unroll
-    for (int i = 0; i < 2048 / kNThreads; i++) sg[tid + i * kNThreads] = sign_row((uint32_t)((tid + i * kNThreads) >> 4));
 }
 
 // Sum over each row of 16 lanes, result in lane 15 of the row (all 64 lanes must be active).
@@ -468,6 +474,8 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 #pragma unroll
     for (int d = 0; d < D; d++) issue(cw[d]);
     DMM_TRACE_MARK(1);
+    stream_stage_signs<64 * W>(smem_raw, tid);
+    __builtin_amdgcn_sched_barrier(0);   // keep the sign rows ahead of the waits for the loads
 
     // x -> LDS (padded pitch): the pieces of row 0 fetched above, then whatever is left
 #pragma unroll
@@ -481,7 +489,7 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
         for (int c = tid; c < row_chunks; c += 64 * W)
             reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = reinterpret_cast<const u4_t *>(x + (int64_t)m * K)[c];
     DMM_TRACE_MARK(2);
-    stream_stage_tables<64 * W>(smem_raw, grow, tid);
+    stream_stage_grid<64 * W>(smem_raw, grow, tid);
     DMM_TRACE_MARK(3);
     __syncthreads();
     DMM_TRACE_MARK(4);
