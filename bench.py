@@ -27,7 +27,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 # HBM bytes one GEMV launch moves, averaged over the four shapes: rocprofv3 FETCH_SIZE and
 # WRITE_SIZE per dispatch (19,132.8 KiB and 28.7 KiB), each scaled by what the same counter
 # reads for a plain 256 MiB device copy (x2.000 and x1.000).  Algorithmic code bytes: 38,797,312.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 39213000
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 39209000
 
 
 def parse():
