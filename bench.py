@@ -50,7 +50,8 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
-              "use --gpus 1.  DESIGN.md says how the path would shard.", file=sys.stderr)
+              "use --gpus 1.  The path shards by rows of the code matrix (column-parallel) or by K "
+              "(row-parallel, one all-reduce of the output).", file=sys.stderr)
         sys.exit(2)
 
     import torch
