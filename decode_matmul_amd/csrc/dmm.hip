@@ -238,11 +238,10 @@ __device__ __forceinline__ uint32_t pk_fma_bcast(uint32_t g, uint32_t s, uint32_
 }
 
 // ------------------------------------------------------------------ streaming matrix-vector path
-// The batch-1 path proper (small M, x small enough to live in LDS).  What the kernel above
-// cannot do is keep enough code bytes in flight: HBM answers in a few microseconds under
-// load, so a CU needs on the order of 100 KB outstanding, and because vector-memory results
-// return in order, any x load queued behind the code prefetch stalls until the whole
-// prefetch has landed.  Here:
+// The batch-1 path proper (small M, x small enough to live in LDS).  Two facts shape it: HBM
+// answers in a few microseconds under load, so a CU must keep tens of KB of code bytes
+// outstanding at all times, and vector-memory results return in order, so any x load queued
+// behind the code prefetch would stall until the whole prefetch had landed.  Hence:
 //   * x is copied once per workgroup into LDS (row pitch 2K + 16 bytes, so the rows read
 //     together fall in different bank groups) and B operands are read from there;
 //   * the code stream is a ring of D register buffers per wave, refilled with raw buffer
