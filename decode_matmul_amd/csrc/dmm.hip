@@ -1404,17 +1404,43 @@ int gemv_cfg_override()
     return cfg;
 }
 
+// State that depends on the device (CU count, per-function attributes) is kept per device
+// ordinal: a process may drive several GPUs, each through its own calls.
+constexpr int kMaxDevices = 64;
+
+inline int current_device()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    return dev;
+}
+
 int cu_count()
 {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
+    static int n[kMaxDevices] = {};
+    const int dev = current_device();
+    if (n[dev] == 0) {
         hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            n = prop.multiProcessorCount;
-        if (n <= 0) n = 256;
+        int v = 0;
+        if (hipGetDeviceProperties(&prop, dev) == hipSuccess) v = prop.multiProcessorCount;
+        n[dev] = v > 0 ? v : 256;
     }
-    return n;
+    return n[dev];
+}
+
+// Allow `bytes` of dynamic LDS for a kernel, once per device (benign race: every thread sets
+// the same value).  Returns 0 or the hipError_t.
+template <typename Kern>
+int allow_dynamic_lds(Kern kernel, int bytes, bool (&done)[kMaxDevices])
+{
+    const int dev = current_device();
+    if (!done[dev]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return (int)e;
+        done[dev] = true;
+    }
+    return 0;
 }
 
 template <int R, int W, int D>
@@ -1426,13 +1452,8 @@ int launch_gemv_stream(const void *x, const void *codes, const void *grid, float
 #else
     const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)M * (2 * K + 16);
 #endif
-    static bool attr_done = false;   // benign race: every thread sets the same value
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_stream_kernel<R, W, D>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return (int)e;
-        attr_done = true;
-    }
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(gemv_stream_kernel<R, W, D>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     return launch(gemv_stream_kernel<R, W, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
@@ -1454,13 +1475,8 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
                      int64_t N, int64_t K, hipStream_t stream)
 {
     const size_t shmem = (size_t)kSTablesBytes + 2 * W * R * MT * kWave * 16;
-    static bool attr_done = false;   // benign race: every thread sets the same value
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_regx_kernel<R, W, MT, D>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return (int)e;
-        attr_done = true;
-    }
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(gemv_regx_kernel<R, W, MT, D>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     return launch(gemv_regx_kernel<R, W, MT, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
@@ -1496,13 +1512,8 @@ int launch_gemm(const void *x, const void *codes, const void *grid, float scale,
                 int64_t N, int64_t K, hipStream_t stream)
 {
     typedef GemmCfg<WN, WM, TN, TM> C;
-    static bool attr_done = false;   // benign race: every thread sets the same value
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<WN, WM, TN, TM>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(typename C::Shared));
-        if (e != hipSuccess) return (int)e;
-        attr_done = true;
-    }
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(gemm_kernel<WN, WM, TN, TM>, (int)sizeof(typename C::Shared), attr_done)) return e;
     dim3 g((unsigned)((N + C::kBN - 1) / C::kBN), (unsigned)((M + C::kBM - 1) / C::kBM));
     return launch(gemm_kernel<WN, WM, TN, TM>, g, dim3(C::kThreads), sizeof(typename C::Shared), stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
@@ -1512,13 +1523,8 @@ template <int TM, bool kSplit>
 int launch_gemm_reg_tm(const void *x, const void *codes, const void *grid, float scale, void *y, float *part,
                        int64_t M, int64_t N, int64_t K, int splits, hipStream_t stream)
 {
-    static bool attr_done = false;   // benign race: every thread sets the same value
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_reg_kernel<TM, kSplit>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, gr_smem_bytes(TM));
-        if (e != hipSuccess) return (int)e;
-        attr_done = true;
-    }
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(gemm_reg_kernel<TM, kSplit>, gr_smem_bytes(TM), attr_done)) return e;
     dim3 g((unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)((N + kGrBN - 1) / kGrBN), (unsigned)splits);
     return launch<true, !kSplit>(gemm_reg_kernel<TM, kSplit>, g, dim3(256), gr_smem_bytes(TM), stream,
                                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, part, (int)M,
