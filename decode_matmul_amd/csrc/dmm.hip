@@ -1074,7 +1074,9 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         const int n = n0 + wave * 64 + i * 32 + l32;
         cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
     }
-    const int x_row = tid >> 3, x_piece = tid & 7;
+    // rows r and r + 8 share a group of 16 lanes: with the 144-byte pitch their 16 pieces fall in
+    // 16 different bank groups, so the LDS writes below are conflict-free like the fragment reads
+    const int x_row = ((tid >> 7) << 4) + ((tid >> 4) & 7) + (((tid >> 3) & 1) << 3), x_piece = tid & 7;
     int xvoff[TM];
 #pragma unroll
     for (int p = 0; p < TM; p++) {
