@@ -264,6 +264,60 @@ def test_full_size_against_decode_then_fp32_matmul(M, N, K):
     assert torch.allclose(y2.float(), 2 * y.float(), rtol=2e-3, atol=1e-3)
 
 
+# ----------------------------------------------------------------- seeded random shapes
+def _random_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        M = int(rng.choice([1, 1, 2, 3, 5, 8, 13, 16, 17, 24, 32, 33, 47, 64, 100, 129, 200]))
+        K = int(rng.choice([8, 24, 64, 72, 256, 320, 512, 1000, 1024, 2048, 2304, 4096]))
+        N = int(rng.choice([1, 3, 4, 15, 16, 17, 36, 64, 100, 255, 256, 257, 500, 1024, 1500]))
+        out.append((M, N, K))
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", _random_shapes(16, 77))
+def test_random_shapes_with_2_byte_aligned_buffers(M, N, K):
+    """x, codes and y at addresses that are only 2-byte aligned: the dispatcher must fall back
+    to kernels without alignment demands, never fault, never write outside y."""
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=M + N + K)
+    ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+
+    def odd(t):   # same values, storage shifted by one element (2 bytes)
+        flat = torch.empty(t.numel() + 1, dtype=t.dtype, device=DEV)
+        flat[1:] = t.reshape(-1).to(DEV)
+        return flat[1:].view(t.shape)
+    xd, cd, gd = odd(x), odd(codes), dev(grid)
+    guard = 63
+    buf = torch.full((M * N + 2 * guard,), 777.0, dtype=torch.float16, device=DEV)
+    y = buf[guard:guard + M * N].view(M, N)
+    assert xd.data_ptr() % 4 == 2 and cd.data_ptr() % 4 == 2 and y.data_ptr() % 4 == 2
+    c_matmul(xd, cd, gd, scale, "auto", out=y)
+    torch.cuda.synchronize()
+    assert_close_to_oracle(y, ref, "unaligned M=%d N=%d K=%d" % (M, N, K))
+    assert torch.all(buf[:guard] == 777.0) and torch.all(buf[guard + M * N:] == 777.0)
+
+
+@pytest.mark.parametrize("M,N,K", _random_shapes(48, 2024))
+def test_random_shapes_dispatch(M, N, K):
+    """Whatever the dispatcher picks for a shape (any of the kernels, with and without a
+    workspace), the result is the oracle's within tolerance and nothing outside y is written."""
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=M * 7 + N * 3 + K)
+    ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+    xd, cd, gd = dev(x), dev(codes), dev(grid)
+    # y inside a guarded buffer: the halves before and after it must keep their pattern
+    guard = 64
+    buf = torch.full((M * N + 2 * guard,), 777.0, dtype=torch.float16, device=DEV)
+    y = buf[guard:guard + M * N].view(M, N)
+    c_matmul(xd, cd, gd, scale, "auto", out=y)
+    torch.cuda.synchronize()
+    assert_close_to_oracle(y, ref, "auto M=%d N=%d K=%d" % (M, N, K))
+    assert torch.all(buf[:guard] == 777.0) and torch.all(buf[guard + M * N:] == 777.0)
+    y_w, _ = c_matmul_ws(xd, cd, gd, scale)
+    torch.cuda.synchronize()
+    assert_close_to_oracle(y_w, ref, "workspace M=%d N=%d K=%d" % (M, N, K))
+
+
 # ----------------------------------------------------------------- split-K with a workspace
 def c_matmul_ws(x, codes, grid, scale, ws_bytes=None):
     M, K = x.shape
