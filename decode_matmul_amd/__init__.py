@@ -40,6 +40,8 @@ __all__ = [
     "decode_matmul",
     "decode_matmul_path",
     "decode_matmul_int8",
+    "pack_codes",
+    "decode_matmul_packed",
     "decode",
     "lib",
     "build_codebook_abs",
@@ -67,6 +69,19 @@ def decode_matmul_int8(x, weights_compressed, codebook_abs, tiled=True):
     table -> int32 [M,N] (decode_matmul_cuda.cu:178-234).  tiled=True: codes as the reference's
     kernel reads them (`transpose_tile`, test_decode_matmul.py:101-109); False: row-major."""
     return _C.decode_matmul_int8(x, weights_compressed, codebook_abs, bool(tiled))
+
+
+def pack_codes(codes):
+    """Offline repack of codes [N, K/8] (K % 256 == 0) for the batch-1 kernel: each wave's load
+    becomes 1 KB of consecutive bytes.  The counterpart of the reference's `transpose_tile`
+    (test_decode_matmul.py:101-109).  Returns [ceil(N/16)*16, K/8], same dtype."""
+    return _C.pack_codes(codes)
+
+
+def decode_matmul_packed(x, packed, grid, scale, N):
+    """`decode_matmul` on codes packed by `pack_codes`; N = rows of the original code matrix.
+    Bit-identical to the row-major call.  Small M with x resident in LDS only (M = 1: K <= 28672)."""
+    return _C.decode_matmul_packed(x, packed, grid, float(scale), int(N))
 
 
 def decode(codes, grid):

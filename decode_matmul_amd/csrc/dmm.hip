@@ -396,7 +396,7 @@ __device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr,
     }
 }
 
-template <int R, int W, int D>
+template <int R, int W, int D, bool kPacked>
 __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__restrict__ x,
                                                              const uint16_t *__restrict__ codes,
                                                              const void *__restrict__ grid, float scale,
@@ -443,15 +443,19 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
     const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
     const int nb_wg = (t1 - t0 + R - 1) / R;
 
+    // Row-major codes [N][K/8]: a lane's 16 bytes are 8 codes of its row, a wave's load touches
+    // 16 rows x 64 bytes.  Packed codes (pack_kernel): the same 16 bytes sit at
+    // ((tile * n_steps + step) * 64 + lane) * 16, so a wave's load is 1 KB of consecutive bytes.
+    const int n_tiles_all = (N + 15) >> 4;
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_tiles_all * 16 : N) * row_bytes), 0x00020000);
     // per-lane byte offset inside a row block (never changes) ...
     int voff[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) voff[r] = (16 * r + c16) * row_bytes + q * 16;
+    for (int r = 0; r < R; r++) voff[r] = kPacked ? lane * 16 + r * n_steps * 1024 : (16 * r + c16) * row_bytes + q * 16;
     // ... and the scalar part: first tile and k step of the next item to prefetch.  Rows past N
-    // land past the end of the buffer by themselves; items past the end get an offset no
-    // buffer reaches.
+    // land past the end of the buffer by themselves (row-major) or are zero padding (packed);
+    // items past the end get an offset no buffer reaches.
     constexpr int kOut = (int)0x80000000;
     int pf_blk = 0, pf_j = 0;
     auto issue = [&](u4_t (&cwd)[R]) {
@@ -462,7 +466,9 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
         const bool ok2 = ok;
 #endif
         const int tb = t0 + pf_blk * R;
-        const int soff = ok2 ? tb * 16 * row_bytes + (wave + pf_j * W) * 64 : kOut;
+        const int soff = !ok2 ? kOut
+                         : kPacked ? (tb * n_steps + wave + pf_j * W) * 1024
+                                   : tb * 16 * row_bytes + (wave + pf_j * W) * 64;
 #pragma unroll
         for (int r = 0; r < R; r++)   // tiles of a partial block that belong to the next workgroup: no access
             cwd[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], (r == 0 || tb + r < t1) ? soff : kOut, 0);
@@ -1344,6 +1350,23 @@ __global__ void zero_i32_kernel(int32_t *y, int64_t n)
         y[i] = 0;
 }
 
+// ------------------------------------------------------------------ offline repack for the streaming kernel
+// packed[((tile * n_steps + step) * 64 + lane) * 8 + e] = codes[16 tile + lane % 16][32 step + 8 (lane / 16) + e]
+// (16-bit units; rows past N are zeros).  One thread moves one 16-byte piece.
+__global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ codes, u4_t *__restrict__ packed,
+                                                   int64_t N, int64_t K, int64_t pieces)
+{
+    const int64_t n_steps = K >> 8, kc = K >> 3;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < pieces; i += (int64_t)gridDim.x * 256) {
+        const int64_t lane = i & 63, chunk = i >> 6;
+        const int64_t step = chunk % n_steps, tile = chunk / n_steps;
+        const int64_t n = tile * 16 + (lane & 15);
+        u4_t v = u4_t{0u, 0u, 0u, 0u};
+        if (n < N) v = *reinterpret_cast<const u4_t *>(codes + n * kc + step * 32 + (lane >> 4) * 8);
+        packed[i] = v;
+    }
+}
+
 // ------------------------------------------------------------------ host side
 thread_local hipEvent_t tls_start = nullptr;
 thread_local hipEvent_t tls_stop = nullptr;
@@ -1445,7 +1468,7 @@ int allow_dynamic_lds(Kern kernel, int bytes, bool (&done)[kMaxDevices])
     return 0;
 }
 
-template <int R, int W, int D>
+template <int R, int W, int D, bool kPacked = false>
 int launch_gemv_stream(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                        int64_t N, int64_t K, hipStream_t stream)
 {
@@ -1455,10 +1478,10 @@ int launch_gemv_stream(const void *x, const void *codes, const void *grid, float
     const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)M * (2 * K + 16);
 #endif
     static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemv_stream_kernel<R, W, D>, 160 * 1024, attr_done)) return e;
+    if (int e = allow_dynamic_lds(gemv_stream_kernel<R, W, D, kPacked>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_stream_kernel<R, W, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+    return launch(gemv_stream_kernel<R, W, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
@@ -1719,6 +1742,37 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
     if (st != DMM_OK || M == 0 || N == 0) return st;
     if (!gemv_ok(x, codes, grid, y, M, N, K)) return DMM_ERR_UNSUPPORTED;
     return run_gemv(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
+}
+
+int64_t dmm_packed_bytes(int64_t N, int64_t K)
+{
+    if (N < 0 || K < 256 || (K & 255)) return 0;
+    return ((N + 15) / 16) * 16 * (K >> 2);
+}
+
+int dmm_pack_codes(const void *codes, void *packed, int64_t N, int64_t K, void *stream)
+{
+    if (N < 0 || K < 0 || (K & 7)) return DMM_ERR_BAD_SHAPE;
+    if (K < 256 || (K & 255)) return DMM_ERR_UNSUPPORTED;
+    if (N == 0) return DMM_OK;
+    if (!codes || !packed) return DMM_ERR_NULL_POINTER;
+    if (!aligned(codes, 16) || !aligned(packed, 16)) return DMM_ERR_MISALIGNED;
+    const int64_t pieces = dmm_packed_bytes(N, K) / 16;
+    int64_t blocks = (pieces + 255) / 256;
+    if (blocks > 65535 * 16) blocks = 65535 * 16;
+    return launch(pack_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)codes,
+                  (u4_t *)packed, N, K, pieces);
+}
+
+int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, float scale, void *y, int64_t M,
+                        int64_t N, int64_t K, void *stream)
+{
+    int st = check_common(x, packed, grid, y, M, N, K);
+    if (st != DMM_OK || M == 0 || N == 0) return st;
+    // the streaming kernel's domain, with the padded size in place of N * K / 4
+    if (!gemv_ok(x, packed, grid, y, M, N, K) || dmm_packed_bytes(N, K) >= (1LL << 31) || !gemv_stream_ok<2, 16>(M, N, K))
+        return DMM_ERR_UNSUPPORTED;
+    return launch_gemv_stream<2, 16, 2, true>(x, packed, grid, scale, y, M, N, K, (hipStream_t)stream);
 }
 
 int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,

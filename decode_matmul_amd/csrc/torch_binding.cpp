@@ -125,6 +125,48 @@ torch::Tensor decode(torch::Tensor codes, torch::Tensor grid)
     return W;
 }
 
+// Offline repack for the batch-1 kernel: codes [N, K/8] -> packed [ceil(N/16)*16, K/8] (same
+// dtype; rows past N are zero padding), and the operator on packed codes.
+torch::Tensor pack_codes(torch::Tensor codes)
+{
+    DMM_CHECK_INPUT(codes);
+    TORCH_CHECK(is_code_dtype(codes) && codes.dim() == 2, "codes must be int16 or uint16 [N, K/8]");
+    const int64_t N = codes.size(0), K = codes.size(1) * 8;
+    TORCH_CHECK(K >= 256 && K % 256 == 0, "packing needs K % 256 == 0");
+    c10::DeviceGuard guard(codes.device());
+    torch::Tensor packed = torch::empty({(N + 15) / 16 * 16, K / 8}, codes.options().requires_grad(false));
+    hipStream_t stream = c10::hip::getCurrentHIPStream(codes.device().index()).stream();
+    int st;
+    {
+        pybind11::gil_scoped_release nogil;
+        st = dmm_pack_codes(codes.data_ptr(), packed.data_ptr(), N, K, stream);
+    }
+    check_status(st, "pack_codes");
+    return packed;
+}
+
+torch::Tensor decode_matmul_packed(torch::Tensor x, torch::Tensor packed, torch::Tensor grid, double scale, int64_t N)
+{
+    DMM_CHECK_INPUT(x);
+    check_codes_grid(packed, grid);
+    TORCH_CHECK(x.scalar_type() == torch::kHalf && x.dim() == 2, "x must be float16 [M, K]");
+    TORCH_CHECK(x.device() == packed.device(), "x and packed must be on the same device");
+    TORCH_CHECK(x.size(-1) == packed.size(-1) * 8, "x.size(-1) must be 8 * packed.size(-1)");
+    TORCH_CHECK(N >= 0 && packed.size(0) == (N + 15) / 16 * 16, "packed must have ceil(N / 16) * 16 rows");
+    const int64_t M = x.size(0), K = x.size(1);
+    c10::DeviceGuard guard(x.device());
+    torch::Tensor y = torch::empty({M, N}, x.options().requires_grad(false));
+    hipStream_t stream = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+    int st;
+    {
+        pybind11::gil_scoped_release nogil;
+        st = dmm_gemv_packed_f16(x.data_ptr(), packed.data_ptr(), grid.data_ptr(), static_cast<float>(scale),
+                                 y.data_ptr(), M, N, K, stream);
+    }
+    check_status(st, "decode_matmul_packed");
+    return y;
+}
+
 // The reference's own signature: int8 x, int16 codes (tiled like its kernel reads them, or
 // row-major), int64[256] table -> int32 (decode_matmul_cuda.cu:178-234).
 torch::Tensor decode_matmul_int8(torch::Tensor x, torch::Tensor weights_compressed, torch::Tensor codebook_abs,
@@ -168,6 +210,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           "The reference's integer operator: int8 x, int16 codes, int64[256] table -> int32",
           pybind11::arg("x"), pybind11::arg("weights_compressed"), pybind11::arg("codebook_abs"),
           pybind11::arg("tiled") = true);
+    m.def("pack_codes", &pack_codes, "codes [N, K/8] -> the batch-1 kernel's packed layout", pybind11::arg("codes"));
+    m.def("decode_matmul_packed", &decode_matmul_packed, "decode_matmul on packed codes (small M, K % 256 == 0)",
+          pybind11::arg("x"), pybind11::arg("packed"), pybind11::arg("grid"), pybind11::arg("scale"), pybind11::arg("N"));
     m.def("decode", &decode, "Decode codes [N, K/8] to the dense half matrix [N, K]",
           pybind11::arg("codes"), pybind11::arg("grid"));
 }

@@ -97,6 +97,23 @@ int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale
 int dmm_generic_f16(const void *x, const void *codes, const void *grid, float scale,
                     void *y, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* Offline repack for the batch-1 kernel (the counterpart of the reference's `transpose_tile`,
+ * /root/reference/test_decode_matmul.py:101-109, which pre-tiles the codes for ITS kernel's
+ * fragment loads).  In the packed form the 16 bytes a lane loads sit at
+ *   ((tile * (K / 256) + step) * 64 + lane) * 16,   tile = n / 16, step = k / 256,
+ *   lane = n % 16 + 16 * (k % 256 / 64),
+ * so a wave's load is 1 KB of consecutive bytes instead of 16 rows x 64 bytes; rows are padded
+ * with zeros to a multiple of 16.  Same arithmetic in the same order as the row-major call:
+ * results are bit-identical.  K % 256 == 0 is required (DMM_ERR_UNSUPPORTED otherwise).
+ *   dmm_packed_bytes     size of the packed buffer (0 if the shape cannot be packed)
+ *   dmm_pack_codes       codes [N, K/8] row-major -> packed; both 16-byte aligned, distinct
+ *   dmm_gemv_packed_f16  the operator on packed codes; domain: that of dmm_gemv_f16 with x
+ *                        resident in LDS (M = 1: K <= 28672), else DMM_ERR_UNSUPPORTED. */
+int64_t dmm_packed_bytes(int64_t N, int64_t K);
+int dmm_pack_codes(const void *codes, void *packed, int64_t N, int64_t K, void *stream);
+int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, float scale,
+                        void *y, int64_t M, int64_t N, int64_t K, void *stream);
+
 /* The reference's operator itself, in integers:
  *   out int32 [M,N] = x int8 [M,K]  @  decode(codes, codebook_abs) int8 [N,K] ^T
  * Replaces `decode_matmul(x, weights_compressed, codebook_abs)` of

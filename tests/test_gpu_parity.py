@@ -318,6 +318,48 @@ def test_random_shapes_dispatch(M, N, K):
     assert_close_to_oracle(y_w, ref, "workspace M=%d N=%d K=%d" % (M, N, K))
 
 
+# ----------------------------------------------------------------- packed codes
+def pack_codes_numpy(codes):
+    """The packed layout, restated with numpy index arithmetic: 16-bit unit
+    ((tile * n_steps + step) * 64 + lane) * 8 + e holds codes[16 tile + lane % 16][32 step + 8 (lane // 16) + e]."""
+    N, kc = codes.shape
+    n_steps = kc // 32
+    tiles = (N + 15) // 16
+    padded = np.zeros((tiles * 16, kc), dtype=codes.dtype)
+    padded[:N] = codes
+    t = padded.reshape(tiles, 16, n_steps, 4, 8)          # [tile][row c16][step][q][e]
+    return np.ascontiguousarray(t.transpose(0, 2, 3, 1, 4)).reshape(tiles * 16, kc)   # [tile][step][q][c16][e]
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 16, 256), (1, 100, 512), (1, 4096, 4096), (3, 1000, 2048), (1, 8192, 8192),
+                                   (1, 1028, 28672), (4, 11008, 4096), (8, 52, 1024)])
+def test_packed_codes_bit_identical(M, N, K):
+    """dmm_pack_codes produces the documented layout, and the operator on packed codes returns
+    exactly the bits of the row-major call (same arithmetic, same order) - which is itself
+    checked against the oracle."""
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=N + K)
+    xd, cd, gd = dev(x), dev(codes), dev(grid)
+    lib = capi.lib()
+    nbytes = lib.dmm_packed_bytes(N, K)
+    assert nbytes == (N + 15) // 16 * 16 * K // 4
+    packed = torch.full((nbytes // 2,), -1, dtype=torch.int16, device=DEV)
+    capi.check("dmm_pack_codes", lib.dmm_pack_codes(cd.data_ptr(), packed.data_ptr(), N, K, None))
+    torch.cuda.synchronize()
+    assert np.array_equal(packed.cpu().numpy().reshape(-1, K // 8), pack_codes_numpy(codes.numpy()))
+    y_ref = c_matmul(xd, cd, gd, scale, "gemv")
+    y = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
+    capi.check("dmm_gemv_packed_f16", lib.dmm_gemv_packed_f16(xd.data_ptr(), packed.data_ptr(), gd.data_ptr(), scale,
+                                                              y.data_ptr(), M, N, K, None))
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_ref)
+    ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+    assert_close_to_oracle(y, ref, "packed M=%d N=%d K=%d" % (M, N, K))
+    # the PyTorch wrappers
+    pk = dmm.pack_codes(cd)
+    assert torch.equal(pk.reshape(-1), packed)
+    assert torch.equal(dmm.decode_matmul_packed(xd, pk, gd, scale, N), y)
+
+
 # ----------------------------------------------------------------- split-K with a workspace
 def c_matmul_ws(x, codes, grid, scale, ws_bytes=None):
     M, K = x.shape

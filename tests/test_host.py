@@ -87,6 +87,16 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert wsf(p, p, p, 1.0, p, 32, 4, 64, ctypes.c_void_p(p.value + 4), 1024, None) == -3
     assert wsf(p, p, p, 1.0, p, 32, 4, 64, p, -5, None) == -2
     assert wsf(None, None, None, 1.0, None, 0, 4, 64, None, 0, None) == 0
+    # packed layout: size query, K % 256, NULLs, alignment
+    assert lib.dmm_packed_bytes(100, 512) == 112 * 128
+    assert lib.dmm_packed_bytes(100, 520) == 0 and lib.dmm_packed_bytes(100, 128) == 0
+    assert lib.dmm_pack_codes(p, p, 16, 520, None) == -5
+    assert lib.dmm_pack_codes(p, p, 16, 12, None) == -2
+    assert lib.dmm_pack_codes(None, p, 16, 512, None) == -1
+    assert lib.dmm_pack_codes(odd, p, 16, 512, None) == -3
+    assert lib.dmm_pack_codes(None, None, 0, 512, None) == 0
+    assert lib.dmm_gemv_packed_f16(p, p, p, 1.0, p, 1, 4, 16, None) == -5
+    assert lib.dmm_gemv_packed_f16(p, p, p, 1.0, p, 64, 16, 512, None) == -5
     # the timing hook wants both events or neither
     assert lib.dmm_set_kernel_events(p, None) == -1
     assert lib.dmm_set_kernel_events(None, None) == 0
