@@ -615,7 +615,7 @@ __device__ __forceinline__ void regx_step(const u4_t (&cw)[R], const u4_t (&xb)[
     }
 }
 
-template <int R, int W, int MT, int D>
+template <int R, int W, int MT, int D, bool kPacked>
 __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__restrict__ x,
                                                            const uint16_t *__restrict__ codes,
                                                            const void *__restrict__ grid, float scale,
@@ -646,14 +646,15 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
     const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
     const int nb_wg = (t1 - t0 + R - 1) / R;
 
+    // row-major or packed codes, addressed as in the streaming kernel
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
     const __amdgpu_buffer_rsrc_t xrsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, M * K * 2, 0x00020000);
     constexpr int kOut = (int)0x80000000;
     int voff[R], xoff[MT];
 #pragma unroll
-    for (int r = 0; r < R; r++) voff[r] = (16 * r + c16) * row_bytes + q * 16;
+    for (int r = 0; r < R; r++) voff[r] = kPacked ? lane * 16 + r * n_steps * 1024 : (16 * r + c16) * row_bytes + q * 16;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
         const int m = 16 * mt + c16;
@@ -670,7 +671,7 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
         const int step = wave + pf_j * W;
         const int xs_off = ok ? step * 512 : kOut;
         const int tb = t0 + pf_blk * R;
-        const int soff = ok ? tb * 16 * row_bytes + step * 64 : kOut;
+        const int soff = !ok ? kOut : kPacked ? (tb * n_steps + step) * 1024 : tb * 16 * row_bytes + step * 64;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
@@ -1495,16 +1496,16 @@ bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
            N * (K >> 2) < (1LL << 31);
 }
 
-template <int R, int W, int MT, int D>
+template <int R, int W, int MT, int D, bool kPacked = false>
 int launch_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                      int64_t N, int64_t K, hipStream_t stream)
 {
     const size_t shmem = (size_t)kSTablesBytes + 2 * W * R * MT * kWave * 16;
     static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemv_regx_kernel<R, W, MT, D>, 160 * 1024, attr_done)) return e;
+    if (int e = allow_dynamic_lds(gemv_regx_kernel<R, W, MT, D, kPacked>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_regx_kernel<R, W, MT, D>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+    return launch(gemv_regx_kernel<R, W, MT, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
@@ -1769,10 +1770,13 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
 {
     int st = check_common(x, packed, grid, y, M, N, K);
     if (st != DMM_OK || M == 0 || N == 0) return st;
-    // the streaming kernel's domain, with the padded size in place of N * K / 4
-    if (!gemv_ok(x, packed, grid, y, M, N, K) || dmm_packed_bytes(N, K) >= (1LL << 31) || !gemv_stream_ok<2, 16>(M, N, K))
-        return DMM_ERR_UNSUPPORTED;
-    return launch_gemv_stream<2, 16, 2, true>(x, packed, grid, scale, y, M, N, K, (hipStream_t)stream);
+    // the matrix-vector kernels' domain, with the padded size in place of N * K / 4; same choice
+    // of kernel as for row-major codes
+    if (!gemv_ok(x, packed, grid, y, M, N, K) || dmm_packed_bytes(N, K) >= (1LL << 31)) return DMM_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    if (M > 16) return launch_gemv_regx<2, 8, 2, 2, true>(x, packed, grid, scale, y, M, N, K, s);
+    if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2, true>(x, packed, grid, scale, y, M, N, K, s);
+    return launch_gemv_regx<2, 8, 1, 3, true>(x, packed, grid, scale, y, M, N, K, s);
 }
 
 int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,

@@ -107,8 +107,8 @@ int dmm_generic_f16(const void *x, const void *codes, const void *grid, float sc
  * results are bit-identical.  K % 256 == 0 is required (DMM_ERR_UNSUPPORTED otherwise).
  *   dmm_packed_bytes     size of the packed buffer (0 if the shape cannot be packed)
  *   dmm_pack_codes       codes [N, K/8] row-major -> packed; both 16-byte aligned, distinct
- *   dmm_gemv_packed_f16  the operator on packed codes; domain: that of dmm_gemv_f16 with x
- *                        resident in LDS (M = 1: K <= 28672), else DMM_ERR_UNSUPPORTED. */
+ *   dmm_gemv_packed_f16  the operator on packed codes; domain: that of dmm_gemv_f16 (M <= 32,
+ *                        N % 4 == 0, aligned pointers), else DMM_ERR_UNSUPPORTED. */
 int64_t dmm_packed_bytes(int64_t N, int64_t K);
 int dmm_pack_codes(const void *codes, void *packed, int64_t N, int64_t K, void *stream);
 int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, float scale,

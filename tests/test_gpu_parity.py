@@ -332,7 +332,8 @@ def pack_codes_numpy(codes):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 16, 256), (1, 100, 512), (1, 4096, 4096), (3, 1000, 2048), (1, 8192, 8192),
-                                   (1, 1028, 28672), (4, 11008, 4096), (8, 52, 1024)])
+                                   (1, 1028, 28672), (4, 11008, 4096), (8, 52, 1024), (16, 52, 1024), (8, 4096, 11008),
+                                   (32, 1000, 4096), (20, 36, 256)])
 def test_packed_codes_bit_identical(M, N, K):
     """dmm_pack_codes produces the documented layout, and the operator on packed codes returns
     exactly the bits of the row-major call (same arithmetic, same order) - which is itself

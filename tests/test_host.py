@@ -96,7 +96,7 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert lib.dmm_pack_codes(odd, p, 16, 512, None) == -3
     assert lib.dmm_pack_codes(None, None, 0, 512, None) == 0
     assert lib.dmm_gemv_packed_f16(p, p, p, 1.0, p, 1, 4, 16, None) == -5
-    assert lib.dmm_gemv_packed_f16(p, p, p, 1.0, p, 64, 16, 512, None) == -5
+    assert lib.dmm_gemv_packed_f16(p, p, p, 1.0, p, 64, 16, 512, None) == -5      # M too large
     # the timing hook wants both events or neither
     assert lib.dmm_set_kernel_events(p, None) == -1
     assert lib.dmm_set_kernel_events(None, None) == 0
