@@ -334,6 +334,21 @@ def prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes):
         for i in range(3):
             fn(i)
         t = timed_kernel(torch, lib, fn, 20)
+        # the same call on codes repacked offline (bit-identical result)
+        packed = [dmm.pack_codes(c) for c in codes]
+        y_pk = torch.empty_like(y)
+
+        def fn_pk(i):
+            st = lib.dmm_decode_matmul_packed_f16(x.data_ptr(), packed[i % 2].data_ptr(), grid.data_ptr(), scale,
+                                                  y_pk.data_ptr(), M, N, K, None, 0, stream)
+            assert st == 0, st
+        for i in range(3):
+            fn_pk(i)
+        t_pk = timed_kernel(torch, lib, fn_pk, 20)
+        fn(1)
+        fn_pk(1)
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_pk), "packed and row-major results differ"
         # comparison: own decode kernel -> dense half W in HBM -> library GEMM (torch.matmul)
         for i in range(3):
             W = dmm.decode(codes[i % 2], grid)
@@ -350,6 +365,8 @@ def prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes):
         tf = workload.flops(M, N, K) / t / 1e12
         rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 2), "TFLOPs": round(tf, 1),
                      "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                     "packed_kernel_us": round(t_pk * 1e6, 2),
+                     "packed_TFLOPs": round(workload.flops(M, N, K) / t_pk / 1e12, 1),
                      "decode_then_library_gemm_us": round(t_cmp * 1e6, 2),
                      "decode_then_library_gemm_TFLOPs": round(workload.flops(M, N, K) / t_cmp / 1e12, 1)})
     tot_f = sum(workload.flops(M, N, K) for K, N in workload.PREFILL)

@@ -80,7 +80,7 @@ def pack_codes(codes):
 
 def decode_matmul_packed(x, packed, grid, scale, N):
     """`decode_matmul` on codes packed by `pack_codes`; N = rows of the original code matrix.
-    Bit-identical to the row-major call.  M <= 32, N % 4 == 0."""
+    Any M; bit-identical to `decode_matmul` on the row-major codes."""
     return _C.decode_matmul_packed(x, packed, grid, float(scale), int(N))
 
 

@@ -24,6 +24,7 @@ SYMBOLS = {
     "dmm_packed_bytes": (ctypes.c_int64, [_I64, _I64]),
     "dmm_pack_codes": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
     "dmm_gemv_packed_f16": (ctypes.c_int, _OP),
+    "dmm_decode_matmul_packed_f16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _I64, _I64, _I64, _P, _I64, _P]),
     "dmm_decode_matmul_i8": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, ctypes.c_int, _P]),
     "dmm_set_kernel_events": (ctypes.c_int, [_P, _P]),
 }

@@ -1026,7 +1026,7 @@ __host__ __device__ constexpr int gr_smem_bytes(int TM) { return kSTablesBytes +
 // shorter x.  kSplit: blockIdx.z picks a contiguous share of the k tiles and the block writes
 // fp32 partial sums to part[z][M][N] instead of y (summed, scaled and rounded by
 // splitk_reduce_kernel), so that short x still fills the chip with workgroups.
-template <int TM, bool kSplit>
+template <int TM, bool kSplit, bool kPacked>
 __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restrict__ x,
                                                        const uint16_t *__restrict__ codes,
                                                        const void *__restrict__ grid, float scale,
@@ -1071,15 +1071,21 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     // of the k tile.  x: load p of thread tid is piece tid % 8 (16 bytes) of row 32 p + tid / 8, so
     // that 8 lanes cover one 128-byte line.  Both as raw buffer
     // loads: rows past N / M and tiles past the end get zeros without a memory access.
+    // Packed codes (pack_kernel): the 16 bytes of (row, k tile) sit at
+    // (((row / 16) * (K / 256) + kt / 4) * 64 + (kt % 4) * 16 + row % 16) * 16, so the per-tile part
+    // of the offset is kt * 256 and a wave's load is two runs of 256 consecutive bytes instead
+    // of 32 pieces of 16.
+    const int n_pad = ((N + 15) >> 4) << 4;
     const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_pad : N) * row_bytes), 0x00020000);
     const __amdgpu_buffer_rsrc_t xrsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, (int)((int64_t)M * K * 2), 0x00020000);
     int cvoff[kGrTN];
 #pragma unroll
     for (int i = 0; i < kGrTN; i++) {
         const int n = n0 + wave * 64 + i * 32 + l32;
-        cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
+        if (kPacked) cvoff[i] = n < n_pad ? (n >> 4) * (K >> 8) * 1024 + (n & 15) * 16 + kq * 8 : kOut;
+        else cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
     }
     // rows r and r + 8 share a group of 16 lanes: with the 144-byte pitch their 16 pieces fall in
     // 16 different bank groups, so the LDS writes below are conflict-free like the fragment reads
@@ -1096,7 +1102,7 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         u4_t xv[TM];
     };
     auto load_codes = [&](Stage &st, int kt) {   // kt counts this block's tiles
-        const int coff = kt < k_tiles ? (kt_lo + kt) * 16 : kOut;
+        const int coff = kt < k_tiles ? (kt_lo + kt) * (kPacked ? 256 : 16) : kOut;
 #pragma unroll
         for (int i = 0; i < kGrTN; i++) st.cw[i] = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
     };
@@ -1545,14 +1551,14 @@ int launch_gemm(const void *x, const void *codes, const void *grid, float scale,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
 }
 
-template <int TM, bool kSplit>
+template <int TM, bool kSplit, bool kPacked>
 int launch_gemm_reg_tm(const void *x, const void *codes, const void *grid, float scale, void *y, float *part,
                        int64_t M, int64_t N, int64_t K, int splits, hipStream_t stream)
 {
     static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemm_reg_kernel<TM, kSplit>, gr_smem_bytes(TM), attr_done)) return e;
+    if (int e = allow_dynamic_lds(gemm_reg_kernel<TM, kSplit, kPacked>, gr_smem_bytes(TM), attr_done)) return e;
     dim3 g((unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)((N + kGrBN - 1) / kGrBN), (unsigned)splits);
-    return launch<true, !kSplit>(gemm_reg_kernel<TM, kSplit>, g, dim3(256), gr_smem_bytes(TM), stream,
+    return launch<true, !kSplit>(gemm_reg_kernel<TM, kSplit, kPacked>, g, dim3(256), gr_smem_bytes(TM), stream,
                                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, part, (int)M,
                                  (int)N, (int)K, splits);
 }
@@ -1560,13 +1566,14 @@ int launch_gemm_reg_tm(const void *x, const void *codes, const void *grid, float
 // rows of x per block: 32, 64 or 128
 inline int gemm_reg_tm(int64_t M) { return M <= 32 ? 1 : M <= 64 ? 2 : 4; }
 
+template <bool kPacked = false>
 int launch_gemm_reg(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                     int64_t N, int64_t K, hipStream_t stream)
 {
     switch (gemm_reg_tm(M)) {
-        case 1: return launch_gemm_reg_tm<1, false>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
-        case 2: return launch_gemm_reg_tm<2, false>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
-        default: return launch_gemm_reg_tm<4, false>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+        case 1: return launch_gemm_reg_tm<1, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+        case 2: return launch_gemm_reg_tm<2, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+        default: return launch_gemm_reg_tm<4, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
     }
 }
 
@@ -1586,15 +1593,16 @@ int splitk_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes)
     return splits < 2 ? 1 : (int)splits;
 }
 
+template <bool kPacked = false>
 int launch_gemm_splitk(const void *x, const void *codes, const void *grid, float scale, void *y, void *workspace,
                        int splits, int64_t M, int64_t N, int64_t K, hipStream_t stream)
 {
     float *part = reinterpret_cast<float *>(workspace);
     int st;
     switch (gemm_reg_tm(M)) {
-        case 1: st = launch_gemm_reg_tm<1, true>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
-        case 2: st = launch_gemm_reg_tm<2, true>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
-        default: st = launch_gemm_reg_tm<4, true>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+        case 1: st = launch_gemm_reg_tm<1, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+        case 2: st = launch_gemm_reg_tm<2, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+        default: st = launch_gemm_reg_tm<4, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
     }
     if (st != 0) return st;
     const int64_t mn = M * N;
@@ -1777,6 +1785,28 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
     if (M > 16) return launch_gemv_regx<2, 8, 2, 2, true>(x, packed, grid, scale, y, M, N, K, s);
     if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2, true>(x, packed, grid, scale, y, M, N, K, s);
     return launch_gemv_regx<2, 8, 1, 3, true>(x, packed, grid, scale, y, M, N, K, s);
+}
+
+int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *grid, float scale, void *y,
+                                 int64_t M, int64_t N, int64_t K, void *workspace, int64_t workspace_bytes,
+                                 void *stream)
+{
+    int st = check_common(x, packed, grid, y, M, N, K);
+    if (st != DMM_OK || M == 0 || N == 0) return st;
+    if (workspace_bytes < 0) return DMM_ERR_BAD_SHAPE;
+    if (workspace && workspace_bytes > 0 && !aligned(workspace, 16)) return DMM_ERR_MISALIGNED;
+    const int64_t pbytes = dmm_packed_bytes(N, K);
+    if (pbytes == 0 || pbytes >= (1LL << 31)) return DMM_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const bool mm_ok = gemm_ok(x, packed, grid, y, M, N, K) && gemm_reg_ok(M, ((N + 15) / 16) * 16, K);
+    if (workspace && workspace_bytes > 0 && mm_ok && M >= splitk_min_m() && aligned(y, 8)) {
+        const int splits = splitk_plan(M, N, K, workspace_bytes);
+        if (splits >= 2) return launch_gemm_splitk<true>(x, packed, grid, scale, y, workspace, splits, M, N, K, s);
+    }
+    if (gemv_ok(x, packed, grid, y, M, N, K))
+        return dmm_gemv_packed_f16(x, packed, grid, scale, y, M, N, K, stream);
+    if (mm_ok) return launch_gemm_reg<true>(x, packed, grid, scale, y, M, N, K, s);
+    return DMM_ERR_UNSUPPORTED;
 }
 
 int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,

@@ -157,11 +157,15 @@ torch::Tensor decode_matmul_packed(torch::Tensor x, torch::Tensor packed, torch:
     c10::DeviceGuard guard(x.device());
     torch::Tensor y = torch::empty({M, N}, x.options().requires_grad(false));
     hipStream_t stream = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+    torch::Tensor workspace;
+    const int64_t ws_bytes = dmm_workspace_bytes(M, N, K);
+    if (ws_bytes > 0) workspace = torch::empty({ws_bytes}, x.options().dtype(torch::kUInt8).requires_grad(false));
     int st;
     {
         pybind11::gil_scoped_release nogil;
-        st = dmm_gemv_packed_f16(x.data_ptr(), packed.data_ptr(), grid.data_ptr(), static_cast<float>(scale),
-                                 y.data_ptr(), M, N, K, stream);
+        st = dmm_decode_matmul_packed_f16(x.data_ptr(), packed.data_ptr(), grid.data_ptr(), static_cast<float>(scale),
+                                          y.data_ptr(), M, N, K, ws_bytes > 0 ? workspace.data_ptr() : nullptr,
+                                          ws_bytes, stream);
     }
     check_status(st, "decode_matmul_packed");
     return y;
@@ -211,7 +215,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           pybind11::arg("x"), pybind11::arg("weights_compressed"), pybind11::arg("codebook_abs"),
           pybind11::arg("tiled") = true);
     m.def("pack_codes", &pack_codes, "codes [N, K/8] -> the batch-1 kernel's packed layout", pybind11::arg("codes"));
-    m.def("decode_matmul_packed", &decode_matmul_packed, "decode_matmul on packed codes (small M, K % 256 == 0)",
+    m.def("decode_matmul_packed", &decode_matmul_packed, "decode_matmul on packed codes (K % 256 == 0)",
           pybind11::arg("x"), pybind11::arg("packed"), pybind11::arg("grid"), pybind11::arg("scale"), pybind11::arg("N"));
     m.def("decode", &decode, "Decode codes [N, K/8] to the dense half matrix [N, K]",
           pybind11::arg("codes"), pybind11::arg("grid"));

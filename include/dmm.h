@@ -107,10 +107,20 @@ int dmm_generic_f16(const void *x, const void *codes, const void *grid, float sc
  * results are bit-identical.  K % 256 == 0 is required (DMM_ERR_UNSUPPORTED otherwise).
  *   dmm_packed_bytes     size of the packed buffer (0 if the shape cannot be packed)
  *   dmm_pack_codes       codes [N, K/8] row-major -> packed; both 16-byte aligned, distinct
- *   dmm_gemv_packed_f16  the operator on packed codes; domain: that of dmm_gemv_f16 (M <= 32,
- *                        N % 4 == 0, aligned pointers), else DMM_ERR_UNSUPPORTED. */
+ *   dmm_decode_matmul_packed_f16  the operator on packed codes, any M: the matrix-vector
+ *                        kernels for M <= 32, the register-operand MFMA kernel above (its code
+ *                        loads become two runs of 256 consecutive bytes per wave), split-K when
+ *                        a workspace is given (same rules as dmm_decode_matmul_ws_f16; NULL, 0
+ *                        for none).  16-byte aligned x, packed, grid; DMM_ERR_UNSUPPORTED for
+ *                        what the packed kernels do not cover (K % 256, unaligned pointers,
+ *                        packed size of 2 GiB or more).
+ *   dmm_gemv_packed_f16  explicit matrix-vector path on packed codes; domain: that of
+ *                        dmm_gemv_f16 (M <= 32, N % 4 == 0, aligned pointers). */
 int64_t dmm_packed_bytes(int64_t N, int64_t K);
 int dmm_pack_codes(const void *codes, void *packed, int64_t N, int64_t K, void *stream);
+int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *grid, float scale,
+                                 void *y, int64_t M, int64_t N, int64_t K, void *workspace,
+                                 int64_t workspace_bytes, void *stream);
 int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, float scale,
                         void *y, int64_t M, int64_t N, int64_t K, void *stream);
 

@@ -358,7 +358,38 @@ def test_packed_codes_bit_identical(M, N, K):
     # the PyTorch wrappers
     pk = dmm.pack_codes(cd)
     assert torch.equal(pk.reshape(-1), packed)
-    assert torch.equal(dmm.decode_matmul_packed(xd, pk, gd, scale, N), y)
+    # (the operators bring a workspace, so for 17 <= M they split K: compare like with like)
+    assert torch.equal(dmm.decode_matmul_packed(xd, pk, gd, scale, N), dmm.decode_matmul(xd, cd, gd, scale))
+
+
+@pytest.mark.parametrize("M,N,K", [(40, 300, 512), (64, 1024, 1024), (200, 771, 2304), (2048, 4096, 4096),
+                                   (130, 52, 256), (33, 4100, 1024)])
+def test_packed_codes_matrix_matrix_bit_identical(M, N, K):
+    """The MFMA kernel on packed codes, with and without a split-K workspace: the bits of the
+    row-major calls."""
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=N + K + M)
+    xd, cd, gd = dev(x), dev(codes), dev(grid)
+    lib = capi.lib()
+    pk = dmm.pack_codes(cd)
+    stream = torch.cuda.current_stream().cuda_stream
+    y_ref = c_matmul(xd, cd, gd, scale, "gemm")
+    y = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
+    capi.check("dmm_decode_matmul_packed_f16",
+               lib.dmm_decode_matmul_packed_f16(xd.data_ptr(), pk.data_ptr(), gd.data_ptr(), scale, y.data_ptr(),
+                                                M, N, K, None, 0, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_ref)
+    y_ws_ref, want = c_matmul_ws(xd, cd, gd, scale)
+    ws = torch.empty(max(want, 16), dtype=torch.uint8, device=DEV)
+    y2 = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
+    capi.check("dmm_decode_matmul_packed_f16",
+               lib.dmm_decode_matmul_packed_f16(xd.data_ptr(), pk.data_ptr(), gd.data_ptr(), scale, y2.data_ptr(),
+                                                M, N, K, ws.data_ptr(), want, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y_ws_ref)
+    assert torch.equal(dmm.decode_matmul_packed(xd, pk, gd, scale, N), y_ws_ref)
+    ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+    assert_close_to_oracle(y, ref, "packed gemm M=%d N=%d K=%d" % (M, N, K))
 
 
 # ----------------------------------------------------------------- split-K with a workspace

@@ -97,6 +97,11 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert lib.dmm_pack_codes(None, None, 0, 512, None) == 0
     assert lib.dmm_gemv_packed_f16(p, p, p, 1.0, p, 1, 4, 16, None) == -5
     assert lib.dmm_gemv_packed_f16(p, p, p, 1.0, p, 64, 16, 512, None) == -5      # M too large
+    pkf = lib.dmm_decode_matmul_packed_f16
+    assert pkf(p, p, p, 1.0, p, 64, 16, 520, None, 0, None) == -5                 # K % 256 != 0
+    assert pkf(p, p, p, 1.0, p, 64, 16, 512, ctypes.c_void_p(p.value + 8), 64, None) == -3
+    assert pkf(p, p, p, 1.0, p, 64, 16, 12, None, 0, None) == -2
+    assert pkf(None, None, None, 1.0, None, 0, 16, 512, None, 0, None) == 0
     # the timing hook wants both events or neither
     assert lib.dmm_set_kernel_events(p, None) == -1
     assert lib.dmm_set_kernel_events(None, None) == 0
