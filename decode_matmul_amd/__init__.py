@@ -10,8 +10,10 @@ in the half-precision form of the same code format:
     W = decode(codes, grid)                       # dense half [N,K], bit-exact decode
 
 The functions are the compiled PyTorch operator (`_C`, host C++) over the C ABI of
-`libdmm.so` (hand-written HIP).  There is no CPU implementation: importing this package
-without the built extension raises, and calling the operator with CPU tensors raises.
+`libdmm.so` (hand-written HIP).  There is no CPU implementation: without the built extension
+every operator raises ImportError (the import itself succeeds, so that
+`python -m decode_matmul_amd.build` can run on a fresh tree), and calling the operator with
+CPU tensors raises.
 """
 import os as _os
 
@@ -21,13 +23,26 @@ EXT_PATH = _os.path.join(_PKG_DIR, "_C.so")
 
 import torch as _torch  # noqa: E402  (loads the HIP runtime the extension links against)
 
-if not (_os.path.exists(LIB_PATH) and _os.path.exists(EXT_PATH)):
-    raise ImportError(
-        "decode_matmul_amd: native libraries are not built (%s, %s); run "
-        "`python -m decode_matmul_amd.build`" % (LIB_PATH, EXT_PATH)
-    )
+_C = None
 
-from . import _C  # noqa: E402
+
+def _ext():
+    """The compiled operator module; loaded on first use, ImportError if it is not built."""
+    global _C
+    if _C is None:
+        if not (_os.path.exists(LIB_PATH) and _os.path.exists(EXT_PATH)):
+            raise ImportError(
+                "decode_matmul_amd: native libraries are not built (%s, %s); run "
+                "`python -m decode_matmul_amd.build`" % (LIB_PATH, EXT_PATH)
+            )
+        import importlib
+        _C = importlib.import_module("._C", __name__)
+    return _C
+
+
+if _os.path.exists(LIB_PATH) and _os.path.exists(EXT_PATH):
+    _ext()
+
 from .capi import lib  # noqa: E402,F401
 from .codebook import (  # noqa: E402,F401
     build_codebook_abs,
@@ -55,35 +70,35 @@ def decode_matmul(x, codes, grid, scale):
     """y[M,N] = half(scale * x @ decode(codes, grid).T), fp32 accumulation, on x's device and
     the current stream, asynchronously.  Same role as the reference's `decode_matmul`
     (decode_matmul_cuda.cu:178-234); raises RuntimeError on bad inputs like its TORCH_CHECKs."""
-    return _C.decode_matmul(x, codes, grid, float(scale))
+    return _ext().decode_matmul(x, codes, grid, float(scale))
 
 
 def decode_matmul_path(x, codes, grid, scale, path="auto"):
     """decode_matmul through one named kernel path: "auto", "gemv", "gemm" or "generic".
     A path asked for outside its domain raises instead of falling back."""
-    return _C.decode_matmul_path(x, codes, grid, float(scale), path)
+    return _ext().decode_matmul_path(x, codes, grid, float(scale), path)
 
 
 def decode_matmul_int8(x, weights_compressed, codebook_abs, tiled=True):
     """The reference's operator with its own dtypes: int8 x [M,K], int16 codes [N,K/8], int64[256]
     table -> int32 [M,N] (decode_matmul_cuda.cu:178-234).  tiled=True: codes as the reference's
     kernel reads them (`transpose_tile`, test_decode_matmul.py:101-109); False: row-major."""
-    return _C.decode_matmul_int8(x, weights_compressed, codebook_abs, bool(tiled))
+    return _ext().decode_matmul_int8(x, weights_compressed, codebook_abs, bool(tiled))
 
 
 def pack_codes(codes):
     """Offline repack of codes [N, K/8] (K % 256 == 0) for the batch-1 kernel: each wave's load
     becomes 1 KB of consecutive bytes.  The counterpart of the reference's `transpose_tile`
     (test_decode_matmul.py:101-109).  Returns [ceil(N/16)*16, K/8], same dtype."""
-    return _C.pack_codes(codes)
+    return _ext().pack_codes(codes)
 
 
 def decode_matmul_packed(x, packed, grid, scale, N):
     """`decode_matmul` on codes packed by `pack_codes`; N = rows of the original code matrix.
     Any M; bit-identical to `decode_matmul` on the row-major codes."""
-    return _C.decode_matmul_packed(x, packed, grid, float(scale), int(N))
+    return _ext().decode_matmul_packed(x, packed, grid, float(scale), int(N))
 
 
 def decode(codes, grid):
     """Dense half matrix W[N,K] from codes[N,K/8]; W[n, 8j+d] is dim d of codes[n, j]."""
-    return _C.decode(codes, grid)
+    return _ext().decode(codes, grid)

@@ -397,11 +397,10 @@ __device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr,
 }
 
 template <int R, int W, int D, bool kPacked>
-__global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__restrict__ x,
-                                                             const uint16_t *__restrict__ codes,
-                                                             const void *__restrict__ grid, float scale,
-                                                             uint16_t *__restrict__ y, int M, int N, int K,
-                                                             int tiles_q, int tiles_r)
+__device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x, const uint16_t *__restrict__ codes,
+                                                 const void *__restrict__ grid, float scale,
+                                                 uint16_t *__restrict__ y, int M, int N, int K, int tiles_q,
+                                                 int tiles_r)
 {
     static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
@@ -576,6 +575,423 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
     }
     DMM_TRACE_MARK(7);
     DMM_TRACE_DUMP();
+}
+
+template <int R, int W, int D, bool kPacked>
+__global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__restrict__ x,
+                                                             const uint16_t *__restrict__ codes,
+                                                             const void *__restrict__ grid, float scale,
+                                                             uint16_t *__restrict__ y, int M, int N, int K,
+                                                             int tiles_q, int tiles_r)
+{
+    gemv_stream_body<R, W, D, kPacked>(x, codes, grid, scale, y, M, N, K, tiles_q, tiles_r);
+}
+
+// ------------------------------------------------------------------ streaming matrix-vector path, 8-bit operands
+// The streaming kernel above is bound by the LDS: two 16-byte table gathers per code.  When
+// every grid value is exactly representable in 8 bits (fp8 e4m3: 4 significant bits - the E8P
+// grid of half-odd values is), the same product can be formed with 8-byte gathers, which the
+// LDS serves at twice the rate, by running the matrix unit on 8-bit operands:
+//   * weights.  w = s g + d, s = +-1 per dim, d = +-1/4 per code.  The grid table holds rows of
+//     8 fp8 bytes, the sign table rows of 8 flag bytes (0x80 = flipped); one exclusive or per
+//     4 weights applies the signs, and the 8 bytes of a code are the A operand of
+//     v_mfma_f32_16x16x32_fp8_bf8 as they are.  d is left out of the decode and added by the
+//     matrix unit instead: sum_k d x[k] = sum over codes of (8 d) * (mean of the code's 8 x
+//     values), one more MFMA per 16 rows x 256 k whose A operand is +-2.0 per code, made from
+//     the code words themselves (shift bit = sign bit of the byte);
+//   * x.  A half with a zero low byte IS a bf8 (e5m2) number in its high byte.  Cutting x after
+//     its top byte, subtracting, scaling what is left by 8 and repeating gives
+//     x = t0 + t1 / 8 + t2 / 64 + t3 / 512 exactly for every normal x (3 significant bits per
+//     term, 11 in a half); the four terms sit in four B columns - at batch 1 the other 15
+//     columns of the 16-wide tile are idle anyway - and the four result columns are added, with
+//     those weights, at the end.  The per-code means (fp32 sum of 8, times 1/8, rounded to
+//     half) are split the same way.
+// s g + d is exact in half for every fp8 g and the terms of x add up to x (subnormal x may lose
+// bits below 2^-24 * 4), so nothing is lost in the operands; what differs from the 16-bit kernel is the matrix unit's own arithmetic: the
+// 8-bit MFMA adds each group of products in an adder narrower than fp32 (small products lose
+// low bits against the largest of the group) and the means are rounded to half.  Measured
+// against the fp64 reference the error is about 2^-14 of a row's scale (1.5 half ulps at the
+// 99th percentile on the benchmark's inputs, where the 16-bit kernel stays below the 0.5 ulp of
+// the output rounding) - a hundredth of the operator's tolerance of 1e-2.  A grid with a value fp8 cannot hold is found
+// while the table is built (convert, convert back, compare), an x that is not finite while it
+// is split; every workgroup then runs the 16-bit kernel above instead: same launch, same
+// result as that kernel gives.
+// LDS map: [0, 32K) sign rows (128 x 32 copies x 8 B), [32K, 96K) grid rows (256 x 32 copies x
+// 8 B; a lane reads copy lane % 32, conflict-free for any codes), partial sums, then the terms
+// of x (column m * 4 + t, pitch K + 16 bytes) and of the means (pitch K / 8 + 16).
+typedef __attribute__((address_space(3))) const u2_t lds_u2_t;
+__device__ __forceinline__ u2_t lds_read8(uint32_t byte_addr)
+{
+    return *reinterpret_cast<lds_u2_t *>(byte_addr);
+}
+
+// terms of x, terms of the means, and one word per wave for the vote on the grid
+__host__ __device__ constexpr int64_t q8_x_bytes(int64_t M, int64_t K) { return 4 * M * (K + 16) + 4 * M * (K / 8 + 16) + 64; }
+
+// the 8 sign flags of a sign-row index as bytes: dims 0-3 in [0], 4-7 in [1]
+__device__ __forceinline__ u2_t sign_bytes(uint32_t s7)
+{
+    const uint32_t s8 = s7 | ((__builtin_popcount(s7) & 1u) << 7);
+    u2_t r;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t n = (s8 >> (4 * i)) & 0xFu;
+        r[i] = ((n & 1u) << 7) | ((n & 2u) << 14) | ((n & 4u) << 21) | ((n & 8u) << 28);
+    }
+    return r;
+}
+
+// a grid row as 8 fp8 bytes; exact: every value survives the round trip
+__device__ __forceinline__ u2_t grid_row_fp8(const u4_t &row, bool &exact)
+{
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const h2_t h = as_h2(row[i]);
+        f[2 * i] = (float)h[0];
+        f[2 * i + 1] = (float)h[1];
+    }
+    u2_t r;
+    exact = true;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * i], f[4 * i + 1], 0, false);
+        p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * i + 2], f[4 * i + 3], p, true);
+        r[i] = (uint32_t)p;
+        exact = exact && __builtin_amdgcn_cvt_f32_fp8(p, 0) == f[4 * i] && __builtin_amdgcn_cvt_f32_fp8(p, 1) == f[4 * i + 1] &&
+                __builtin_amdgcn_cvt_f32_fp8(p, 2) == f[4 * i + 2] && __builtin_amdgcn_cvt_f32_fp8(p, 3) == f[4 * i + 3];
+    }
+    return r;
+}
+
+// One half (bits) as four bf8 bytes t0..t3 (byte t of the result) with
+// h = t0 + t1 / 8 + t2 / 64 + t3 / 512: a term is the top byte of what is left, and what is left
+// after it is scaled by 8 (exact, and it keeps the remainder as far above the subnormal range
+// as h itself was), so every normal h is split without loss.  Non-finite h: t0 alone carries it.
+__device__ __forceinline__ uint32_t split_half_bf8(uint16_t bits)
+{
+    uint32_t out = 0;
+    uint16_t r = bits;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const uint16_t hi = r & 0xFF00u;
+        out |= (uint32_t)(hi >> 8) << (8 * t);
+        if ((bits & 0x7C00u) == 0x7C00u) break;
+        r = __builtin_bit_cast(uint16_t, (half_t)((__builtin_bit_cast(half_t, r) - __builtin_bit_cast(half_t, hi)) * (half_t)8.0f));
+    }
+    return out;
+}
+
+// 8 halves (one 16-byte piece of x) as four terms of 8 bf8 bytes each.  Returns whether all
+// 8 are finite; if not, the terms still add up for the finite ones and t0 alone carries the
+// others (the caller hands the launch to the 16-bit kernel anyway: an infinity must meet the
+// whole weight, not its two terms one after the other).
+__device__ __forceinline__ bool split_piece_bf8(const u4_t &v, u2_t (&t)[4])
+{
+    bool finite = true;
+#pragma unroll
+    for (int i = 0; i < 4; i++) finite = finite && (v[i] & 0x7C00u) != 0x7C00u && (v[i] & 0x7C000000u) != 0x7C000000u;
+    if (__builtin_expect(finite, 1)) {
+        u4_t r = v;
+#pragma unroll
+        for (int term = 0; term < 4; term++) {
+            const u4_t hi = r & 0xFF00FF00u;
+            t[term][0] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07050301u);   // the high bytes of halves 0..3
+            t[term][1] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07050301u);   // and of halves 4..7
+            if (term < 3) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) r[i] = as_u32((as_h2(r[i]) - as_h2(hi[i])) * h2_t{(half_t)8.0f, (half_t)8.0f});
+            }
+        }
+    } else {
+        uint32_t b[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            b[2 * i] = split_half_bf8((uint16_t)(v[i] & 0xFFFFu));
+            b[2 * i + 1] = split_half_bf8((uint16_t)(v[i] >> 16));
+        }
+#pragma unroll
+        for (int term = 0; term < 4; term++) {
+            t[term][0] = t[term][1] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                t[term][0] |= ((b[e] >> (8 * term)) & 0xFFu) << (8 * e);
+                t[term][1] |= ((b[4 + e] >> (8 * term)) & 0xFFu) << (8 * e);
+            }
+        }
+    }
+    return finite;
+}
+
+// mean of the 8 halves of a piece (fp32 sum in a fixed order), as a half
+__device__ __forceinline__ uint16_t piece_mean(const u4_t &v)
+{
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const h2_t h = as_h2(v[i]);
+        sum += (float)h[0];
+        sum += (float)h[1];
+    }
+    return __builtin_bit_cast(uint16_t, (half_t)(sum * 0.125f));
+}
+
+struct Q8Gather {
+    u2_t g0, s0, g1, s1;
+};
+
+// lane_base = (lane % 32) * 8; the tables start at LDS address 0
+__device__ __forceinline__ void q8_gather(Q8Gather &o, uint32_t w, uint32_t lane_base)
+{
+    const uint32_t w7 = w & 0x7FFF7FFFu;                 // sign-row index must not see the shift bit
+    o.g0 = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u) + kSSignBytes);
+    o.s0 = lds_read8(__builtin_amdgcn_perm(w7, lane_base, 0x0C0C0500u));
+    o.g1 = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u) + kSSignBytes);
+    o.s1 = lds_read8(__builtin_amdgcn_perm(w7, lane_base, 0x0C0C0700u));
+}
+
+__device__ __forceinline__ long q8_pack(uint32_t lo, uint32_t hi)
+{
+    return (long)(((unsigned long)hi << 32) | (unsigned long)lo);
+}
+
+// One 256-wide k step for the first nv (uniform, 1 <= nv <= R) of R row tiles; same item order
+// as stream_step.  xaddr: this lane's x terms of the step (16 bytes per word pair: the B
+// operands of its two codes), x8addr: its 8 means.
+template <int R>
+__device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t x8addr, uint32_t lane_base,
+                                        f4_t (&acc)[R][2], int nv)
+{
+    constexpr int kItems = 4 * R;
+    Q8Gather buf[2];
+    u4_t xb[2];
+    xb[0] = lds_read16(xaddr);
+    q8_gather(buf[0], cw[0][0], lane_base);
+    const u2_t x8 = lds_read8(x8addr);
+#pragma unroll
+    for (int i = 0; i < kItems; i++) {
+        const int t2 = i / R, r = i % R;
+        if (i + 1 < kItems) {
+            const int nt2 = (i + 1) / R, nr = (i + 1) % R;
+            if (nr == 0) {
+                xb[nt2 & 1] = lds_read16(xaddr + nt2 * 16);
+                q8_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base);
+            } else if (nr < nv) {
+                q8_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base);
+            }
+        }
+        if (r == 0 || r < nv) {
+            const Q8Gather &b = buf[i & 1];
+            const u4_t &xv = xb[t2 & 1];
+            acc[r][0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(b.g0[0] ^ b.s0[0], b.g0[1] ^ b.s0[1]),
+                                                                   q8_pack(xv[0], xv[1]), acc[r][0], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            acc[r][1] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(b.g1[0] ^ b.s1[0], b.g1[1] ^ b.s1[1]),
+                                                                   q8_pack(xv[2], xv[3]), acc[r][1], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (t2 == 3) {
+                // the shift term: byte order of the A operand is codes 0, 2, 1, 3 | 4, 6, 5, 7 of the
+                // lane's eight (bit 15 of a word lands in byte 1 or, shifted, byte 0; bit 31 in
+                // byte 3 or byte 2) - the means are stored in the same order
+                const uint32_t a8lo = ((cw[r][0] >> 8) & 0x00800080u) | (cw[r][1] & 0x80008000u) | 0x40404040u;
+                const uint32_t a8hi = ((cw[r][2] >> 8) & 0x00800080u) | (cw[r][3] & 0x80008000u) | 0x40404040u;
+                acc[r][0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]),
+                                                                       acc[r][0], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+}
+
+template <int R, int W, int D, bool kPacked>
+__global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restrict__ x,
+                                                         const uint16_t *__restrict__ codes,
+                                                         const void *__restrict__ grid, float scale,
+                                                         uint16_t *__restrict__ y, int M, int N, int K,
+                                                         int tiles_q, int tiles_r)
+{
+    static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
+    static_assert(W == 16, "the table staging below assumes 1024 threads");
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
+    f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // [2][W][R][4 * M]
+    const int red_par = W * R * 4 * M;                                 // float4 per parity
+    unsigned char *xt = smem_raw + kSTablesBytes + stream_red_bytes(R, W, M);
+    const int xt_pitch = K + 16, x8_pitch = (K >> 3) + 16;
+    unsigned char *x8t = xt + 4 * M * xt_pitch;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c16 = lane & 15;
+    const int q = lane >> 4;
+    const int n_steps = K >> 8;
+    const int row_bytes = K >> 2;
+    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;
+
+    // ---- prologue, in the order of the 16-bit kernel: grid row and x first, then the code
+    // stream, then the tables and the terms of x while the code loads fly --------------------
+    const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid & 255];
+    const int row_chunks = K >> 3;                     // 16-byte pieces per row of x
+    constexpr int kXPer = 2;                           // pieces of row 0 per thread fetched up front
+    u4_t xv[kXPer];
+#pragma unroll
+    for (int u = 0; u < kXPer; u++) {
+        const int c = u * 64 * W + tid;
+        xv[u] = c < row_chunks ? reinterpret_cast<const u4_t *>(x)[c] : u4_t{0u, 0u, 0u, 0u};
+    }
+
+    const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;   // k steps of this wave per row block
+    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
+    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
+    const int nb_wg = (t1 - t0 + R - 1) / R;
+
+    const int n_tiles_all = (N + 15) >> 4;
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_tiles_all * 16 : N) * row_bytes), 0x00020000);
+    int voff[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) voff[r] = kPacked ? lane * 16 + r * n_steps * 1024 : (16 * r + c16) * row_bytes + q * 16;
+    constexpr int kOut = (int)0x80000000;
+    int pf_blk = 0, pf_j = 0;
+    auto issue = [&](u4_t (&cwd)[R]) {
+        const bool ok = pf_blk < nb_wg && n_sw > 0;
+        const int tb = t0 + pf_blk * R;
+        const int soff = !ok ? kOut
+                         : kPacked ? (tb * n_steps + wave + pf_j * W) * 1024
+                                   : tb * 16 * row_bytes + (wave + pf_j * W) * 64;
+#pragma unroll
+        for (int r = 0; r < R; r++)   // tiles of a partial block that belong to the next workgroup: no access
+            cwd[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], (r == 0 || tb + r < t1) ? soff : kOut, 0);
+        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
+    };
+
+    u4_t cw[D][R];
+#pragma unroll
+    for (int d = 0; d < D; d++) issue(cw[d]);
+
+    // sign rows: 2048 slots of 16 bytes (two copies each), two per thread
+    {
+        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const u2_t sb = sign_bytes((uint32_t)((tid + i * 1024) >> 4));
+            sg[tid + i * 1024] = u4_t{sb[0], sb[1], sb[0], sb[1]};
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // keep the sign rows ahead of the waits for the loads
+
+    // x -> its four terms, and the means of every 8 values -> theirs
+    bool fits = true;   // stays true while x is finite and (below) the grid fits fp8
+    auto stage_piece = [&](const u4_t &v, int m, int c) {
+        u2_t t[4];
+        fits = split_piece_bf8(v, t) && fits;
+        const uint32_t mb = split_half_bf8(piece_mean(v));
+        const int c8 = (c & ~3) | ((c & 1) << 1) | ((c >> 1) & 1);   // codes 0, 2, 1, 3 of each four
+#pragma unroll
+        for (int term = 0; term < 4; term++) {
+            *reinterpret_cast<u2_t *>(xt + (m * 4 + term) * xt_pitch + c * 8) = t[term];
+            x8t[(m * 4 + term) * x8_pitch + c8] = (unsigned char)(mb >> (8 * term));
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < kXPer; u++) {
+        const int c = u * 64 * W + tid;
+        if (c < row_chunks) stage_piece(xv[u], 0, c);
+    }
+    for (int c = kXPer * 64 * W + tid; c < row_chunks; c += 64 * W) stage_piece(reinterpret_cast<const u4_t *>(x)[c], 0, c);
+    for (int m = 1; m < M; m++)
+        for (int c = tid; c < row_chunks; c += 64 * W) stage_piece(reinterpret_cast<const u4_t *>(x + (int64_t)m * K)[c], m, c);
+
+    // grid rows: thread tid converts row tid % 256 and writes 4 of its 16 slots (two copies each)
+    {
+        bool exact;
+        const u2_t g8 = grid_row_fp8(grow, exact);
+        fits = fits && exact;
+        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes);
+        const int row = tid & 255, c0 = (tid >> 8) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; i++) gg[row * 16 + ((c0 + i + tid) & 15)] = u4_t{g8[0], g8[1], g8[0], g8[1]};
+    }
+    // the vote: every wave publishes whether one of its rows or pieces failed, in a word of its own (so
+    // nothing needs clearing first), and after the barrier every wave reads all of them
+    uint32_t *votes = reinterpret_cast<uint32_t *>(x8t + 4 * M * x8_pitch);
+    const bool wave_bad = __builtin_amdgcn_ballot_w64(!fits) != 0;
+    if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
+    __syncthreads();
+    if (__builtin_amdgcn_ballot_w64(votes[lane & (W - 1)] != 0) != 0) {
+        // a grid value does not fit 8 bits, or x is not finite: the 16-bit kernel takes over (it
+        // builds its own tables)
+        gemv_stream_body<R, W, 2, kPacked>(x, codes, grid, scale, y, M, N, K, tiles_q, tiles_r);
+        return;
+    }
+
+    // B operand addresses of this lane: column c16 = 4 m + term (column 0 for the idle ones)
+    const int col = c16 < 4 * M ? c16 : 0;
+    const uint32_t xlane = lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64);
+    const uint32_t x8lane = lds_addr(x8t) + (uint32_t)(col * x8_pitch + q * 8);
+
+    f4_t acc[R][2];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+    const float term_weight = __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)(c16 & 3) * 3u << 23));   // 8^-(c16 % 4)
+
+    auto finish_block = [&](int blk) {
+        f4_t *rp = red + (blk & 1) * red_par;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            // the four term columns of an x row are added first, each with the weight of its term:
+            // lane 4 m gets columns 4 m .. 4 m + 3
+            f4_t v = (acc[r][0] + acc[r][1]) * term_weight;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                v[e] = dpp_shr_add<0x101>(v[e]);   // row_shl:1
+                v[e] = dpp_shr_add<0x102>(v[e]);   // row_shl:2
+            }
+            if ((c16 & 3) == 0 && c16 < 4 * M) rp[(wave * R + r) * 4 * M + q * M + (c16 >> 2)] = v;
+            acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+        }
+        __syncthreads();
+        for (int p = wave; p < R * M; p += W) {
+            const int r = M == 1 ? p : p / M, m = p - r * M;
+            f4_t v = f4_t{0.f, 0.f, 0.f, 0.f};
+            if (c16 < W) v = rp[(c16 * R + r) * 4 * M + q * M + m];
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
+            const int tile = t0 + blk * R + r;
+            const int n = tile * 16 + 4 * q;
+            if (c16 == 15 && tile < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
+                h4_t o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
+                *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
+            }
+        }
+    };
+
+    if (n_sw == 0) {
+        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
+        return;
+    }
+
+    const int n_items = nb_wg * n_sw;
+    int blk = 0, j = 0;
+    for (int i0 = 0; i0 < n_items; i0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (i0 + d < n_items) {
+                const uint32_t step = (uint32_t)(wave + j * W);
+                const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
+                q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 32u, lane_base, acc, nv);
+                if (++j >= n_sw) {
+                    j = 0;
+                    finish_block(blk);
+                    blk++;
+                }
+            }
+            issue(cw[d]);
+        }
+    }
 }
 
 // ------------------------------------------------------------------ small-batch matrix-vector path
@@ -1209,12 +1625,20 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         __syncthreads();
     };
 
-    for (int kt = 0; kt < k_tiles; kt += 4) {
+    // Four tiles per trip with no way out in between: a path that left the loop body early
+    // would reach the loop head with the newest loads still pending on registers the body
+    // reuses, and the wait the compiler places there for that path (all loads done) would
+    // be paid by every trip.  The up to three tiles left over run after the loop.
+    int kt = 0;
+    for (; kt + 4 <= k_tiles; kt += 4) {
         tile(kt, 0, ring[1], ring[0]);
-        if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1]);
-        if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
-        if (kt + 3 < k_tiles) tile(kt + 3, 1, ring[0], ring[3]);
+        tile(kt + 1, 1, ring[2], ring[1]);
+        tile(kt + 2, 0, ring[3], ring[2]);
+        tile(kt + 3, 1, ring[0], ring[3]);
     }
+    if (kt < k_tiles) tile(kt, 0, ring[1], ring[0]);
+    if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1]);
+    if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
 
     // D layout of 32x32: element e of lane: row (n) = 8*(e/4) + 4*(lane/32) + e%4, column (m) = lane%32
     const bool n_vec = (N & 3) == 0;
@@ -1496,6 +1920,28 @@ int launch_gemv_stream(const void *x, const void *codes, const void *grid, float
 // tables, partial sums and x fit in the 160 KB of LDS, and every byte offset of the code
 // matrix fits the 31 bits the buffer addressing is used with
 template <int R, int W>
+bool gemv_q8_ok(int64_t M, int64_t N, int64_t K)
+{
+    return M <= 4 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + q8_x_bytes(M, K) <= 160 * 1024 &&
+           N * (K >> 2) < (1LL << 31);
+}
+
+template <int R, int W, int D, bool kPacked = false>
+int launch_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                   int64_t N, int64_t K, hipStream_t stream)
+{
+    // the 8-bit layout is the larger one, so the 16-bit kernel it may hand over to fits as well
+    const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(gemv_q8_kernel<R, W, D, kPacked>, 160 * 1024, attr_done)) return e;
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(gemv_q8_kernel<R, W, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+template <int R, int W>
 bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
 {
     return M <= 16 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + M * (2 * K + 16) <= 160 * 1024 &&
@@ -1516,6 +1962,29 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
 
+// The 8-bit kernel, one row tile at a time; the code stream three loads deep per wave when a
+// workgroup has more than two row tiles to walk through, two deep for shorter launches (where
+// a larger first burst only delays the first tile).
+// DMM_GEMV_8BIT=0 in the environment keeps batch 1 on the 16-bit kernel (read once).
+inline bool gemv_q8_enabled()
+{
+    static int on = -1;
+    if (on < 0) {
+        const char *e = getenv("DMM_GEMV_8BIT");
+        on = (e && e[0] == '0') ? 0 : 1;
+    }
+    return on == 1;
+}
+
+template <bool kPacked>
+int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                int64_t N, int64_t K, hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16;
+    if (n_tiles > 2 * cu_count()) return launch_gemv_q8<1, 16, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    return launch_gemv_q8<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+}
+
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
@@ -1530,11 +1999,23 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
         DMM_STREAM_CASE(1, 16, 4)
         DMM_STREAM_CASE(2, 16, 2)
         DMM_STREAM_CASE(2, 16, 3)
+#define DMM_Q8_CASE(TAG, R, D)                                                                     \
+    case TAG * 10000 + 1600 + D:                                                                   \
+        if (gemv_q8_ok<R, 16>(M, N, K))                                                            \
+            return launch_gemv_q8<R, 16, D>(x, codes, grid, scale, y, M, N, K, stream);            \
+        break;
+        DMM_Q8_CASE(8, 2, 2)
+        DMM_Q8_CASE(8, 2, 3)
+        DMM_Q8_CASE(9, 1, 2)
+        DMM_Q8_CASE(9, 1, 3)
+        DMM_Q8_CASE(9, 1, 4)
+#undef DMM_Q8_CASE
         case 20803: return launch_gemv_regx<2, 8, 1, 3>(x, codes, grid, scale, y, M, N, K, stream);
         case 20802: return launch_gemv_regx<2, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
         default: break;
     }
 #undef DMM_STREAM_CASE
+    if (gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return run_gemv_q8<false>(x, codes, grid, scale, y, M, N, K, stream);
     if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2>(x, codes, grid, scale, y, M, N, K, stream);
     return launch_gemv_regx<2, 8, 1, 3>(x, codes, grid, scale, y, M, N, K, stream);
 }
@@ -1783,6 +2264,7 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
     if (!gemv_ok(x, packed, grid, y, M, N, K) || dmm_packed_bytes(N, K) >= (1LL << 31)) return DMM_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if (M > 16) return launch_gemv_regx<2, 8, 2, 2, true>(x, packed, grid, scale, y, M, N, K, s);
+    if (gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return run_gemv_q8<true>(x, packed, grid, scale, y, M, N, K, s);
     if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2, true>(x, packed, grid, scale, y, M, N, K, s);
     return launch_gemv_regx<2, 8, 1, 3, true>(x, packed, grid, scale, y, M, N, K, s);
 }

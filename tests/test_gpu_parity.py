@@ -126,6 +126,89 @@ def test_auto_dispatch_and_torch_operator(M, N, K):
         assert torch.equal(y_w, y_t)
 
 
+# ----------------------------------------------------------------- batch-1 kernel, 8-bit operands
+# M <= 4 with x small enough for the LDS runs on fp8 weights / bf8 terms of x when every grid
+# value fits fp8, and hands over to the 16-bit kernel inside the same launch when one does not.
+def _gemv_vs_oracle(x, codes, grid, scale, packed=False):
+    W = orc.decode_f16(codes, grid)
+    ref = orc.matmul_f32(x, W, scale)
+    if packed:
+        y = dmm.decode_matmul_packed(dev(x), dmm.pack_codes(dev(codes)), dev(grid), scale, codes.shape[0])
+    else:
+        y = c_matmul(dev(x), dev(codes), dev(grid), scale, "gemv")
+    torch.cuda.synchronize()
+    return y, ref
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+@pytest.mark.parametrize("N,K", [(16, 256), (52, 1024), (4096, 2048), (1000, 4096), (12288, 8192)])
+@pytest.mark.parametrize("grid_kind", ["e8p", "fp8_all", "half_any", "one_off"])
+def test_gemv_8bit_operands_and_fallback(M, N, K, grid_kind):
+    if K == 8192 and M > 1:
+        pytest.skip("larger x: covered by the small-batch kernels elsewhere")
+    rng = np.random.default_rng(M * 7 + N + K)
+    if grid_kind == "e8p":
+        grid = orc.grid_from_codebook(orc.build_codebook_abs())
+    elif grid_kind == "fp8_all":
+        # every finite fp8 (e4m3) value, subnormals and both zeros included, as halves
+        b = np.arange(256, dtype=np.uint32)
+        b = b[(b & 0x7F) != 0x7F]
+        e, m = (b >> 3) & 0xF, b & 7
+        v = np.where(e == 0, m * 2.0 ** -9, (1 + m / 8.0) * 2.0 ** (e.astype(np.float64) - 7)) * np.where(b & 0x80, -1.0, 1.0)
+        grid = rng.choice(v, size=(256, 8)).astype(np.float16)
+        grid[0, :4] = [448.0, -448.0, 2.0 ** -9, -0.0]
+    elif grid_kind == "half_any":
+        grid = finite_random_grid(M + N)                                     # no fp8 can hold these
+        grid = (grid.astype(np.float32).clip(-8, 8)).astype(np.float16)
+    else:
+        grid = orc.grid_from_codebook(orc.build_codebook_abs()).copy()
+        grid[rng.integers(0, 256), rng.integers(0, 8)] = np.float16(1.0 + 2.0 ** -4)   # one value with 5 significant bits
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    codes = rng.integers(0, 65536, size=(N, K // 8)).astype(np.uint16)
+    # scale brings y to order 1, as the operator is used (the tolerance has an absolute part)
+    scale = float(np.float32(1.0 / (np.sqrt(K) * max(1.0, float(np.sqrt(np.mean(grid.astype(np.float64) ** 2)))))))
+    y, ref = _gemv_vs_oracle(x, codes, grid, scale)
+    assert_close_to_oracle(y, ref, "8-bit gemv %s M=%d N=%d K=%d" % (grid_kind, M, N, K))
+    yp, _ = _gemv_vs_oracle(x, codes, grid, scale, packed=True)
+    assert torch.equal(y, yp)                    # packed codes: same arithmetic, same order
+
+
+def test_gemv_8bit_exact_for_extreme_x():
+    """One non-zero x at a time, from all over the half range (largest, smallest normal,
+    subnormals, all 11 significant bits set), against weights 0 and +-0.5: the four bf8 terms
+    add up to x exactly and so does the mean of its code, so y = x w with no rounding at all."""
+    K, N = 2048, 64
+    grid = np.full((256, 8), 0.25, dtype=np.float16)   # w = 0.25 s + d: 0 or +-0.5
+    special = np.array([65504.0, -65504.0, 2.0 ** -14, 2.0 ** -21, -24 * 2.0 ** -24, 1023.5, 0.333251953125,
+                        2047.0, -6.103515625e-05 * 1.5, 40000.0, 3.0], dtype=np.float16)
+    rng = np.random.default_rng(5)
+    codes = rng.integers(0, 65536, size=(N, K // 8)).astype(np.uint16)
+    W = orc.decode_f16(codes, grid).astype(np.float64)
+    assert set(np.unique(W)) <= {-0.5, 0.0, 0.5}
+    for i, v in enumerate(special):
+        x = np.zeros((1, K), dtype=np.float16)
+        k = int(rng.integers(0, K))
+        x[0, k] = v
+        y = c_matmul(dev(x), dev(codes), dev(grid), 1.0, "gemv")
+        torch.cuda.synchronize()
+        want = float(v) * W[:, k]
+        assert np.array_equal(y.cpu().numpy().astype(np.float64)[0], want), (i, float(v))
+
+
+def test_gemv_8bit_non_finite_x():
+    K, N = 1024, 48
+    rng = np.random.default_rng(9)
+    grid = orc.grid_from_codebook(orc.build_codebook_abs())
+    x = rng.standard_normal((2, K)).astype(np.float16)
+    x[0, 17] = np.inf
+    x[1, 900] = np.nan
+    codes = rng.integers(0, 65536, size=(N, K // 8)).astype(np.uint16)
+    y, ref = _gemv_vs_oracle(x, codes, grid, 0.03125)
+    got = y.cpu().numpy().astype(np.float32)
+    assert np.array_equal(np.isnan(got), np.isnan(ref)) and np.array_equal(np.isinf(got), np.isinf(ref))
+    assert np.array_equal(got[np.isinf(got)], ref[np.isinf(ref)])   # the signs of the infinities
+
+
 def test_empty_problems():
     grid = dev(quarter_grid(0))
     x = torch.zeros(0, 64, dtype=torch.float16, device=DEV)
