@@ -17,6 +17,7 @@ SYMBOLS = {
     "dmm_decode_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "dmm_decode_matmul_f16": (ctypes.c_int, _OP),
     "dmm_gemv_f16": (ctypes.c_int, _OP),
+    "dmm_gemv_8bit_f16": (ctypes.c_int, _OP),
     "dmm_gemm_f16": (ctypes.c_int, _OP),
     "dmm_generic_f16": (ctypes.c_int, _OP),
     "dmm_workspace_bytes": (ctypes.c_int64, [_I64, _I64, _I64]),

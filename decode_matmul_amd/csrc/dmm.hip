@@ -664,76 +664,50 @@ __device__ __forceinline__ u2_t grid_row_fp8(const u4_t &row, bool &exact)
     return r;
 }
 
-// One half (bits) as four bf8 bytes t0..t3 (byte t of the result) with
-// h = t0 + t1 / 8 + t2 / 64 + t3 / 512: a term is the top byte of what is left, and what is left
-// after it is scaled by 8 (exact, and it keeps the remainder as far above the subnormal range
-// as h itself was), so every normal h is split without loss.  Non-finite h: t0 alone carries it.
-__device__ __forceinline__ uint32_t split_half_bf8(uint16_t bits)
-{
-    uint32_t out = 0;
-    uint16_t r = bits;
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        const uint16_t hi = r & 0xFF00u;
-        out |= (uint32_t)(hi >> 8) << (8 * t);
-        if ((bits & 0x7C00u) == 0x7C00u) break;
-        r = __builtin_bit_cast(uint16_t, (half_t)((__builtin_bit_cast(half_t, r) - __builtin_bit_cast(half_t, hi)) * (half_t)8.0f));
-    }
-    return out;
-}
-
-// 8 halves (one 16-byte piece of x) as four terms of 8 bf8 bytes each.  Returns whether all
-// 8 are finite; if not, the terms still add up for the finite ones and t0 alone carries the
-// others (the caller hands the launch to the 16-bit kernel anyway: an infinity must meet the
-// whole weight, not its two terms one after the other).
+// A half as four bf8 terms, h = t0 + t1 / 8 + t2 / 64 + t3 / 512: a term is the top byte of what
+// is left, and what is left after it is scaled by 8 (exact, and it keeps the remainder as far
+// above the subnormal range as h itself was), so every normal h is split without loss.
+// 8 halves (one 16-byte piece of x) at a time: term t of the 8 as 8 bytes in t[t].  Returns
+// whether all 8 are finite (if not, the caller hands the launch to the 16-bit kernel: an
+// infinity must meet the whole weight, not its two parts one after the other).
 __device__ __forceinline__ bool split_piece_bf8(const u4_t &v, u2_t (&t)[4])
 {
     bool finite = true;
 #pragma unroll
     for (int i = 0; i < 4; i++) finite = finite && (v[i] & 0x7C00u) != 0x7C00u && (v[i] & 0x7C000000u) != 0x7C000000u;
-    if (__builtin_expect(finite, 1)) {
-        u4_t r = v;
+    const h2_t eight = h2_t{(half_t)8.0f, (half_t)8.0f};
+    u4_t r = v;
 #pragma unroll
-        for (int term = 0; term < 4; term++) {
-            const u4_t hi = r & 0xFF00FF00u;
-            t[term][0] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07050301u);   // the high bytes of halves 0..3
-            t[term][1] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07050301u);   // and of halves 4..7
-            if (term < 3) {
+    for (int term = 0; term < 4; term++) {
+        const u4_t hi = r & 0xFF00FF00u;
+        t[term][0] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07050301u);   // the high bytes of halves 0..3
+        t[term][1] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07050301u);   // and of halves 4..7
+        if (term < 3) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) r[i] = as_u32((as_h2(r[i]) - as_h2(hi[i])) * h2_t{(half_t)8.0f, (half_t)8.0f});
-            }
-        }
-    } else {
-        uint32_t b[8];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            b[2 * i] = split_half_bf8((uint16_t)(v[i] & 0xFFFFu));
-            b[2 * i + 1] = split_half_bf8((uint16_t)(v[i] >> 16));
-        }
-#pragma unroll
-        for (int term = 0; term < 4; term++) {
-            t[term][0] = t[term][1] = 0;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                t[term][0] |= ((b[e] >> (8 * term)) & 0xFFu) << (8 * e);
-                t[term][1] |= ((b[4 + e] >> (8 * term)) & 0xFFu) << (8 * e);
-            }
+            for (int i = 0; i < 4; i++) r[i] = as_u32((as_h2(r[i]) - as_h2(hi[i])) * eight);
         }
     }
     return finite;
 }
 
-// mean of the 8 halves of a piece (fp32 sum in a fixed order), as a half
-__device__ __forceinline__ uint16_t piece_mean(const u4_t &v)
+// The mean of the 8 halves of a piece (fp32 sum, times 1/8, rounded to half) as its four bf8
+// terms, term t in byte t.  Finite pieces only.
+__device__ __forceinline__ uint32_t piece_mean_bf8(const u4_t &v)
 {
+    const h2_t ones = h2_t{(half_t)1.0f, (half_t)1.0f};
     float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const h2_t h = as_h2(v[i]);
-        sum += (float)h[0];
-        sum += (float)h[1];
+    for (int i = 0; i < 4; i++) sum = __builtin_amdgcn_fdot2(as_h2(v[i]), ones, sum, false);
+    uint32_t r = (uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sum * 0.125f));
+    const h2_t eight = h2_t{(half_t)8.0f, (half_t)8.0f};
+    uint32_t out = 0;
+#pragma unroll
+    for (int term = 0; term < 4; term++) {
+        const uint32_t hi = r & 0xFF00u;
+        out |= (hi >> 8) << (8 * term);
+        if (term < 3) r = as_u32((as_h2(r) - as_h2(hi)) * eight);
     }
-    return __builtin_bit_cast(uint16_t, (half_t)(sum * 0.125f));
+    return out;
 }
 
 struct Q8Gather {
@@ -814,6 +788,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     static_assert(W == 16, "the table staging below assumes 1024 threads");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
     if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
+    DMM_TRACE_MARK(0);
     f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // [2][W][R][4 * M]
     const int red_par = W * R * 4 * M;                                 // float4 per parity
     unsigned char *xt = smem_raw + kSTablesBytes + stream_red_bytes(R, W, M);
@@ -829,17 +804,16 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     const int row_bytes = K >> 2;
     const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;
 
-    // ---- prologue, in the order of the 16-bit kernel: grid row and x first, then the code
-    // stream, then the tables and the terms of x while the code loads fly --------------------
-    const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid & 255];
+    // ---- prologue: the loads with nothing queued in front of them first (grid rows, the first
+    // pieces of x), then the code stream, then the tables and the terms of x while the code
+    // loads fly.  The three kinds of staging go to different waves - grid rows to waves 0-3 (one
+    // row per thread), sign rows to waves 4-7, x to everybody - because every instruction of
+    // the prologue is paid once per wave that runs it, needed or not.
+    u4_t grow = u4_t{0u, 0u, 0u, 0u};
+    if (wave < 4) grow = reinterpret_cast<const u4_t *>(grid)[tid];
     const int row_chunks = K >> 3;                     // 16-byte pieces per row of x
-    constexpr int kXPer = 2;                           // pieces of row 0 per thread fetched up front
-    u4_t xv[kXPer];
-#pragma unroll
-    for (int u = 0; u < kXPer; u++) {
-        const int c = u * 64 * W + tid;
-        xv[u] = c < row_chunks ? reinterpret_cast<const u4_t *>(x)[c] : u4_t{0u, 0u, 0u, 0u};
-    }
+    const int n_pieces = M * row_chunks;               // x is [M][K] contiguous: piece p sits at x + 16 p
+    u4_t xnext = tid < n_pieces ? reinterpret_cast<const u4_t *>(x)[tid] : u4_t{0u, 0u, 0u, 0u};
 
     const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;   // k steps of this wave per row block
     const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
@@ -869,50 +843,51 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     u4_t cw[D][R];
 #pragma unroll
     for (int d = 0; d < D; d++) issue(cw[d]);
+    DMM_TRACE_MARK(1);
 
-    // sign rows: 2048 slots of 16 bytes (two copies each), two per thread
-    {
-        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw);
+    bool fits = true;   // stays true while x is finite and the grid fits fp8
+    if (wave >= 4 && wave < 8) {
+        // sign rows: 128 rows of 16 slots (16 bytes = two copies each); thread t of these 256 writes
+        // 8 slots of row t / 2 (16 neighbouring lanes hit 16 different slot positions)
+        const int t = tid - 256, row = t >> 1;
+        const u2_t sb = sign_bytes((uint32_t)row);
+        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw) + row * 16 + (t & 1) * 8;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const u2_t sb = sign_bytes((uint32_t)((tid + i * 1024) >> 4));
-            sg[tid + i * 1024] = u4_t{sb[0], sb[1], sb[0], sb[1]};
-        }
+        for (int i = 0; i < 8; i++) sg[(i + row) & 7] = u4_t{sb[0], sb[1], sb[0], sb[1]};
     }
     __builtin_amdgcn_sched_barrier(0);   // keep the sign rows ahead of the waits for the loads
 
-    // x -> its four terms, and the means of every 8 values -> theirs
-    bool fits = true;   // stays true while x is finite and (below) the grid fits fp8
-    auto stage_piece = [&](const u4_t &v, int m, int c) {
-        u2_t t[4];
-        fits = split_piece_bf8(v, t) && fits;
-        const uint32_t mb = split_half_bf8(piece_mean(v));
-        const int c8 = (c & ~3) | ((c & 1) << 1) | ((c >> 1) & 1);   // codes 0, 2, 1, 3 of each four
-#pragma unroll
-        for (int term = 0; term < 4; term++) {
-            *reinterpret_cast<u2_t *>(xt + (m * 4 + term) * xt_pitch + c * 8) = t[term];
-            x8t[(m * 4 + term) * x8_pitch + c8] = (unsigned char)(mb >> (8 * term));
-        }
-    };
-#pragma unroll
-    for (int u = 0; u < kXPer; u++) {
-        const int c = u * 64 * W + tid;
-        if (c < row_chunks) stage_piece(xv[u], 0, c);
-    }
-    for (int c = kXPer * 64 * W + tid; c < row_chunks; c += 64 * W) stage_piece(reinterpret_cast<const u4_t *>(x)[c], 0, c);
-    for (int m = 1; m < M; m++)
-        for (int c = tid; c < row_chunks; c += 64 * W) stage_piece(reinterpret_cast<const u4_t *>(x + (int64_t)m * K)[c], m, c);
-
-    // grid rows: thread tid converts row tid % 256 and writes 4 of its 16 slots (two copies each)
+    // x -> its four terms, and the means of every 8 values -> theirs.  One piece per thread and
+    // trip, the next one already on its way.
     {
+        int m = 0, c = tid;
+        for (int p = tid; p < n_pieces; p += 64 * W) {
+            const u4_t v = xnext;
+            if (p + 64 * W < n_pieces) xnext = reinterpret_cast<const u4_t *>(x)[p + 64 * W];
+            while (c >= row_chunks) { c -= row_chunks; m++; }
+            u2_t t[4];
+            fits = split_piece_bf8(v, t) && fits;
+            const uint32_t mb = piece_mean_bf8(v);
+            const int c8 = (c & ~3) | ((c & 1) << 1) | ((c >> 1) & 1);   // codes 0, 2, 1, 3 of each four
+#pragma unroll
+            for (int term = 0; term < 4; term++) {
+                *reinterpret_cast<u2_t *>(xt + (m * 4 + term) * xt_pitch + c * 8) = t[term];
+                x8t[(m * 4 + term) * x8_pitch + c8] = (unsigned char)(mb >> (8 * term));
+            }
+            c += 64 * W;
+        }
+    }
+    DMM_TRACE_MARK(2);
+    if (wave < 4) {
+        // grid rows: thread tid converts row tid and writes its 16 slots (two copies each)
         bool exact;
         const u2_t g8 = grid_row_fp8(grow, exact);
         fits = fits && exact;
-        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes);
-        const int row = tid & 255, c0 = (tid >> 8) * 4;
+        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes) + tid * 16;
 #pragma unroll
-        for (int i = 0; i < 4; i++) gg[row * 16 + ((c0 + i + tid) & 15)] = u4_t{g8[0], g8[1], g8[0], g8[1]};
+        for (int i = 0; i < 16; i++) gg[(i + tid) & 15] = u4_t{g8[0], g8[1], g8[0], g8[1]};
     }
+    DMM_TRACE_MARK(3);
     // the vote: every wave publishes whether one of its rows or pieces failed, in a word of its own (so
     // nothing needs clearing first), and after the barrier every wave reads all of them
     uint32_t *votes = reinterpret_cast<uint32_t *>(x8t + 4 * M * x8_pitch);
@@ -926,6 +901,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
         return;
     }
 
+    DMM_TRACE_MARK(4);
     // B operand addresses of this lane: column c16 = 4 m + term (column 0 for the idle ones)
     const int col = c16 < 4 * M ? c16 : 0;
     const uint32_t xlane = lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64);
@@ -982,16 +958,24 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             if (i0 + d < n_items) {
                 const uint32_t step = (uint32_t)(wave + j * W);
                 const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
+#ifdef DMM_TRACE
+                if (i0 + d < 7) { asm volatile("" ::"v"(cw[d][0])); DMM_TRACE_MARK(8 + 2 * (i0 + d)); }
+#endif
                 q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 32u, lane_base, acc, nv);
+                if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
                 if (++j >= n_sw) {
                     j = 0;
+                    if (blk == 0) DMM_TRACE_MARK(5);
                     finish_block(blk);
+                    if (blk == 0) DMM_TRACE_MARK(6);
                     blk++;
                 }
             }
             issue(cw[d]);
         }
     }
+    DMM_TRACE_MARK(7);
+    DMM_TRACE_DUMP();
 }
 
 // ------------------------------------------------------------------ small-batch matrix-vector path
@@ -1931,7 +1915,11 @@ int launch_gemv_q8(const void *x, const void *codes, const void *grid, float sca
                    int64_t N, int64_t K, hipStream_t stream)
 {
     // the 8-bit layout is the larger one, so the 16-bit kernel it may hand over to fits as well
+#ifdef DMM_TRACE
+    const size_t shmem = 160 * 1024;
+#else
     const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
+#endif
     static bool attr_done[kMaxDevices] = {};
     if (int e = allow_dynamic_lds(gemv_q8_kernel<R, W, D, kPacked>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
@@ -1985,6 +1973,23 @@ int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale,
     return launch_gemv_q8<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
 }
 
+// The choice among the matrix-vector kernels.  At most one row tile per workgroup: the 16-bit
+// streaming kernel, one tile at a time (its prologue is the cheaper one and there is no steady
+// state to speak of).  More: the 8-bit kernel where it applies, else the 16-bit one two tiles
+// at a time; the register-x kernel when x does not fit the LDS.
+template <bool kPacked>
+int run_gemv_auto(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                  int64_t N, int64_t K, hipStream_t stream)
+{
+    const bool short_launch = (N + 15) / 16 <= cu_count();
+    if (short_launch && gemv_stream_ok<1, 16>(M, N, K))
+        return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    if (gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    return launch_gemv_regx<2, 8, 1, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+}
+
+
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
@@ -1997,6 +2002,8 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
     switch (gemv_cfg_override()) {
         DMM_STREAM_CASE(2, 8, 4)
         DMM_STREAM_CASE(1, 16, 4)
+        DMM_STREAM_CASE(1, 16, 3)
+        DMM_STREAM_CASE(1, 16, 2)
         DMM_STREAM_CASE(2, 16, 2)
         DMM_STREAM_CASE(2, 16, 3)
 #define DMM_Q8_CASE(TAG, R, D)                                                                     \
@@ -2015,9 +2022,7 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
         default: break;
     }
 #undef DMM_STREAM_CASE
-    if (gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return run_gemv_q8<false>(x, codes, grid, scale, y, M, N, K, stream);
-    if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2>(x, codes, grid, scale, y, M, N, K, stream);
-    return launch_gemv_regx<2, 8, 1, 3>(x, codes, grid, scale, y, M, N, K, stream);
+    return run_gemv_auto<false>(x, codes, grid, scale, y, M, N, K, stream);
 }
 
 template <int WN, int WM, int TN, int TM>
@@ -2234,6 +2239,15 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
     return run_gemv(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
 }
 
+int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                      int64_t N, int64_t K, void *stream)
+{
+    int st = check_common(x, codes, grid, y, M, N, K);
+    if (st != DMM_OK || M == 0 || N == 0) return st;
+    if (!gemv_ok(x, codes, grid, y, M, N, K) || !gemv_q8_ok<1, 16>(M, N, K)) return DMM_ERR_UNSUPPORTED;
+    return run_gemv_q8<false>(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
+}
+
 int64_t dmm_packed_bytes(int64_t N, int64_t K)
 {
     if (N < 0 || K < 256 || (K & 255)) return 0;
@@ -2264,9 +2278,7 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
     if (!gemv_ok(x, packed, grid, y, M, N, K) || dmm_packed_bytes(N, K) >= (1LL << 31)) return DMM_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if (M > 16) return launch_gemv_regx<2, 8, 2, 2, true>(x, packed, grid, scale, y, M, N, K, s);
-    if (gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return run_gemv_q8<true>(x, packed, grid, scale, y, M, N, K, s);
-    if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2, true>(x, packed, grid, scale, y, M, N, K, s);
-    return launch_gemv_regx<2, 8, 1, 3, true>(x, packed, grid, scale, y, M, N, K, s);
+    return run_gemv_auto<true>(x, packed, grid, scale, y, M, N, K, s);
 }
 
 int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *grid, float scale, void *y,

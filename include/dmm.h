@@ -92,6 +92,23 @@ int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid,
  *                    DPP wave reduction.  The catch-all. */
 int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale,
                  void *y, int64_t M, int64_t N, int64_t K, void *stream);
+/*   dmm_gemv_8bit_f16  the matrix-vector kernel on 8-bit MFMA operands, which dmm_gemv_f16 and
+ *                    the operator pick for M <= 4 on launches of more than one 16-row tile per
+ *                    compute unit.  Weights as fp8 (e4m3) bytes - exact when every grid value
+ *                    has at most 4 significant bits in fp8's range, as the E8P grid does - and x
+ *                    as four bf8 (e5m2) terms that add up to it exactly; the +-1/4 shift of a
+ *                    code is added through the per-code means of x.  Nothing is lost in the
+ *                    operands; the 8-bit MFMA adds its products in an adder narrower than fp32,
+ *                    so y differs from the 16-bit kernel's by about 2^-14 of a row's scale (the
+ *                    tolerance of the operator is 1e-2).  A grid that does not fit fp8, or an x
+ *                    that is not finite, is detected inside the launch and served by the 16-bit
+ *                    kernel: same call, same status.  DMM_GEMV_8BIT=0 in the environment keeps
+ *                    the operator off this kernel.  Domain: that of dmm_gemv_f16 with M <= 4 and
+ *                    4 M (K + 16 + K / 8 + 16) bytes of x terms fitting the LDS beside the
+ *                    tables (K <= 13 K at M = 1); DMM_ERR_UNSUPPORTED outside.  No counterpart
+ *                    in the reference (its kernel multiplies int8 by int8). */
+int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float scale,
+                      void *y, int64_t M, int64_t N, int64_t K, void *stream);
 int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale,
                  void *y, int64_t M, int64_t N, int64_t K, void *stream);
 int dmm_generic_f16(const void *x, const void *codes, const void *grid, float scale,

@@ -28,6 +28,7 @@ def c_decode(codes, grid, out=None):
 _ENTRY = {
     "auto": "dmm_decode_matmul_f16",
     "gemv": "dmm_gemv_f16",
+    "gemv8": "dmm_gemv_8bit_f16",
     "gemm": "dmm_gemm_f16",
     "generic": "dmm_generic_f16",
 }

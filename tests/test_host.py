@@ -59,6 +59,9 @@ def test_argument_errors_are_status_codes_not_crashes():
     # explicit paths refuse shapes outside their domain instead of falling back
     assert lib.dmm_gemv_f16(p, p, p, 1.0, p, 1, 4, 16, None) == -5       # K % 256 != 0
     assert lib.dmm_gemv_f16(p, p, p, 1.0, p, 64, 4, 256, None) == -5     # M too large
+    assert lib.dmm_gemv_8bit_f16(p, p, p, 1.0, p, 5, 4, 256, None) == -5    # M > 4
+    assert lib.dmm_gemv_8bit_f16(p, p, p, 1.0, p, 1, 4, 28672, None) == -5  # x terms do not fit the LDS
+    assert lib.dmm_gemv_8bit_f16(None, p, p, 1.0, p, 1, 4, 256, None) == -1
     assert lib.dmm_gemm_f16(p, p, p, 1.0, p, 64, 4, 16, None) == -5      # K % 64 != 0
     # empty problems succeed without touching the device
     assert lib.dmm_decode_f16(None, None, None, 0, 64, None) == 0
