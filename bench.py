@@ -5,9 +5,10 @@ Headline (the JSON line's `value`): batch-1 decode-GEMV at the Llama-2-70B proje
 shapes.  One step = the four GEMVs (8192->10240, 8192->8192, 8192->28672, 28672->8192), each
 on the next of several distinct code buffers so that the 256 MB Infinity Cache cannot serve
 the weights; `value` is code bytes (N*K/4 per GEMV) per second over the timed region, inputs
-resident in HBM.  `roofline` is the GEMV kernel alone: code bytes per launch over the
-kernel's own duration (HIP events placed around the kernel by the library's timing hook)
-against 8 TB/s.  `prefill` and `small_batch` carry the M=2048 and M=4..32 figures;
+resident in HBM.  `roofline` is the GEMV kernel that carries most of the step's bytes, alone:
+code bytes per launch over the kernel's own duration (HIP events placed around the kernel by
+the library's timing hook) against 8 TB/s; `all_gemv_launches` is the same figure over every
+launch of the step, per kernel.  `prefill` and `small_batch` carry the M=2048 and M=4..32 figures;
 `cpu_baseline` is the torch CPU path on the host cores on one 8192x8192 GEMV.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
@@ -24,10 +25,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
-# HBM bytes one GEMV launch moves, averaged over the four shapes: rocprofv3 FETCH_SIZE and
-# WRITE_SIZE per dispatch (19,132.8 KiB and 28.7 KiB), each scaled by what the same counter
-# reads for a plain 256 MiB device copy (x2.000 and x1.000).  Algorithmic code bytes: 38,797,312.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 39209000
+# HBM bytes one GEMV launch moves, per kernel, averaged over the shapes of the step that kernel
+# serves: rocprofv3 FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter
+# reads for a plain 256 MiB device copy (x2.000 and x1.000).
+# gemv_q8_kernel: 15,856.2 KiB fetched, 30.9 KiB written per dispatch (32,156,331 code bytes);
+# gemv_stream_kernel: 28,979.6 KiB and 16.0 KiB (58,720,256 code bytes).
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8_kernel": 32502000, "dmm::gemv_stream_kernel": 59361000}
 
 
 def parse():
@@ -165,13 +168,24 @@ def main():
             per_shape.setdefault((p["K"], p["N"]), []).append(ev[j][0].elapsed_time(ev[j][1]) * 1e-3)
             j += 1
     kern_s = sum(sum(v) for v in per_shape.values())
-    achieved = step_bytes * args.steps / kern_s / 1e9
     shape_rows = []
+    kernels = {}    # kernel name -> launches, seconds, code bytes (the step runs two GEMV kernels)
     for (K, N), v in per_shape.items():
         avg = sum(v) / len(v)
         gbs = workload.code_bytes(N, K) / avg / 1e9
+        name = lib.dmm_gemv_kernel_name(1, N, K).decode()
         shape_rows.append({"K": K, "N": N, "code_bytes": workload.code_bytes(N, K), "kernel_us": round(avg * 1e6, 3),
-                           "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
+                           "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "kernel": name})
+        k = kernels.setdefault(name, {"launches": 0, "seconds": 0.0, "bytes": 0})
+        k["launches"] += len(v)
+        k["seconds"] += sum(v)
+        k["bytes"] += workload.code_bytes(N, K) * len(v)
+    # the roofline object covers the kernel that carries most of the step's bytes; all launches
+    # together are in `all_gemv_launches`
+    dom = max(kernels, key=lambda n: kernels[n]["bytes"])
+    kd = kernels[dom]
+    achieved = kd["bytes"] / kd["seconds"] / 1e9
+    all_gbs = step_bytes * args.steps / kern_s / 1e9
 
     out = {
         "metric": "batch-1 effective weight GB/s (code bytes N*K/4 per second, Llama-2-70B projection shapes)",
@@ -190,10 +204,17 @@ def main():
                    "M": 1, "code_buffers_rotated": copies, "distinct_code_MB": round(copies * step_bytes / 1e6, 1),
                    "step": "4 GEMVs, one per shape", "launch": launch_mode},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "dmm::gemv_stream_kernel", "launches": n_launch,
-                     "avg_launch_us": round(kern_s / n_launch * 1e6, 3),
-                     "algorithmic_bytes_per_launch": step_bytes / len(probs)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+                     "kernel": dom, "launches": kd["launches"],
+                     "avg_launch_us": round(kd["seconds"] / kd["launches"] * 1e6, 3),
+                     "algorithmic_bytes_per_launch": kd["bytes"] / kd["launches"]},
+        "all_gemv_launches": {"launches": n_launch, "avg_launch_us": round(kern_s / n_launch * 1e6, 3),
+                              "GBps": round(all_gbs, 2), "frac_hbm": round(all_gbs / HBM_PEAK_GBS, 4),
+                              "kernels": {n: {"launches": k["launches"],
+                                              "avg_launch_us": round(k["seconds"] / k["launches"] * 1e6, 3),
+                                              "GBps": round(k["bytes"] / k["seconds"] / 1e9, 2)}
+                                          for n, k in kernels.items()}},
         "gemv_shapes": shape_rows,
     }
 

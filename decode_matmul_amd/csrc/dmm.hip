@@ -1977,18 +1977,28 @@ int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale,
 // streaming kernel, one tile at a time (its prologue is the cheaper one and there is no steady
 // state to speak of).  More: the 8-bit kernel where it applies, else the 16-bit one two tiles
 // at a time; the register-x kernel when x does not fit the LDS.
+enum GemvKind { kGemvStreamShort, kGemvQ8, kGemvStream, kGemvRegx };
+
+GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
+{
+    const bool short_launch = (N + 15) / 16 <= cu_count();
+    if (short_launch && gemv_stream_ok<1, 16>(M, N, K)) return kGemvStreamShort;
+    if (gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return kGemvQ8;
+    if (gemv_stream_ok<2, 16>(M, N, K)) return kGemvStream;
+    return kGemvRegx;
+}
+
 template <bool kPacked>
 int run_gemv_auto(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                   int64_t N, int64_t K, hipStream_t stream)
 {
-    const bool short_launch = (N + 15) / 16 <= cu_count();
-    if (short_launch && gemv_stream_ok<1, 16>(M, N, K))
-        return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    if (gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    if (gemv_stream_ok<2, 16>(M, N, K)) return launch_gemv_stream<2, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    return launch_gemv_regx<2, 8, 1, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    switch (pick_gemv(M, N, K)) {
+        case kGemvStreamShort: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case kGemvStream: return launch_gemv_stream<2, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return launch_gemv_regx<2, 8, 1, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    }
 }
-
 
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
@@ -2237,6 +2247,18 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
     if (st != DMM_OK || M == 0 || N == 0) return st;
     if (!gemv_ok(x, codes, grid, y, M, N, K)) return DMM_ERR_UNSUPPORTED;
     return run_gemv(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
+}
+
+const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K)
+{
+    if (M < 1 || M > 32 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31)) return "";
+    if (M > 16) return "dmm::gemv_regx_kernel";
+    switch (pick_gemv(M, N, K)) {
+        case kGemvStreamShort:
+        case kGemvStream: return "dmm::gemv_stream_kernel";
+        case kGemvQ8: return "dmm::gemv_q8_kernel";
+        default: return "dmm::gemv_regx_kernel";
+    }
 }
 
 int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,

@@ -109,6 +109,11 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
  *                    in the reference (its kernel multiplies int8 by int8). */
 int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float scale,
                       void *y, int64_t M, int64_t N, int64_t K, void *stream);
+/* Which matrix-vector kernel the operator runs for a shape with aligned pointers, as a profiler's
+ * kernel trace names it without the template arguments ("dmm::gemv_q8_kernel",
+ * "dmm::gemv_stream_kernel", "dmm::gemv_regx_kernel"; "" outside dmm_gemv_f16's domain).  For
+ * benchmarks that report per kernel.  Static storage.  No counterpart in the reference. */
+const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K);
 int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale,
                  void *y, int64_t M, int64_t N, int64_t K, void *stream);
 int dmm_generic_f16(const void *x, const void *codes, const void *grid, float scale,
