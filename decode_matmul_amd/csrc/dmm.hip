@@ -29,6 +29,7 @@ typedef float f4_t __attribute__((ext_vector_type(4)));
 typedef float f16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+typedef int i8_t __attribute__((ext_vector_type(8)));
 
 constexpr int kWave = 64;
 
@@ -594,11 +595,13 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 // LDS serves at twice the rate, by running the matrix unit on 8-bit operands:
 //   * weights.  w = s g + d, s = +-1 per dim, d = +-1/4 per code.  The grid table holds rows of
 //     8 fp8 bytes, the sign table rows of 8 flag bytes (0x80 = flipped); one exclusive or per
-//     4 weights applies the signs, and the 8 bytes of a code are the A operand of
-//     v_mfma_f32_16x16x32_fp8_bf8 as they are.  d is left out of the decode and added by the
+//     4 weights applies the signs, and the 8 bytes of a code are a quarter of the A operand of
+//     v_mfma_f32_16x16x128_f8f6f4 (four codes = 32 consecutive k per lane; twice the time of the
+//     16x16x32 form for four times the work) as they are.  d is left out of the decode and added by the
 //     matrix unit instead: sum_k d x[k] = sum over codes of (8 d) * (mean of the code's 8 x
-//     values), one more MFMA per 16 rows x 256 k whose A operand is +-2.0 per code, made from
-//     the code words themselves (shift bit = sign bit of the byte);
+//     values), one more MFMA per 16 rows x 256 k (into an accumulator of its own) whose A
+//     operand is +-2.0 per code, made from the code words themselves (shift bit = sign bit of
+//     the byte);
 //   * x.  A half with a zero low byte IS a bf8 (e5m2) number in its high byte.  Cutting x after
 //     its top byte, subtracting, scaling what is left by 8 and repeating gives
 //     x = t0 + t1 / 8 + t2 / 64 + t3 / 512 exactly for every normal x (3 significant bits per
@@ -607,15 +610,18 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 //     those weights, at the end.  The per-code means (fp32 sum of 8, times 1/8, rounded to
 //     half) are split the same way.
 // s g + d is exact in half for every fp8 g and the terms of x add up to x (subnormal x may lose
-// bits below 2^-24 * 4), so nothing is lost in the operands; what differs from the 16-bit kernel is the matrix unit's own arithmetic: the
-// 8-bit MFMA adds each group of products in an adder narrower than fp32 (small products lose
-// low bits against the largest of the group) and the means are rounded to half.  Measured
-// against the fp64 reference the error is about 2^-14 of a row's scale (1.5 half ulps at the
-// 99th percentile on the benchmark's inputs, where the 16-bit kernel stays below the 0.5 ulp of
-// the output rounding) - a hundredth of the operator's tolerance of 1e-2.  A grid with a value fp8 cannot hold is found
-// while the table is built (convert, convert back, compare), an x that is not finite while it
-// is split; every workgroup then runs the 16-bit kernel above instead: same launch, same
-// result as that kernel gives.
+// bits below 2^-24 * 4), so nothing is lost in the operands, and the products are exact in the
+// fp32 accumulators.  Two things remain: the means (at M = 1 they are carried in eight terms,
+// i.e. to the full fp32 sum; at M = 2 .. 4, where the columns are needed for x, in four, i.e.
+// rounded to half), and the matrix unit's adder, which aligns the products of a group to the
+// largest of them.  Measured against the fp64 reference on the benchmark's inputs at M = 1: 98 %
+// of the outputs are the correctly rounded ones and the 99th percentile of the error is 0.57
+// half ulps (the 16-bit kernel: 0.5, the output rounding alone); with 100-fold outliers in x
+// 2.6 ulps; x with few significant bits: every output correctly rounded.  At M = 2 .. 4 the
+// rounded means bring it to 1.5 ulps.  All of it a hundredth of the operator's tolerance of
+// 1e-2 or less.  A grid with a value fp8 cannot hold is found while the table is built
+// (convert, convert back, compare), an x that is not finite while it is split; every workgroup
+// then runs the 16-bit kernel above instead: same launch, same result as that kernel gives.
 // LDS map: [0, 32K) sign rows (128 x 32 copies x 8 B), [32K, 96K) grid rows (256 x 32 copies x
 // 8 B; a lane reads copy lane % 32, conflict-free for any codes), partial sums, then the terms
 // of x (column m * 4 + t, pitch K + 16 bytes) and of the means (pitch K / 8 + 16).
@@ -626,7 +632,11 @@ __device__ __forceinline__ u2_t lds_read8(uint32_t byte_addr)
 }
 
 // terms of x, terms of the means, and one word per wave for the vote on the grid
-__host__ __device__ constexpr int64_t q8_x_bytes(int64_t M, int64_t K) { return 4 * M * (K + 16) + 4 * M * (K / 8 + 16) + 64; }
+__host__ __device__ constexpr int q8_mean_terms(int64_t M) { return M == 1 ? 8 : 4; }
+__host__ __device__ constexpr int64_t q8_x_bytes(int64_t M, int64_t K)
+{
+    return 4 * M * (K + 16) + q8_mean_terms(M) * M * (K / 8 + 16) + 64;
+}
 
 // the 8 sign flags of a sign-row index as bytes: dims 0-3 in [0], 4-7 in [1]
 __device__ __forceinline__ u2_t sign_bytes(uint32_t s7)
@@ -690,22 +700,24 @@ __device__ __forceinline__ bool split_piece_bf8(const u4_t &v, u2_t (&t)[4])
     return finite;
 }
 
-// The mean of the 8 halves of a piece (fp32 sum, times 1/8, rounded to half) as its four bf8
-// terms, term t in byte t.  Finite pieces only.
-__device__ __forceinline__ uint32_t piece_mean_bf8(const u4_t &v)
+// The mean of the 8 halves of a piece (fp32 sum, times 1/8) as eight bf8 terms,
+// mean = sum_t term[t] / 8^t, term t in byte t % 4 of word t / 4.  The split runs in fp32: a
+// term is the top byte of the half nearest to what is left (it may overshoot: the remainder is
+// signed), the remainder is scaled by 8 - eight terms of 3 significant bits carry the 24 bits
+// of the fp32 mean.  Four terms (the first word) are the mean to half precision.
+__device__ __forceinline__ u2_t piece_mean_bf8(const u4_t &v)
 {
     const h2_t ones = h2_t{(half_t)1.0f, (half_t)1.0f};
-    float sum = 0.f;
+    float r = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; i++) sum = __builtin_amdgcn_fdot2(as_h2(v[i]), ones, sum, false);
-    uint32_t r = (uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sum * 0.125f));
-    const h2_t eight = h2_t{(half_t)8.0f, (half_t)8.0f};
-    uint32_t out = 0;
+    for (int i = 0; i < 4; i++) r = __builtin_amdgcn_fdot2(as_h2(v[i]), ones, r, false);
+    r *= 0.125f;
+    u2_t out = u2_t{0u, 0u};
 #pragma unroll
-    for (int term = 0; term < 4; term++) {
-        const uint32_t hi = r & 0xFF00u;
-        out |= (hi >> 8) << (8 * term);
-        if (term < 3) r = as_u32((as_h2(r) - as_h2(hi)) * eight);
+    for (int term = 0; term < 8; term++) {
+        const uint32_t hi = (uint32_t)__builtin_bit_cast(uint16_t, (half_t)r) & 0xFF00u;
+        out[term >> 2] |= (hi >> 8) << (8 * (term & 3));
+        if (term < 7) r = (r - (float)__builtin_bit_cast(half_t, (uint16_t)hi)) * 8.0f;
     }
     return out;
 }
@@ -734,9 +746,39 @@ __device__ __forceinline__ long q8_pack(uint32_t lo, uint32_t hi)
 // operands of its two codes), x8addr: its 8 means.
 template <int R>
 __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t x8addr, uint32_t lane_base,
-                                        f4_t (&acc)[R][2], int nv)
+                                        f4_t (&acc)[R][2], f4_t (&accd)[R], int nv)
 {
     constexpr int kItems = 4 * R;
+    if constexpr (R == 1) {
+        // one tile: all 16 table gathers and the 5 reads of x of the step go out first (8-byte
+        // results: 48 registers), so the wave meets the LDS latency once per step, not once
+        // per word
+        Q8Gather g[4];
+        u4_t xq[4];
+#pragma unroll
+        for (int t2 = 0; t2 < 4; t2++) {
+            xq[t2] = lds_read16(xaddr + t2 * 16);
+            q8_gather(g[t2], cw[0][t2], lane_base);
+        }
+        const u2_t x8 = lds_read8(x8addr);
+        // two words = four codes = 32 consecutive k of the lane's 64: one 16x16x128 MFMA (32
+        // bytes per lane and operand, A fp8, B bf8, no scaling), which does four times the work
+        // of the 16x16x32 form in twice its time
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const Q8Gather &b0 = g[2 * h], &b1 = g[2 * h + 1];
+            const i8_t a = i8_t{(int)(b0.g0[0] ^ b0.s0[0]), (int)(b0.g0[1] ^ b0.s0[1]), (int)(b0.g1[0] ^ b0.s1[0]),
+                                (int)(b0.g1[1] ^ b0.s1[1]), (int)(b1.g0[0] ^ b1.s0[0]), (int)(b1.g0[1] ^ b1.s0[1]),
+                                (int)(b1.g1[0] ^ b1.s1[0]), (int)(b1.g1[1] ^ b1.s1[1])};
+            const u4_t &x0 = xq[2 * h], &x1 = xq[2 * h + 1];
+            const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+            acc[0][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[0][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
+        }
+        const uint32_t a8lo = ((cw[0][0] >> 8) & 0x00800080u) | (cw[0][1] & 0x80008000u) | 0x40404040u;
+        const uint32_t a8hi = ((cw[0][2] >> 8) & 0x00800080u) | (cw[0][3] & 0x80008000u) | 0x40404040u;
+        accd[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]), accd[0], 0, 0, 0);
+        return;
+    }
     Q8Gather buf[2];
     u4_t xb[2];
     xb[0] = lds_read16(xaddr);
@@ -769,8 +811,8 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
                 // byte 3 or byte 2) - the means are stored in the same order
                 const uint32_t a8lo = ((cw[r][0] >> 8) & 0x00800080u) | (cw[r][1] & 0x80008000u) | 0x40404040u;
                 const uint32_t a8hi = ((cw[r][2] >> 8) & 0x00800080u) | (cw[r][3] & 0x80008000u) | 0x40404040u;
-                acc[r][0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]),
-                                                                       acc[r][0], 0, 0, 0);
+                accd[r] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]),
+                                                                     accd[r], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -792,6 +834,10 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // [2][W][R][4 * M]
     const int red_par = W * R * 4 * M;                                 // float4 per parity
     unsigned char *xt = smem_raw + kSTablesBytes + stream_red_bytes(R, W, M);
+    // M == 1: eight terms of the means in columns 0..7 (the shift term has an accumulator of its
+    // own, so columns 4..7 of the main one are simply not used); M > 1: four terms, column
+    // 4 m + t like x
+    const int n_mt = q8_mean_terms(M);
     const int xt_pitch = K + 16, x8_pitch = (K >> 3) + 16;
     unsigned char *x8t = xt + 4 * M * xt_pitch;
 
@@ -867,12 +913,16 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             while (c >= row_chunks) { c -= row_chunks; m++; }
             u2_t t[4];
             fits = split_piece_bf8(v, t) && fits;
-            const uint32_t mb = piece_mean_bf8(v);
+            const u2_t mb = piece_mean_bf8(v);
             const int c8 = (c & ~3) | ((c & 1) << 1) | ((c >> 1) & 1);   // codes 0, 2, 1, 3 of each four
 #pragma unroll
             for (int term = 0; term < 4; term++) {
                 *reinterpret_cast<u2_t *>(xt + (m * 4 + term) * xt_pitch + c * 8) = t[term];
-                x8t[(m * 4 + term) * x8_pitch + c8] = (unsigned char)(mb >> (8 * term));
+                x8t[(m * n_mt + term) * x8_pitch + c8] = (unsigned char)(mb[0] >> (8 * term));
+            }
+            if (M == 1) {
+#pragma unroll
+                for (int term = 0; term < 4; term++) x8t[(4 + term) * x8_pitch + c8] = (unsigned char)(mb[1] >> (8 * term));
             }
             c += 64 * W;
         }
@@ -890,7 +940,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     DMM_TRACE_MARK(3);
     // the vote: every wave publishes whether one of its rows or pieces failed, in a word of its own (so
     // nothing needs clearing first), and after the barrier every wave reads all of them
-    uint32_t *votes = reinterpret_cast<uint32_t *>(x8t + 4 * M * x8_pitch);
+    uint32_t *votes = reinterpret_cast<uint32_t *>(x8t + n_mt * M * x8_pitch);
     const bool wave_bad = __builtin_amdgcn_ballot_w64(!fits) != 0;
     if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
     __syncthreads();
@@ -904,13 +954,21 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     DMM_TRACE_MARK(4);
     // B operand addresses of this lane: column c16 = 4 m + term (column 0 for the idle ones)
     const int col = c16 < 4 * M ? c16 : 0;
+    const int col8 = c16 < n_mt * M ? c16 : 0;
     const uint32_t xlane = lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64);
-    const uint32_t x8lane = lds_addr(x8t) + (uint32_t)(col * x8_pitch + q * 8);
+    const uint32_t x8lane = lds_addr(x8t) + (uint32_t)(col8 * x8_pitch + q * 8);
 
     f4_t acc[R][2];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
-    const float term_weight = __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)(c16 & 3) * 3u << 23));   // 8^-(c16 % 4)
+    // weights of this lane's column: 8^-t with t = c16 % 4 for x, and for the means t = c16 % 4
+    // (M > 1) or c16 % 8 (M == 1); columns that hold nothing count as zero
+    const float x_weight = c16 < 4 * M ? __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)(c16 & 3) * 3u << 23)) : 0.f;
+    const float mean_weight =
+        c16 < n_mt * M ? __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)(c16 & (n_mt - 1)) * 3u << 23)) : 0.f;
+    f4_t accd[R];   // the shift term
+#pragma unroll
+    for (int r = 0; r < R; r++) accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
 
     auto finish_block = [&](int blk) {
         f4_t *rp = red + (blk & 1) * red_par;
@@ -918,14 +976,15 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
         for (int r = 0; r < R; r++) {
             // the four term columns of an x row are added first, each with the weight of its term:
             // lane 4 m gets columns 4 m .. 4 m + 3
-            f4_t v = (acc[r][0] + acc[r][1]) * term_weight;
+            f4_t v = (acc[r][0] + acc[r][1]) * x_weight + accd[r] * mean_weight;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 v[e] = dpp_shr_add<0x101>(v[e]);   // row_shl:1
                 v[e] = dpp_shr_add<0x102>(v[e]);   // row_shl:2
+                if (M == 1) v[e] = dpp_shr_add<0x104>(v[e]);   // row_shl:4: columns 0..7
             }
             if ((c16 & 3) == 0 && c16 < 4 * M) rp[(wave * R + r) * 4 * M + q * M + (c16 >> 2)] = v;
-            acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+            acc[r][0] = acc[r][1] = accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
         }
         __syncthreads();
         for (int p = wave; p < R * M; p += W) {
@@ -961,7 +1020,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
 #ifdef DMM_TRACE
                 if (i0 + d < 7) { asm volatile("" ::"v"(cw[d][0])); DMM_TRACE_MARK(8 + 2 * (i0 + d)); }
 #endif
-                q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 32u, lane_base, acc, nv);
+                q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 32u, lane_base, acc, accd, nv);
                 if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
                 if (++j >= n_sw) {
                     j = 0;

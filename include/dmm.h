@@ -97,15 +97,19 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
  *                    compute unit.  Weights as fp8 (e4m3) bytes - exact when every grid value
  *                    has at most 4 significant bits in fp8's range, as the E8P grid does - and x
  *                    as four bf8 (e5m2) terms that add up to it exactly; the +-1/4 shift of a
- *                    code is added through the per-code means of x.  Nothing is lost in the
- *                    operands; the 8-bit MFMA adds its products in an adder narrower than fp32,
- *                    so y differs from the 16-bit kernel's by about 2^-14 of a row's scale (the
- *                    tolerance of the operator is 1e-2).  A grid that does not fit fp8, or an x
+ *                    code is added through the per-code means of x (kept to the full fp32 sum
+ *                    at M = 1, rounded to half at M = 2 .. 4).  Nothing is lost in the operands;
+ *                    the 8-bit MFMA aligns the products of a group to the largest of them, so y
+ *                    is not always the 16-bit kernel's bit for bit: at M = 1, 98 % of the outputs
+ *                    are the correctly rounded ones and the rest are one half ulp off (99th
+ *                    percentile of the error 0.57 ulps; the tolerance of the operator is 1e-2,
+ *                    thousands of ulps).  A grid that does not fit fp8, or an x
  *                    that is not finite, is detected inside the launch and served by the 16-bit
  *                    kernel: same call, same status.  DMM_GEMV_8BIT=0 in the environment keeps
  *                    the operator off this kernel.  Domain: that of dmm_gemv_f16 with M <= 4 and
- *                    4 M (K + 16 + K / 8 + 16) bytes of x terms fitting the LDS beside the
- *                    tables (K <= 13 K at M = 1); DMM_ERR_UNSUPPORTED outside.  No counterpart
+ *                    the terms of x and of its means fitting the LDS beside the tables
+ *                    (4 M (K + 16) + T M (K / 8 + 16) bytes, T = 8 at M = 1, else 4: K <= 12544
+ *                    at M = 1); DMM_ERR_UNSUPPORTED outside.  No counterpart
  *                    in the reference (its kernel multiplies int8 by int8). */
 int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float scale,
                       void *y, int64_t M, int64_t N, int64_t K, void *stream);
