@@ -28,9 +28,9 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 # HBM bytes one GEMV launch moves, per kernel, averaged over the shapes of the step that kernel
 # serves: rocprofv3 FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter
 # reads for a plain 256 MiB device copy (x2.000 and x1.000).
-# gemv_q8_kernel: 15,856.2 KiB fetched, 30.9 KiB written per dispatch (32,156,331 code bytes);
-# gemv_stream_kernel: 28,979.6 KiB and 16.0 KiB (58,720,256 code bytes).
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8_kernel": 32502000, "dmm::gemv_stream_kernel": 59361000}
+# gemv_q8_kernel: 15,862.3 KiB fetched, 30.9 KiB written per dispatch (32,156,331 code bytes);
+# gemv_stream_kernel: 28,979.5 KiB and 16.0 KiB (58,720,256 code bytes).
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8_kernel": 32515000, "dmm::gemv_stream_kernel": 59361000}
 
 
 def parse():
