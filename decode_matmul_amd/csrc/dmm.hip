@@ -12,6 +12,7 @@
 // 16x16x32 / 32x32x16 half MFMA.  Nothing decoded ever goes back through memory on the
 // matrix-vector path.
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -2012,13 +2013,18 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
 // The 8-bit kernel, one row tile at a time; the code stream three loads deep per wave when a
 // workgroup has more than two row tiles to walk through, two deep for shorter launches (where
 // a larger first burst only delays the first tile).
-// DMM_GEMV_8BIT=0 in the environment keeps batch 1 on the 16-bit kernel (read once).
+// Whether the operator may pick the 8-bit kernel: dmm_set_gemv_8bit, or DMM_GEMV_8BIT=0 in the
+// environment (read once, at the first call that needs it) for hosts that cannot call it.
+std::atomic<int> g_gemv_q8{-1};
+
 inline bool gemv_q8_enabled()
 {
-    static int on = -1;
+    int on = g_gemv_q8.load(std::memory_order_relaxed);
     if (on < 0) {
         const char *e = getenv("DMM_GEMV_8BIT");
         on = (e && e[0] == '0') ? 0 : 1;
+        int expected = -1;
+        if (!g_gemv_q8.compare_exchange_strong(expected, on)) on = expected;   // a setter came first
     }
     return on == 1;
 }
@@ -2306,6 +2312,13 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
     if (st != DMM_OK || M == 0 || N == 0) return st;
     if (!gemv_ok(x, codes, grid, y, M, N, K)) return DMM_ERR_UNSUPPORTED;
     return run_gemv(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
+}
+
+int dmm_set_gemv_8bit(int enabled)
+{
+    const int before = gemv_q8_enabled() ? 1 : 0;
+    g_gemv_q8.store(enabled ? 1 : 0, std::memory_order_relaxed);
+    return before;
 }
 
 const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K)

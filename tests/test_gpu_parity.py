@@ -198,6 +198,36 @@ def test_gemv_8bit_exact_for_extreme_x():
         assert np.array_equal(y.cpu().numpy().astype(np.float64)[0], want), (i, float(v))
 
 
+def test_gemv_8bit_switch_and_kernel_name():
+    """The operator's choice follows dmm_set_gemv_8bit; with the 8-bit kernel off the result is the
+    16-bit kernel's, i.e. what the explicit 16-bit configuration of the same launch gives."""
+    lib = capi.lib()
+    M, N, K = 1, 8192, 2048                                  # 512 tiles: long enough for the 8-bit kernel
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=11)
+    ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+    was = lib.dmm_set_gemv_8bit(1)
+    try:
+        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_q8_kernel"
+        assert lib.dmm_gemv_kernel_name(M, 4096, K) == b"dmm::gemv_stream_kernel"     # one tile per CU
+        assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_stream_kernel"    # x terms do not fit
+        assert lib.dmm_gemv_kernel_name(32, N, K) == b"dmm::gemv_regx_kernel"
+        assert lib.dmm_gemv_kernel_name(M, N, 264) == b""
+        y8 = c_matmul(dev(x), dev(codes), dev(grid), scale, "auto")
+        assert torch.equal(y8, c_matmul(dev(x), dev(codes), dev(grid), scale, "gemv8"))
+        assert lib.dmm_set_gemv_8bit(0) == 1
+        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_stream_kernel"
+        y16 = c_matmul(dev(x), dev(codes), dev(grid), scale, "auto")
+        torch.cuda.synchronize()
+        assert_close_to_oracle(y8, ref, "8-bit")
+        assert_close_to_oracle(y16, ref, "16-bit")
+        # the 16-bit kernel's y is the correctly rounded product
+        want = (x.numpy().astype(np.float64) @ orc.decode_f16(codes.numpy(), grid.numpy()).astype(np.float64).T) * np.float64(np.float32(scale))
+        assert (y16.cpu().numpy() != want.astype(np.float16)).mean() < 0.005
+        assert (y8.cpu().numpy() != want.astype(np.float16)).mean() < 0.05
+    finally:
+        lib.dmm_set_gemv_8bit(was)
+
+
 def test_gemv_8bit_non_finite_x():
     K, N = 1024, 48
     rng = np.random.default_rng(9)
