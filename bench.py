@@ -219,7 +219,7 @@ def main():
     }
 
     if not args.quick:
-        out["gemv_packed"] = gemv_packed(torch, lib, capi, workload, probs, copies, stream)
+        out["gemv_packed"] = gemv_packed(torch, lib, capi, workload, probs, copies, stream, args.steps)
         out["gemv_7b_shapes"] = gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes)
         out["small_batch"] = small_batch(torch, lib, capi, workload, dev, stream, rand_codes)
         out["prefill"] = prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes)
@@ -244,39 +244,61 @@ def timed_kernel(torch, lib, fn, reps):
     return sum(t) / len(t)
 
 
-def gemv_packed(torch, lib, capi, workload, probs, copies, stream):
+def gemv_packed(torch, lib, capi, workload, probs, copies, stream, steps):
     """The headline step again with the codes repacked offline (dmm_pack_codes: a wave's load is
-    1 KB of consecutive bytes).  Same inputs, bit-identical outputs; kernel durations by events."""
-    rows = []
-    tot_b = tot_t = 0.0
+    1 KB of consecutive bytes).  Same inputs, bit-identical outputs; kernel durations by events,
+    measured like the row-major ones: the four shapes take turns and every launch reads the next
+    of `copies` distinct buffers of its shape, so that the Infinity Cache cannot serve the codes
+    (a loop over one shape alone would cycle through 50 - 176 MB and be served from it in part)."""
+    packed = []
     for p in probs:
         K, N = p["K"], p["N"]
-        packed = []
+        bufs = []
         for c in p["codes"]:
             buf = torch.empty(lib.dmm_packed_bytes(N, K) // 2, dtype=torch.int16, device=c.device)
             st = lib.dmm_pack_codes(c.data_ptr(), buf.data_ptr(), N, K, stream)
             assert st == 0, st
-            packed.append(buf)
-        y = torch.empty_like(p["y"])
+            bufs.append(buf)
+        packed.append(bufs)
+    ys = [torch.empty_like(p["y"]) for p in probs]
 
-        def fn(i):
-            st = lib.dmm_gemv_packed_f16(p["x"].data_ptr(), packed[i % copies].data_ptr(), p["grid"].data_ptr(),
-                                         p["scale"], y.data_ptr(), 1, N, K, stream)
-            assert st == 0, st
-        for i in range(5):
-            fn(i)
+    def fn(k, i):
+        p = probs[k]
+        st = lib.dmm_gemv_packed_f16(p["x"].data_ptr(), packed[k][i % copies].data_ptr(), p["grid"].data_ptr(),
+                                     p["scale"], ys[k].data_ptr(), 1, p["N"], p["K"], stream)
+        assert st == 0, st
+    for k, p in enumerate(probs):        # bit-identity against the row-major call on the same codes
+        fn(k, 1)
+        lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][1 % copies].data_ptr(), p["grid"].data_ptr(), p["scale"],
+                                  p["y"].data_ptr(), 1, p["N"], p["K"], stream)
         torch.cuda.synchronize()
-        lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][4 % copies].data_ptr(), p["grid"].data_ptr(), p["scale"],
-                                  p["y"].data_ptr(), 1, N, K, stream)
-        torch.cuda.synchronize()
-        assert torch.equal(y, p["y"]), "packed and row-major results differ"
-        t = timed_kernel(torch, lib, fn, 50)
-        b = workload.code_bytes(N, K)
+        assert torch.equal(ys[k], p["y"]), "packed and row-major results differ"
+    for i in range(3):
+        for k in range(len(probs)):
+            fn(k, i)
+    n = steps * len(probs)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for a, b in ev:
+        a.record(); b.record()
+    torch.cuda.synchronize()
+    j = 0
+    for i in range(steps):
+        for k in range(len(probs)):
+            lib.dmm_set_kernel_events(ev[j][0].cuda_event, ev[j][1].cuda_event)
+            fn(k, i)
+            j += 1
+    lib.dmm_set_kernel_events(None, None)
+    torch.cuda.synchronize()
+    rows = []
+    tot_b = tot_t = 0.0
+    for k, p in enumerate(probs):
+        v = [ev[i * len(probs) + k][0].elapsed_time(ev[i * len(probs) + k][1]) * 1e-3 for i in range(steps)]
+        t = sum(v) / len(v)
+        b = workload.code_bytes(p["N"], p["K"])
         tot_b += b
         tot_t += t
-        rows.append({"K": K, "N": N, "kernel_us": round(t * 1e6, 3), "GBps": round(b / t / 1e9, 1),
+        rows.append({"K": p["K"], "N": p["N"], "kernel_us": round(t * 1e6, 3), "GBps": round(b / t / 1e9, 1),
                      "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBS, 4)})
-        del packed
     return {"shapes": rows, "achieved_GBps": round(tot_b / tot_t / 1e9, 2),
             "frac_hbm": round(tot_b / tot_t / 1e9 / HBM_PEAK_GBS, 4)}
 
