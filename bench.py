@@ -304,11 +304,11 @@ def gemv_packed(torch, lib, capi, workload, probs, copies, stream, steps):
 
 
 def gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes):
-    """configs[1]: batch-1 GEMV at the Llama-2-7B projection shapes, 30 code buffers in rotation
-    per shape (> 256 MB except 4096 -> 4096: 126 MB)."""
+    """configs[1]: batch-1 GEMV at the Llama-2-7B projection shapes, enough code buffers in
+    rotation per shape (30 or more, at least 320 MB) that the 256 MB Infinity Cache cannot serve them."""
     rows = []
     for K, N in workload.LLAMA2_7B:
-        copies = 30
+        copies = max(30, -(-320_000_000 // workload.code_bytes(N, K)))
         codes = rand_codes(N, K, copies, 7)
         x, _, grid, scale = workload.make_inputs(1, 8, K, seed=0)
         x, grid = x.to(dev), grid.to(dev)
