@@ -634,6 +634,14 @@ __device__ __forceinline__ u2_t lds_read8(uint32_t byte_addr)
 
 // terms of x, terms of the means, and one word per wave for the vote on the grid
 __host__ __device__ constexpr int q8_mean_terms(int64_t M) { return M == 1 ? 8 : 4; }
+// Partial sums of a row block, two parities.  M > 1: one float4 per (wave, tile, quarter, x row), the
+// term columns already added by the wave.  M == 1: all 8 columns per (wave, tile, quarter), added
+// (with their weights) by the one wave that sums the block up; a wave's slots are padded by one
+// float4 so that the 16 waves' slots fall in 16 different bank groups.
+__host__ __device__ constexpr int q8_red_bytes(int R, int W, int M)
+{
+    return M == 1 ? 2 * W * (R * 4 * 8 + 1) * 16 : 2 * W * R * 4 * M * 16;
+}
 __host__ __device__ constexpr int64_t q8_x_bytes(int64_t M, int64_t K)
 {
     return 4 * M * (K + 16) + q8_mean_terms(M) * M * (K / 8 + 16) + 64;
@@ -832,9 +840,9 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
     if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     DMM_TRACE_MARK(0);
-    f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // [2][W][R][4 * M]
-    const int red_par = W * R * 4 * M;                                 // float4 per parity
-    unsigned char *xt = smem_raw + kSTablesBytes + stream_red_bytes(R, W, M);
+    f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // two parities, see q8_red_bytes
+    const int red_par = q8_red_bytes(R, W, M) / 32;                    // float4 per parity
+    unsigned char *xt = smem_raw + kSTablesBytes + q8_red_bytes(R, W, M);
     // M == 1: eight terms of the means in columns 0..7 (the shift term has an accumulator of its
     // own, so columns 4..7 of the main one are simply not used); M > 1: four terms, column
     // 4 m + t like x
@@ -973,6 +981,37 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
 
     auto finish_block = [&](int blk) {
         f4_t *rp = red + (blk & 1) * red_par;
+        if (M == 1) {
+            // Batch 1: the wave only leaves its 8 columns (x terms in 0..3, the later terms of the
+            // means in 4..7, where the main accumulators hold nothing of use) ...
+            const float x_mask = c16 < 4 ? 1.f : 0.f;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const f4_t v = (acc[r][0] + acc[r][1]) * x_mask + accd[r];
+                if (c16 < 8) rp[wave * (R * 32 + 1) + (r * 4 + q) * 8 + c16] = v;
+                acc[r][0] = acc[r][1] = accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
+            }
+            __syncthreads();
+            // ... and one wave per tile adds them up: lane (w, quarter) takes wave w's 8 columns with
+            // their weights 8^-c, then the 16 lanes of a row are added with DPP shifts
+            for (int r = wave; r < R; r += W) {
+                const f4_t *src = rp + c16 * (R * 32 + 1) + (r * 4 + q) * 8;
+                f4_t v = src[0];
+#pragma unroll
+                for (int c = 1; c < 8; c++) v += src[c] * __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)c * 3u << 23));
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
+                const int tile = t0 + blk * R + r;
+                const int n = tile * 16 + 4 * q;
+                if (c16 == 15 && tile < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
+                    h4_t o;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
+                    *reinterpret_cast<h4_t *>(y + n) = o;
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < R; r++) {
             // the four term columns of an x row are added first, each with the weight of its term:
@@ -982,14 +1021,13 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             for (int e = 0; e < 4; e++) {
                 v[e] = dpp_shr_add<0x101>(v[e]);   // row_shl:1
                 v[e] = dpp_shr_add<0x102>(v[e]);   // row_shl:2
-                if (M == 1) v[e] = dpp_shr_add<0x104>(v[e]);   // row_shl:4: columns 0..7
             }
             if ((c16 & 3) == 0 && c16 < 4 * M) rp[(wave * R + r) * 4 * M + q * M + (c16 >> 2)] = v;
             acc[r][0] = acc[r][1] = accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
         }
         __syncthreads();
         for (int p = wave; p < R * M; p += W) {
-            const int r = M == 1 ? p : p / M, m = p - r * M;
+            const int r = p / M, m = p - r * M;
             f4_t v = f4_t{0.f, 0.f, 0.f, 0.f};
             if (c16 < W) v = rp[(c16 * R + r) * 4 * M + q * M + m];
 #pragma unroll
@@ -1966,7 +2004,7 @@ int launch_gemv_stream(const void *x, const void *codes, const void *grid, float
 template <int R, int W>
 bool gemv_q8_ok(int64_t M, int64_t N, int64_t K)
 {
-    return M <= 4 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + q8_x_bytes(M, K) <= 160 * 1024 &&
+    return M <= 4 && (int64_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + q8_x_bytes(M, K) <= 160 * 1024 &&
            N * (K >> 2) < (1LL << 31);
 }
 
@@ -1978,7 +2016,7 @@ int launch_gemv_q8(const void *x, const void *codes, const void *grid, float sca
 #ifdef DMM_TRACE
     const size_t shmem = 160 * 1024;
 #else
-    const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
+    const size_t shmem = (size_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
 #endif
     static bool attr_done[kMaxDevices] = {};
     if (int e = allow_dynamic_lds(gemv_q8_kernel<R, W, D, kPacked>, 160 * 1024, attr_done)) return e;

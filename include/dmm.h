@@ -106,11 +106,12 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
  *                    thousands of ulps).  A grid that does not fit fp8, or an x
  *                    that is not finite, is detected inside the launch and served by the 16-bit
  *                    kernel: same call, same status.  dmm_set_gemv_8bit(0), or DMM_GEMV_8BIT=0
- *                    in the environment, keeps the operator off this kernel.  Domain: that of dmm_gemv_f16 with M <= 4 and
- *                    the terms of x and of its means fitting the LDS beside the tables
- *                    (4 M (K + 16) + T M (K / 8 + 16) bytes, T = 8 at M = 1, else 4: K <= 12544
- *                    at M = 1); DMM_ERR_UNSUPPORTED outside.  No counterpart
- *                    in the reference (its kernel multiplies int8 by int8). */
+ *                    in the environment, keeps the operator off this kernel.  Domain: that of
+ *                    dmm_gemv_f16 with M <= 4 and the terms of x and of its means fitting the
+ *                    LDS beside the tables and the partial sums (4 M (K + 16) + T M (K / 8 + 16)
+ *                    bytes, T = 8 at M = 1, else 4: K <= 9472 at M = 1); DMM_ERR_UNSUPPORTED
+ *                    outside.  No counterpart in the reference (its kernel multiplies int8 by
+ *                    int8). */
 int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float scale,
                       void *y, int64_t M, int64_t N, int64_t K, void *stream);
 /* Process-wide switch for the 8-bit kernel in the operator's choice (explicit calls of
