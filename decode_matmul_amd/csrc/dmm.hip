@@ -783,8 +783,10 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
             const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
             acc[0][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[0][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
         }
-        const uint32_t a8lo = ((cw[0][0] >> 8) & 0x00800080u) | (cw[0][1] & 0x80008000u) | 0x40404040u;
-        const uint32_t a8hi = ((cw[0][2] >> 8) & 0x00800080u) | (cw[0][3] & 0x80008000u) | 0x40404040u;
+        // the top bytes of the four codes of two words, in the order codes 0, 2, 1, 3 (the means are
+        // stored in the same order): shift bit = sign of +-2.0
+        const uint32_t a8lo = (__builtin_amdgcn_perm(cw[0][1], cw[0][0], 0x07030501u) & 0x80808080u) | 0x40404040u;
+        const uint32_t a8hi = (__builtin_amdgcn_perm(cw[0][3], cw[0][2], 0x07030501u) & 0x80808080u) | 0x40404040u;
         accd[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]), accd[0], 0, 0, 0);
         return;
     }
