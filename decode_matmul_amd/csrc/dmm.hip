@@ -757,19 +757,19 @@ template <int R>
 __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t x8addr, uint32_t lane_base,
                                         f4_t (&acc)[R][2], f4_t (&accd)[R], int nv)
 {
-    constexpr int kItems = 4 * R;
-    if constexpr (R == 1) {
-        // one tile: all 16 table gathers and the 5 reads of x of the step go out first (8-byte
-        // results: 48 registers), so the wave meets the LDS latency once per step, not once
-        // per word
-        Q8Gather g[4];
-        u4_t xq[4];
+    // All 16 table gathers of a tile's step and the 5 reads of x go out before the first MFMA
+    // (8-byte results: 48 registers), so the wave meets the LDS latency once per step and tile,
+    // not once per word; with two tiles the reads of x serve both.
+    u4_t xq[4];
 #pragma unroll
-        for (int t2 = 0; t2 < 4; t2++) {
-            xq[t2] = lds_read16(xaddr + t2 * 16);
-            q8_gather(g[t2], cw[0][t2], lane_base);
-        }
-        const u2_t x8 = lds_read8(x8addr);
+    for (int t2 = 0; t2 < 4; t2++) xq[t2] = lds_read16(xaddr + t2 * 16);
+    const u2_t x8 = lds_read8(x8addr);
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (r > 0 && r >= nv) break;   // tiles past nv: nothing to do (uniform)
+        Q8Gather g[4];
+#pragma unroll
+        for (int t2 = 0; t2 < 4; t2++) q8_gather(g[t2], cw[r][t2], lane_base);
         // two words = four codes = 32 consecutive k of the lane's 64: one 16x16x128 MFMA (32
         // bytes per lane and operand, A fp8, B bf8, no scaling), which does four times the work
         // of the 16x16x32 form in twice its time
@@ -781,52 +781,13 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
                                 (int)(b1.g1[0] ^ b1.s1[0]), (int)(b1.g1[1] ^ b1.s1[1])};
             const u4_t &x0 = xq[2 * h], &x1 = xq[2 * h + 1];
             const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
-            acc[0][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[0][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
+            acc[r][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[r][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
         }
-        // the top bytes of the four codes of two words, in the order codes 0, 2, 1, 3 (the means are
-        // stored in the same order): shift bit = sign of +-2.0
-        const uint32_t a8lo = (__builtin_amdgcn_perm(cw[0][1], cw[0][0], 0x07030501u) & 0x80808080u) | 0x40404040u;
-        const uint32_t a8hi = (__builtin_amdgcn_perm(cw[0][3], cw[0][2], 0x07030501u) & 0x80808080u) | 0x40404040u;
-        accd[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]), accd[0], 0, 0, 0);
-        return;
-    }
-    Q8Gather buf[2];
-    u4_t xb[2];
-    xb[0] = lds_read16(xaddr);
-    q8_gather(buf[0], cw[0][0], lane_base);
-    const u2_t x8 = lds_read8(x8addr);
-#pragma unroll
-    for (int i = 0; i < kItems; i++) {
-        const int t2 = i / R, r = i % R;
-        if (i + 1 < kItems) {
-            const int nt2 = (i + 1) / R, nr = (i + 1) % R;
-            if (nr == 0) {
-                xb[nt2 & 1] = lds_read16(xaddr + nt2 * 16);
-                q8_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base);
-            } else if (nr < nv) {
-                q8_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base);
-            }
-        }
-        if (r == 0 || r < nv) {
-            const Q8Gather &b = buf[i & 1];
-            const u4_t &xv = xb[t2 & 1];
-            acc[r][0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(b.g0[0] ^ b.s0[0], b.g0[1] ^ b.s0[1]),
-                                                                   q8_pack(xv[0], xv[1]), acc[r][0], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            acc[r][1] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(b.g1[0] ^ b.s1[0], b.g1[1] ^ b.s1[1]),
-                                                                   q8_pack(xv[2], xv[3]), acc[r][1], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (t2 == 3) {
-                // the shift term: byte order of the A operand is codes 0, 2, 1, 3 | 4, 6, 5, 7 of the
-                // lane's eight (bit 15 of a word lands in byte 1 or, shifted, byte 0; bit 31 in
-                // byte 3 or byte 2) - the means are stored in the same order
-                const uint32_t a8lo = ((cw[r][0] >> 8) & 0x00800080u) | (cw[r][1] & 0x80008000u) | 0x40404040u;
-                const uint32_t a8hi = ((cw[r][2] >> 8) & 0x00800080u) | (cw[r][3] & 0x80008000u) | 0x40404040u;
-                accd[r] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]),
-                                                                     accd[r], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
+        // the shift term: the top bytes of the four codes of two words, in the order codes 0, 2, 1, 3
+        // (the means are stored in the same order); shift bit = sign of +-2.0
+        const uint32_t a8lo = (__builtin_amdgcn_perm(cw[r][1], cw[r][0], 0x07030501u) & 0x80808080u) | 0x40404040u;
+        const uint32_t a8hi = (__builtin_amdgcn_perm(cw[r][3], cw[r][2], 0x07030501u) & 0x80808080u) | 0x40404040u;
+        accd[r] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]), accd[r], 0, 0, 0);
     }
 }
 
