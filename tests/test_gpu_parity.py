@@ -200,6 +200,40 @@ def test_gemv_8bit_exact_for_extreme_x():
         assert np.array_equal(y.cpu().numpy().astype(np.float64)[0], want), (i, float(v))
 
 
+def _random_8bit_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        M = int(rng.integers(1, 5))
+        K = 256 * int(rng.integers(1, 38))
+        red = 2 * 16 * 33 * 16 if M == 1 else 2 * 16 * 4 * M * 16
+        if 96 * 1024 + red + 4 * M * (K + 16) + (8 if M == 1 else 4) * M * (K // 8 + 16) + 64 > 160 * 1024:
+            continue
+        N = 4 * int(rng.integers(1, 1400)) if len(out) % 3 else 4 * int(rng.integers(1100, 2600))
+        out.append((M, N, K))
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", _random_8bit_cases(30, 4242))
+def test_gemv_8bit_random_shapes(M, N, K):
+    """Seeded random shapes of the 8-bit kernel's whole domain (ragged last tiles, a single k step,
+    the largest x that fits), fp8-exact grids, y inside a guarded buffer."""
+    rng = np.random.default_rng(M * 1000003 + N * 101 + K)
+    fp8_vals = np.array([0.0, 0.25, 0.5, 0.75, 1.0, 1.25, 1.5, 1.75, 2.25, 2.5, 2.75, 3.5, 5.0, 7.5, 0.015625, 0.109375])
+    grid = (rng.choice(fp8_vals, size=(256, 8)) * rng.choice([-1.0, 1.0], size=(256, 8))).astype(np.float16)
+    x = (rng.standard_normal((M, K)) * rng.choice([0.01, 1.0, 30.0])).astype(np.float16)
+    codes = rng.integers(0, 65536, size=(N, K // 8)).astype(np.uint16)
+    scale = float(np.float32(1.0 / (np.sqrt(K) * max(1e-3, float(np.abs(x.astype(np.float64)).mean())))))
+    ref = orc.matmul_f32(x, orc.decode_f16(codes, grid), scale)
+    guard = 64
+    buf = torch.full((M * N + 2 * guard,), 777.0, dtype=torch.float16, device=DEV)
+    y = buf[guard:guard + M * N].view(M, N)
+    c_matmul(dev(x), dev(codes), dev(grid), scale, "gemv8", out=y)
+    torch.cuda.synchronize()
+    assert_close_to_oracle(y, ref, "8-bit random M=%d N=%d K=%d" % (M, N, K))
+    assert torch.all(buf[:guard] == 777.0) and torch.all(buf[guard + M * N:] == 777.0)
+
+
 def test_gemv_8bit_switch_and_kernel_name():
     """The operator's choice follows dmm_set_gemv_8bit; with the 8-bit kernel off the result is the
     16-bit kernel's, i.e. what the explicit 16-bit configuration of the same launch gives."""
