@@ -297,7 +297,9 @@ def test_empty_problems():
 
 # ----------------------------------------------------------------- exact integer bridge
 @pytest.mark.parametrize("path,M,N,K", [("gemv", 8, 16, 4096), ("gemm", 8, 16, 4096), ("generic", 8, 16, 4096),
-                                         ("gemv", 1, 64, 8192), ("gemm", 64, 64, 8192)])
+                                         ("gemv", 1, 64, 8192), ("gemm", 64, 64, 8192),
+                                         ("gemv8", 1, 64, 8192), ("gemv8", 1, 8192, 2048), ("gemv8", 3, 4100, 4096),
+                                         ("auto", 1, 8192, 8192)])
 def test_integer_bridge_is_exact(path, M, N, K):
     """x integer-valued, grid = E8P bytes / 4, scale a power of two: every partial sum is a
     multiple of 1/4 below 2^24 quarters, so fp32 accumulation in any order is exact and the
