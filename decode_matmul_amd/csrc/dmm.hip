@@ -288,26 +288,31 @@ constexpr int kSTablesBytes = kSSignBytes + kSGridBytes;
 
 __host__ __device__ constexpr int stream_red_bytes(int R, int W, int M) { return 2 * W * R * 4 * M * 16; }
 
-// Table staging: thread tid fetches ONE grid row (row tid % 256) and writes 4096 / kNThreads
-// of its 16 copies (stream_stage_grid); the 2048 sign slots are computed, 2048 / kNThreads per
-// thread (stream_stage_signs: needs no load, so it runs while the loads are in flight).
+// Table staging.  Every instruction of the prologue is paid once per wave that runs it, so the
+// two tables go to different waves instead of a share of each to every thread: the first 256
+// threads (waves 0-3) fetch one grid row each and write its 16 copies, the next 256 (waves 4-7)
+// compute the sign rows (thread t: row t / 2, 8 of its 16 copies; needs no load, so it runs
+// while the loads are in flight).  16 neighbouring lanes always write 16 different copy
+// positions, i.e. 16 bank groups.
 template <int kNThreads>
 __device__ __forceinline__ void stream_stage_signs(unsigned char *smem, int tid)
 {
-    u4_t *sg = reinterpret_cast<u4_t *>(smem);
+    static_assert(kNThreads >= 512, "staging assumes at least 8 waves");
+    if (tid < 256 || tid >= 512) return;
+    const int t = tid - 256, row = t >> 1;
+    const u4_t sv = sign_row((uint32_t)row);
+    u4_t *sg = reinterpret_cast<u4_t *>(smem) + row * 16 + (t & 1) * 8;
 #pragma unroll
-    for (int i = 0; i < 2048 / kNThreads; i++) sg[tid + i * kNThreads] = sign_row((uint32_t)((tid + i * kNThreads) >> 4));
+    for (int i = 0; i < 8; i++) sg[(i + row) & 7] = sv;
 }
 
 template <int kNThreads>
 __device__ __forceinline__ void stream_stage_grid(unsigned char *smem, const u4_t &grow, int tid)
 {
-    static_assert(kNThreads == 512 || kNThreads == 1024, "staging assumes 512 or 1024 threads");
-    constexpr int kCopiesPer = 4096 / kNThreads;          // copies of its row a thread writes
-    u4_t *gg = reinterpret_cast<u4_t *>(smem + kSSignBytes);
-    const int row = tid & 255, c0 = (tid >> 8) * kCopiesPer;
+    if (tid >= 256) return;
+    u4_t *gg = reinterpret_cast<u4_t *>(smem + kSSignBytes) + tid * 16;
 #pragma unroll
-    for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + ((c0 + i + tid) & 15)] = grow;   // 16 lanes, 16 bank groups
+    for (int i = 0; i < 16; i++) gg[(i + tid) & 15] = grow;
 }
 
 // Sum over each row of 16 lanes, result in lane 15 of the row (all 64 lanes must be active).
@@ -426,7 +431,7 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
     // ---- prologue: this thread's grid row and its share of x first (short latency, nothing
     // queued in front of them), then the first D items of the code stream; the tables and the
     // LDS copy of x are built while the code loads fly ---------------------------------------
-    const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid & 255];
+    const u4_t grow = tid < 256 ? reinterpret_cast<const u4_t *>(grid)[tid] : u4_t{0u, 0u, 0u, 0u};   // waves 0-3 stage the grid
     const int row_chunks = K >> 3;                     // 16-byte pieces per row of x
     constexpr int kXPer = 4;                           // pieces of row 0 per thread fetched up front
     u4_t xv[kXPer];
