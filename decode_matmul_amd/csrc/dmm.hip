@@ -2016,9 +2016,6 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
 
-// The 8-bit kernel, one row tile at a time; the code stream three loads deep per wave when a
-// workgroup has more than two row tiles to walk through, two deep for shorter launches (where
-// a larger first burst only delays the first tile).
 // Whether the operator may pick the 8-bit kernel: dmm_set_gemv_8bit, or DMM_GEMV_8BIT=0 in the
 // environment (read once, at the first call that needs it) for hosts that cannot call it.
 std::atomic<int> g_gemv_q8{-1};
@@ -2035,6 +2032,9 @@ inline bool gemv_q8_enabled()
     return on == 1;
 }
 
+// The 8-bit kernel, one row tile at a time; the code stream three loads deep per wave when a
+// workgroup has more than two row tiles to walk through, two deep for shorter launches (where
+// a larger first burst only delays the first tile).
 template <bool kPacked>
 int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                 int64_t N, int64_t K, hipStream_t stream)
@@ -2044,18 +2044,18 @@ int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale,
     return launch_gemv_q8<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
 }
 
-// The choice among the matrix-vector kernels.  At most one row tile per workgroup: the 16-bit
-// streaming kernel, one tile at a time (its prologue is the cheaper one and there is no steady
-// state to speak of).  More: the 8-bit kernel where it applies, else the 16-bit one two tiles
-// at a time; the register-x kernel when x does not fit the LDS.
-enum GemvKind { kGemvStreamShort, kGemvQ8, kGemvStream, kGemvRegx };
+// The choice among the matrix-vector kernels.  Launches of more than three row tiles per
+// workgroup: the 8-bit kernel where it applies (14 % faster at seven tiles, 2 % at two and a
+// half - below that its dearer prologue is not won back, and the 16-bit kernel's y is the
+// correctly rounded one).  Otherwise the 16-bit streaming kernel, one tile at a time (two at a
+// time is 6 - 10 % slower at K = 8192); the register-x kernel when x does not fit the LDS.
+enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
 
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
-    const bool short_launch = (N + 15) / 16 <= cu_count();
-    if (short_launch && gemv_stream_ok<1, 16>(M, N, K)) return kGemvStreamShort;
-    if (gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return kGemvQ8;
-    if (gemv_stream_ok<2, 16>(M, N, K)) return kGemvStream;
+    const bool long_launch = (N + 15) / 16 > 3 * (int64_t)cu_count();
+    if (long_launch && gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return kGemvQ8;
+    if (gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
     return kGemvRegx;
 }
 
@@ -2064,9 +2064,8 @@ int run_gemv_auto(const void *x, const void *codes, const void *grid, float scal
                   int64_t N, int64_t K, hipStream_t stream)
 {
     switch (pick_gemv(M, N, K)) {
-        case kGemvStreamShort: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        case kGemvStream: return launch_gemv_stream<2, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         default: return launch_gemv_regx<2, 8, 1, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
     }
 }
@@ -2332,7 +2331,6 @@ const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K)
     if (M < 1 || M > 32 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31)) return "";
     if (M > 16) return "dmm::gemv_regx_kernel";
     switch (pick_gemv(M, N, K)) {
-        case kGemvStreamShort:
         case kGemvStream: return "dmm::gemv_stream_kernel";
         case kGemvQ8: return "dmm::gemv_q8_kernel";
         default: return "dmm::gemv_regx_kernel";

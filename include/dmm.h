@@ -93,9 +93,10 @@ int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid,
 int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale,
                  void *y, int64_t M, int64_t N, int64_t K, void *stream);
 /*   dmm_gemv_8bit_f16  the matrix-vector kernel on 8-bit MFMA operands, which dmm_gemv_f16 and
- *                    the operator pick for M <= 4 on launches of more than one 16-row tile per
- *                    compute unit.  Weights as fp8 (e4m3) bytes - exact when every grid value
- *                    has at most 4 significant bits in fp8's range, as the E8P grid does - and x
+ *                    the operator pick for M <= 4 on launches of more than three 16-row tiles
+ *                    per compute unit (shorter ones gain nothing from it).  Weights as fp8
+ *                    (e4m3) bytes - exact when every grid value has at most 4 significant bits
+ *                    in fp8's range, as the E8P grid does - and x
  *                    as four bf8 (e5m2) terms that add up to it exactly; the +-1/4 shift of a
  *                    code is added through the per-code means of x (kept to the full fp32 sum
  *                    at M = 1, rounded to half at M = 2 .. 4).  Nothing is lost in the operands;
