@@ -2066,7 +2066,7 @@ int run_gemv_auto(const void *x, const void *codes, const void *grid, float scal
     switch (pick_gemv(M, N, K)) {
         case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        default: return launch_gemv_regx<2, 8, 1, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return launch_gemv_regx<2, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
     }
 }
 
