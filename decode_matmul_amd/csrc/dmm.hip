@@ -605,51 +605,50 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__r
 //     v_mfma_f32_16x16x128_f8f6f4 (four codes = 32 consecutive k per lane; twice the time of the
 //     16x16x32 form for four times the work) as they are.  d is left out of the decode and added by the
 //     matrix unit instead: sum_k d x[k] = sum over codes of (8 d) * (mean of the code's 8 x
-//     values), one more MFMA per 16 rows x 256 k (into an accumulator of its own) whose A
-//     operand is +-2.0 per code, made from the code words themselves (shift bit = sign bit of
-//     the byte);
+//     values), one more MFMA (the 16-bit 16x16x32 form) per 16 rows x 256 k, into an
+//     accumulator of its own, whose A operand is +-2.0 per code, made from the code words
+//     themselves (the shift bit is the sign bit of a half), and whose B operand is the means as
+//     two halves, hi + lo (22 bits of the fp32 sum of the 8 values), in two columns;
 //   * x.  A half with a zero low byte IS a bf8 (e5m2) number in its high byte.  Cutting x after
 //     its top byte, subtracting, scaling what is left by 8 and repeating gives
 //     x = t0 + t1 / 8 + t2 / 64 + t3 / 512 exactly for every normal x (3 significant bits per
 //     term, 11 in a half); the four terms sit in four B columns - at batch 1 the other 15
 //     columns of the 16-wide tile are idle anyway - and the four result columns are added, with
-//     those weights, at the end.  The per-code means (fp32 sum of 8, times 1/8, rounded to
-//     half) are split the same way.
+//     those weights, at the end.
 // s g + d is exact in half for every fp8 g and the terms of x add up to x (subnormal x may lose
 // bits below 2^-24 * 4), so nothing is lost in the operands, and the products are exact in the
-// fp32 accumulators.  Two things remain: the means (at M = 1 they are carried in eight terms,
-// i.e. to the full fp32 sum; at M = 2 .. 4, where the columns are needed for x, in four, i.e.
-// rounded to half), and the matrix unit's adder, which aligns the products of a group to the
-// largest of them.  Measured against the fp64 reference on the benchmark's inputs at M = 1: 98 %
+// fp32 accumulators.  Two things remain: the means (hi + lo drops what lies 22 bits below the
+// leading one of a mean) and the matrix unit's adder, which aligns the products of a group to
+// the largest of them.  Measured against the fp64 reference on the benchmark's inputs: 98 %
 // of the outputs are the correctly rounded ones and the 99th percentile of the error is 0.57
 // half ulps (the 16-bit kernel: 0.5, the output rounding alone); with 100-fold outliers in x
-// 2.6 ulps; x with few significant bits: every output correctly rounded.  At M = 2 .. 4 the
-// rounded means bring it to 1.5 ulps.  All of it a hundredth of the operator's tolerance of
-// 1e-2 or less.  A grid with a value fp8 cannot hold is found while the table is built
+// 2.6 ulps; x with few significant bits: every output correctly rounded.  All of it a
+// hundredth of the operator's tolerance of 1e-2 or less.  A grid with a value fp8 cannot hold is found while the table is built
 // (convert, convert back, compare), an x that is not finite while it is split; every workgroup
 // then runs the 16-bit kernel above instead: same launch, same result as that kernel gives.
 // LDS map: [0, 32K) sign rows (128 x 32 copies x 8 B), [32K, 96K) grid rows (256 x 32 copies x
 // 8 B; a lane reads copy lane % 32, conflict-free for any codes), partial sums, then the terms
-// of x (column m * 4 + t, pitch K + 16 bytes) and of the means (pitch K / 8 + 16).
+// of x (column m * 4 + t, pitch K + 16 bytes) and the means (rows 2 m: hi, 2 m + 1: lo; K / 8
+// halves each, pitch K / 4 + 16 bytes).
 typedef __attribute__((address_space(3))) const u2_t lds_u2_t;
 __device__ __forceinline__ u2_t lds_read8(uint32_t byte_addr)
 {
     return *reinterpret_cast<lds_u2_t *>(byte_addr);
 }
 
-// terms of x, terms of the means, and one word per wave for the vote on the grid
-__host__ __device__ constexpr int q8_mean_terms(int64_t M) { return M == 1 ? 8 : 4; }
 // Partial sums of a row block, two parities.  M > 1: one float4 per (wave, tile, quarter, x row), the
-// term columns already added by the wave.  M == 1: all 8 columns per (wave, tile, quarter), added
+// term columns already added by the wave.  M == 1: the 4 columns per (wave, tile, quarter), added
 // (with their weights) by the one wave that sums the block up; a wave's slots are padded by one
 // float4 so that the 16 waves' slots fall in 16 different bank groups.
 __host__ __device__ constexpr int q8_red_bytes(int R, int W, int M)
 {
-    return M == 1 ? 2 * W * (R * 4 * 8 + 1) * 16 : 2 * W * R * 4 * M * 16;
+    return M == 1 ? 2 * W * (R * 4 * 4 + 1) * 16 : 2 * W * R * 4 * M * 16;
 }
+// terms of x (4 rows of K bytes per x row), the per-code means of x as two halves each (hi + lo:
+// 2 rows of K / 8 halves per x row), and one word per wave for the vote on the grid
 __host__ __device__ constexpr int64_t q8_x_bytes(int64_t M, int64_t K)
 {
-    return 4 * M * (K + 16) + q8_mean_terms(M) * M * (K / 8 + 16) + 64;
+    return 4 * M * (K + 16) + 2 * M * (K / 4 + 16) + 64;
 }
 
 // the 8 sign flags of a sign-row index as bytes: dims 0-3 in [0], 4-7 in [1]
@@ -714,26 +713,18 @@ __device__ __forceinline__ bool split_piece_bf8(const u4_t &v, u2_t (&t)[4])
     return finite;
 }
 
-// The mean of the 8 halves of a piece (fp32 sum, times 1/8) as eight bf8 terms,
-// mean = sum_t term[t] / 8^t, term t in byte t % 4 of word t / 4.  The split runs in fp32: a
-// term is the top byte of the half nearest to what is left (it may overshoot: the remainder is
-// signed), the remainder is scaled by 8 - eight terms of 3 significant bits carry the 24 bits
-// of the fp32 mean.  Four terms (the first word) are the mean to half precision.
-__device__ __forceinline__ u2_t piece_mean_bf8(const u4_t &v)
+// The mean of the 8 halves of a piece (fp32 sum, times 1/8) as two halves, hi + lo: 22 of the
+// fp32 sum's 24 bits.  Low half of the result: hi.
+__device__ __forceinline__ uint32_t piece_mean_hi_lo(const u4_t &v)
 {
     const h2_t ones = h2_t{(half_t)1.0f, (half_t)1.0f};
     float r = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) r = __builtin_amdgcn_fdot2(as_h2(v[i]), ones, r, false);
     r *= 0.125f;
-    u2_t out = u2_t{0u, 0u};
-#pragma unroll
-    for (int term = 0; term < 8; term++) {
-        const uint32_t hi = (uint32_t)__builtin_bit_cast(uint16_t, (half_t)r) & 0xFF00u;
-        out[term >> 2] |= (hi >> 8) << (8 * (term & 3));
-        if (term < 7) r = (r - (float)__builtin_bit_cast(half_t, (uint16_t)hi)) * 8.0f;
-    }
-    return out;
+    const half_t hi = (half_t)r;
+    const half_t lo = (half_t)(r - (float)hi);
+    return as_u32(h2_t{hi, lo});
 }
 
 struct Q8Gather {
@@ -757,7 +748,7 @@ __device__ __forceinline__ long q8_pack(uint32_t lo, uint32_t hi)
 
 // One 256-wide k step for the first nv (uniform, 1 <= nv <= R) of R row tiles; same item order
 // as stream_step.  xaddr: this lane's x terms of the step (16 bytes per word pair: the B
-// operands of its two codes), x8addr: its 8 means.
+// operands of its two codes), x8addr: the means of its 8 codes (8 halves: hi or lo, by column).
 template <int R>
 __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t x8addr, uint32_t lane_base,
                                         f4_t (&acc)[R][2], f4_t (&accd)[R], int nv)
@@ -768,7 +759,7 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
     u4_t xq[4];
 #pragma unroll
     for (int t2 = 0; t2 < 4; t2++) xq[t2] = lds_read16(xaddr + t2 * 16);
-    const u2_t x8 = lds_read8(x8addr);
+    const u4_t x8 = lds_read16(x8addr);
 #pragma unroll
     for (int r = 0; r < R; r++) {
         if (r > 0 && r >= nv) break;   // tiles past nv: nothing to do (uniform)
@@ -788,11 +779,10 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
             const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
             acc[r][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[r][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
         }
-        // the shift term: the top bytes of the four codes of two words, in the order codes 0, 2, 1, 3
-        // (the means are stored in the same order); shift bit = sign of +-2.0
-        const uint32_t a8lo = (__builtin_amdgcn_perm(cw[r][1], cw[r][0], 0x07030501u) & 0x80808080u) | 0x40404040u;
-        const uint32_t a8hi = (__builtin_amdgcn_perm(cw[r][3], cw[r][2], 0x07030501u) & 0x80808080u) | 0x40404040u;
-        accd[r] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(q8_pack(a8lo, a8hi), q8_pack(x8[0], x8[1]), accd[r], 0, 0, 0);
+        // the shift term, in 16-bit arithmetic: +-2.0 per code (a code word with everything but its
+        // shift bits replaced by the bits of 2.0) against the means
+        const u4_t a8 = (cw[r] & 0x80008000u) | 0x40004000u;
+        accd[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8_t, a8), __builtin_bit_cast(h8_t, x8), accd[r], 0, 0, 0);
     }
 }
 
@@ -811,11 +801,9 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // two parities, see q8_red_bytes
     const int red_par = q8_red_bytes(R, W, M) / 32;                    // float4 per parity
     unsigned char *xt = smem_raw + kSTablesBytes + q8_red_bytes(R, W, M);
-    // M == 1: eight terms of the means in columns 0..7 (the shift term has an accumulator of its
-    // own, so columns 4..7 of the main one are simply not used); M > 1: four terms, column
-    // 4 m + t like x
-    const int n_mt = q8_mean_terms(M);
-    const int xt_pitch = K + 16, x8_pitch = (K >> 3) + 16;
+    // the means: rows 2 m (hi) and 2 m + 1 (lo) of K / 8 halves; the shift term has an accumulator of
+    // its own, where they sit in columns 4 m and 4 m + 1
+    const int xt_pitch = K + 16, x8_pitch = (K >> 2) + 16;
     unsigned char *x8t = xt + 4 * M * xt_pitch;
 
     const int tid = threadIdx.x;
@@ -890,17 +878,11 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             while (c >= row_chunks) { c -= row_chunks; m++; }
             u2_t t[4];
             fits = split_piece_bf8(v, t) && fits;
-            const u2_t mb = piece_mean_bf8(v);
-            const int c8 = (c & ~3) | ((c & 1) << 1) | ((c >> 1) & 1);   // codes 0, 2, 1, 3 of each four
+            const uint32_t mb = piece_mean_hi_lo(v);
 #pragma unroll
-            for (int term = 0; term < 4; term++) {
-                *reinterpret_cast<u2_t *>(xt + (m * 4 + term) * xt_pitch + c * 8) = t[term];
-                x8t[(m * n_mt + term) * x8_pitch + c8] = (unsigned char)(mb[0] >> (8 * term));
-            }
-            if (M == 1) {
-#pragma unroll
-                for (int term = 0; term < 4; term++) x8t[(4 + term) * x8_pitch + c8] = (unsigned char)(mb[1] >> (8 * term));
-            }
+            for (int term = 0; term < 4; term++) *reinterpret_cast<u2_t *>(xt + (m * 4 + term) * xt_pitch + c * 8) = t[term];
+            reinterpret_cast<uint16_t *>(x8t + (2 * m) * x8_pitch)[c] = (uint16_t)mb;
+            reinterpret_cast<uint16_t *>(x8t + (2 * m + 1) * x8_pitch)[c] = (uint16_t)(mb >> 16);
             c += 64 * W;
         }
     }
@@ -917,7 +899,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     DMM_TRACE_MARK(3);
     // the vote: every wave publishes whether one of its rows or pieces failed, in a word of its own (so
     // nothing needs clearing first), and after the barrier every wave reads all of them
-    uint32_t *votes = reinterpret_cast<uint32_t *>(x8t + n_mt * M * x8_pitch);
+    uint32_t *votes = reinterpret_cast<uint32_t *>(x8t + 2 * M * x8_pitch);
     const bool wave_bad = __builtin_amdgcn_ballot_w64(!fits) != 0;
     if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
     __syncthreads();
@@ -931,18 +913,17 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     DMM_TRACE_MARK(4);
     // B operand addresses of this lane: column c16 = 4 m + term (column 0 for the idle ones)
     const int col = c16 < 4 * M ? c16 : 0;
-    const int col8 = c16 < n_mt * M ? c16 : 0;
+    const int row8 = (c16 < 4 * M && (c16 & 3) < 2) ? 2 * (c16 >> 2) + (c16 & 3) : 0;   // hi or lo of x row c16 / 4
     const uint32_t xlane = lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64);
-    const uint32_t x8lane = lds_addr(x8t) + (uint32_t)(col8 * x8_pitch + q * 8);
+    const uint32_t x8lane = lds_addr(x8t) + (uint32_t)(row8 * x8_pitch + q * 16);
 
     f4_t acc[R][2];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
-    // weights of this lane's column: 8^-t with t = c16 % 4 for x, and for the means t = c16 % 4
-    // (M > 1) or c16 % 8 (M == 1); columns that hold nothing count as zero
+    // weights of this lane's column: 8^-t with t = c16 % 4 for the terms of x, 1 for the two halves
+    // of the means; columns that hold nothing count as zero
     const float x_weight = c16 < 4 * M ? __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)(c16 & 3) * 3u << 23)) : 0.f;
-    const float mean_weight =
-        c16 < n_mt * M ? __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)(c16 & (n_mt - 1)) * 3u << 23)) : 0.f;
+    const float mean_weight = (c16 < 4 * M && (c16 & 3) < 2) ? 1.f : 0.f;
     f4_t accd[R];   // the shift term
 #pragma unroll
     for (int r = 0; r < R; r++) accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
@@ -950,23 +931,23 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     auto finish_block = [&](int blk) {
         f4_t *rp = red + (blk & 1) * red_par;
         if (M == 1) {
-            // Batch 1: the wave only leaves its 8 columns (x terms in 0..3, the later terms of the
-            // means in 4..7, where the main accumulators hold nothing of use) ...
-            const float x_mask = c16 < 4 ? 1.f : 0.f;
+            // Batch 1: the wave only leaves its 4 columns (the shift term's columns 0 and 1 ride in
+            // the same slots, column 1 times 8 to meet the weight 1/8 it gets below) ...
+            const float d_scale = c16 == 0 ? 1.f : c16 == 1 ? 8.f : 0.f;
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const f4_t v = (acc[r][0] + acc[r][1]) * x_mask + accd[r];
-                if (c16 < 8) rp[wave * (R * 32 + 1) + (r * 4 + q) * 8 + c16] = v;
+                const f4_t v = acc[r][0] + acc[r][1] + accd[r] * d_scale;
+                if (c16 < 4) rp[wave * (R * 16 + 1) + (r * 4 + q) * 4 + c16] = v;
                 acc[r][0] = acc[r][1] = accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
             }
             __syncthreads();
-            // ... and one wave per tile adds them up: lane (w, quarter) takes wave w's 8 columns with
+            // ... and one wave per tile adds them up: lane (w, quarter) takes wave w's 4 columns with
             // their weights 8^-c, then the 16 lanes of a row are added with DPP shifts
             for (int r = wave; r < R; r += W) {
-                const f4_t *src = rp + c16 * (R * 32 + 1) + (r * 4 + q) * 8;
+                const f4_t *src = rp + c16 * (R * 16 + 1) + (r * 4 + q) * 4;
                 f4_t v = src[0];
 #pragma unroll
-                for (int c = 1; c < 8; c++) v += src[c] * __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)c * 3u << 23));
+                for (int c = 1; c < 4; c++) v += src[c] * __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)c * 3u << 23));
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
                 const int tile = t0 + blk * R + r;
@@ -1027,7 +1008,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
 #ifdef DMM_TRACE
                 if (i0 + d < 7) { asm volatile("" ::"v"(cw[d][0])); DMM_TRACE_MARK(8 + 2 * (i0 + d)); }
 #endif
-                q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 32u, lane_base, acc, accd, nv);
+                q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 64u, lane_base, acc, accd, nv);
                 if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
                 if (++j >= n_sw) {
                     j = 0;

@@ -98,10 +98,10 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
  *                    (e4m3) bytes - exact when every grid value has at most 4 significant bits
  *                    in fp8's range, as the E8P grid does - and x
  *                    as four bf8 (e5m2) terms that add up to it exactly; the +-1/4 shift of a
- *                    code is added through the per-code means of x (kept to the full fp32 sum
- *                    at M = 1, rounded to half at M = 2 .. 4).  Nothing is lost in the operands;
+ *                    code is added through the per-code means of x (two halves, hi + lo, times
+ *                    +-2 in a 16-bit MFMA of their own).  Nothing is lost in the operands;
  *                    the 8-bit MFMA aligns the products of a group to the largest of them, so y
- *                    is not always the 16-bit kernel's bit for bit: at M = 1, 98 % of the outputs
+ *                    is not always the 16-bit kernel's bit for bit: 98 % of the outputs
  *                    are the correctly rounded ones and the rest are one half ulp off (99th
  *                    percentile of the error 0.57 ulps; the tolerance of the operator is 1e-2,
  *                    thousands of ulps).  A grid that does not fit fp8, or an x
@@ -109,8 +109,8 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
  *                    kernel: same call, same status.  dmm_set_gemv_8bit(0), or DMM_GEMV_8BIT=0
  *                    in the environment, keeps the operator off this kernel.  Domain: that of
  *                    dmm_gemv_f16 with M <= 4 and the terms of x and of its means fitting the
- *                    LDS beside the tables and the partial sums (4 M (K + 16) + T M (K / 8 + 16)
- *                    bytes, T = 8 at M = 1, else 4: K <= 9472 at M = 1); DMM_ERR_UNSUPPORTED
+ *                    LDS beside the tables and the partial sums (4 M (K + 16) + 2 M (K / 4 + 16)
+ *                    bytes: K <= 12544 at M = 1); DMM_ERR_UNSUPPORTED
  *                    outside.  No counterpart in the reference (its kernel multiplies int8 by
  *                    int8). */
 int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float scale,

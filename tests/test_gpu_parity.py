@@ -144,8 +144,8 @@ def _gemv_vs_oracle(x, codes, grid, scale, packed=False, path="gemv8"):
 @pytest.mark.parametrize("N,K", [(16, 256), (52, 1024), (4360, 2048), (1000, 4096), (12304, 8192)])
 @pytest.mark.parametrize("grid_kind", ["e8p", "fp8_all", "half_any", "one_off"])
 def test_gemv_8bit_operands_and_fallback(M, N, K, grid_kind):
-    red = 2 * 16 * 33 * 16 if M == 1 else 2 * 16 * 4 * M * 16
-    terms = 4 * M * (K + 16) + (8 if M == 1 else 4) * M * (K // 8 + 16) + 64
+    red = 2 * 16 * 17 * 16 if M == 1 else 2 * 16 * 4 * M * 16
+    terms = 4 * M * (K + 16) + 2 * M * (K // 4 + 16) + 64
     if 96 * 1024 + red + terms > 160 * 1024:
         pytest.skip("the terms of x do not fit the LDS beside the tables: outside the kernel's domain")
     rng = np.random.default_rng(M * 7 + N + K)
@@ -205,9 +205,9 @@ def _random_8bit_cases(n, seed):
     out = []
     while len(out) < n:
         M = int(rng.integers(1, 5))
-        K = 256 * int(rng.integers(1, 38))
-        red = 2 * 16 * 33 * 16 if M == 1 else 2 * 16 * 4 * M * 16
-        if 96 * 1024 + red + 4 * M * (K + 16) + (8 if M == 1 else 4) * M * (K // 8 + 16) + 64 > 160 * 1024:
+        K = 256 * int(rng.integers(1, 50))
+        red = 2 * 16 * 17 * 16 if M == 1 else 2 * 16 * 4 * M * 16
+        if 96 * 1024 + red + 4 * M * (K + 16) + 2 * M * (K // 4 + 16) + 64 > 160 * 1024:
             continue
         N = 4 * int(rng.integers(1, 1400)) if len(out) % 3 else 4 * int(rng.integers(1100, 2600))
         out.append((M, N, K))
