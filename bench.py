@@ -41,6 +41,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="skip prefill / small-batch / CPU legs")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
+    ap.add_argument("--graph-steps", type=int, default=12,
+                    help="steps per HIP graph replay (rounded down to whole turns of the code-buffer sets)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the M = 2048 leg and print its object (for profiling the matrix-matrix kernel)")
     ap.add_argument("--rotate-mb", type=int, default=400, help="distinct code bytes to rotate through, at least")
@@ -111,38 +113,54 @@ def main():
         for p in probs:
             call(p["x"], p["codes"][i % copies], p["grid"], p["scale"], p["y"])
 
-    # One HIP graph per code-buffer set (a step = its four launches), so that the timed loop
-    # costs the host one graph launch per step: with four ctypes calls per 56 us step the loop
-    # sits close to being bound by the host, and a busy host core then shows up in `value`.
-    run_step = step
+    # HIP graphs of several consecutive steps each (a step = its four launches, on the next set
+    # of code buffers), so that the timed loop costs the host one graph launch per
+    # `--graph-steps` steps.  A decode step of a model is one graph of hundreds of launches (80
+    # layers of these four projections at this size), not one of four: with a graph per step the
+    # GPU sat idle for about 15 us between replays, a fifth of the step, and with four ctypes
+    # calls per 56 us step the eager loop sits close to being bound by the host.
+    def run_steps(n):
+        for i in range(n):
+            step(i)
     launch_mode = "eager"
     if not args.no_graph:
         try:
             for i in range(copies):
                 step(i)                      # kernel attributes are set outside the capture
             torch.cuda.synchronize()
-            graphs = []
-            for c in range(copies):
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    cap = torch.cuda.current_stream().cuda_stream
-                    for p in probs:
-                        st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][c].data_ptr(), p["grid"].data_ptr(),
-                                                       p["scale"], p["y"].data_ptr(), 1, p["N"], p["K"], cap)
-                        if st != 0:
-                            raise capi.DmmError("dmm_decode_matmul_f16", st)
-                graphs.append(g)
-            run_step = lambda i: graphs[i % copies].replay()
-            launch_mode = "hip graph, one replay per step"
+            chunk = max(copies, args.graph_steps // copies * copies)   # whole turns of the buffer sets
+            graphs = {}
+
+            def graph_of(n):                 # n consecutive steps, starting on buffer set 0
+                if n not in graphs:
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g):
+                        cap = torch.cuda.current_stream().cuda_stream
+                        for i in range(n):
+                            for p in probs:
+                                st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][i % copies].data_ptr(),
+                                                               p["grid"].data_ptr(), p["scale"], p["y"].data_ptr(),
+                                                               1, p["N"], p["K"], cap)
+                                if st != 0:
+                                    raise capi.DmmError("dmm_decode_matmul_f16", st)
+                    graphs[n] = g
+                return graphs[n]
+
+            for n in {chunk, args.steps % chunk, args.warmup % chunk} - {0}:
+                graph_of(n)
+
+            def run_steps(n):                # exactly n steps: whole chunks, then the rest
+                for _ in range(n // chunk):
+                    graphs[chunk].replay()
+                if n % chunk:
+                    graphs[n % chunk].replay()
+            launch_mode = "hip graph, %d steps (%d launches) per replay" % (chunk, chunk * len(probs))
         except Exception as e:   # capture unavailable: time the eager loop
             print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
-            run_step = step
-    for i in range(args.warmup):
-        run_step(i)
+    run_steps(args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        run_step(i)
+    run_steps(args.steps)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
