@@ -363,18 +363,38 @@ __device__ __forceinline__ h8_t stream_finish(const u4_t &g, const u4_t &sg, uin
 }
 
 // One 256-wide k step for the first nv (uniform, 1 <= nv <= R) of R row tiles.  Items (word
-// t2 of row tile r) run t2-major so that the two B operands of a word pair are read from LDS
-// once and used for all tiles; the gathers of item i+1 are issued before the math of item i.
+// t2 of row tile r) run t2-major; the gathers of item i+1 are issued before the math of item i.
 // Tiles past nv are skipped by uniform branches around their gathers and their math.
-template <int R>
+//
+// The B operand.  A lane's 8 codes of the step feed 8 MFMAs (i = 0 .. 7), and MFMA i needs the
+// 16-byte piece i of the lane quarter's 128 bytes of x in the lanes of ONE column per x row.
+// JP = 1: column m holds row m (M <= 16) and every MFMA reads its piece, 8 wave-wide LDS reads
+// per step, a third of the kernel's LDS traffic for one useful lane in 16.  JP = 4 (M <= 4):
+// column 4 m + j holds piece 4 s + j of row m in register set s, so TWO reads fetch the whole
+// step; MFMA i multiplies by set i / 4, and since its other columns hold the pieces of other
+// MFMAs, MFMA i adds into accumulator i % 4, of which only the columns 4 m + i % 4 are ever
+// looked at (finish_block adds column 4 m + j of accumulator j over j).  Lanes of columns past
+// 4 M read zeros.
+template <int JP>
+struct StreamB {
+    static constexpr int kAcc = JP == 1 ? 2 : JP;   // accumulators per row tile
+};
+
+template <int R, int JP>
 __device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t lane_base,
-                                            uint32_t quarter_bits, f4_t (&acc)[R][2], int nv)
+                                            uint32_t quarter_bits, f4_t (&acc)[R][StreamB<JP>::kAcc], int nv)
 {
     constexpr int kItems = 4 * R;
     StreamGather buf[2];
-    u4_t xb[2][2];
-    xb[0][0] = lds_read16(xaddr);
-    xb[0][1] = lds_read16(xaddr + 16);
+    constexpr int kSets = JP == 1 ? 4 : 8 / JP;
+    u4_t xb[kSets];
+    if constexpr (JP == 1) {
+        xb[0] = lds_read16(xaddr);
+        xb[1] = lds_read16(xaddr + 16);
+    } else {
+#pragma unroll
+        for (int s = 0; s < kSets; s++) xb[s] = lds_read16(xaddr + s * JP * 16);
+    }
     stream_gather(buf[0], cw[0][0], lane_base, quarter_bits);
 #pragma unroll
     for (int i = 0; i < kItems; i++) {
@@ -382,8 +402,10 @@ __device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr,
         if (i + 1 < kItems) {
             const int nt2 = (i + 1) / R, nr = (i + 1) % R;
             if (nr == 0) {
-                xb[nt2 & 1][0] = lds_read16(xaddr + nt2 * 32);
-                xb[nt2 & 1][1] = lds_read16(xaddr + nt2 * 32 + 16);
+                if constexpr (JP == 1) {
+                    xb[(nt2 & 1) * 2] = lds_read16(xaddr + nt2 * 32);
+                    xb[(nt2 & 1) * 2 + 1] = lds_read16(xaddr + nt2 * 32 + 16);
+                }
                 stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
             } else if (nr < nv) {
                 stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
@@ -393,17 +415,32 @@ __device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr,
             // 4 packed FMAs, MFMA, 4 packed FMAs, MFMA: the second group and the next item's
             // address math run in the shadow of the matrix unit
             const StreamGather &b = buf[i & 1];
+            constexpr int kA = StreamB<JP>::kAcc;
+            const int i0 = 2 * t2, i1 = 2 * t2 + 1;
+            const u4_t &b0 = JP == 1 ? xb[(t2 & 1) * 2] : xb[i0 / JP];
+            const u4_t &b1 = JP == 1 ? xb[(t2 & 1) * 2 + 1] : xb[i1 / JP];
             const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
-            acc[r][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[t2 & 1][0]), acc[r][0], 0, 0, 0);
+            acc[r][i0 % kA] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, b0), acc[r][i0 % kA], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
-            acc[r][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[t2 & 1][1]), acc[r][1], 0, 0, 0);
+            acc[r][i1 % kA] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, b1), acc[r][i1 % kA], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
 
-template <int R, int W, int D, bool kPacked>
+// v + (the value of the lane kShl places up the row of 16)
+template <int kShl>
+__device__ __forceinline__ float dpp_shl_add(float v, float w)
+{
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, w), 0x100 + kShl, 0xF, 0xF, true));
+}
+
+// bytes of the LDS copy of x: M padded rows and 128 bytes of zeros behind them (the B operand
+// of the columns that hold no x)
+__host__ __device__ constexpr int64_t stream_x_bytes(int64_t M, int64_t K) { return M * (2 * K + 16) + 128; }
+
+template <int R, int W, int D, bool kPacked, int JP>
 __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x, const uint16_t *__restrict__ codes,
                                                  const void *__restrict__ grid, float scale,
                                                  uint16_t *__restrict__ y, int M, int N, int K, int tiles_q,
@@ -499,29 +536,56 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
     for (int m = 1; m < M; m++)
         for (int c = tid; c < row_chunks; c += 64 * W)
             reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = reinterpret_cast<const u4_t *>(x + (int64_t)m * K)[c];
+    if (tid >= 64 * W - 8) reinterpret_cast<u4_t *>(xs + M * x_pitch)[tid - (64 * W - 8)] = u4_t{0u, 0u, 0u, 0u};
     DMM_TRACE_MARK(2);
     stream_stage_grid<64 * W>(smem_raw, grow, tid);
     DMM_TRACE_MARK(3);
     __syncthreads();
     DMM_TRACE_MARK(4);
 
-    // B operand address of this lane: row m = c16 (row 0 for columns past M), quarter q
-    const uint32_t xlane = lds_addr(xs) + (uint32_t)((c16 < M ? c16 : 0) * x_pitch + q * 128);
+    // B operand address of this lane.  JP = 1: row m = c16 (row 0 for columns past M), quarter
+    // q.  JP = 4: column c16 = 4 m + j reads piece j (and 4 + j) of row m's quarter; columns past
+    // 4 M read the zeros behind x, at every step (their step stride is 0).
+    constexpr int kAcc = StreamB<JP>::kAcc;
+    const bool col_live = JP == 1 || c16 / JP < M;
+    const uint32_t xlane = JP == 1    ? lds_addr(xs) + (uint32_t)((c16 < M ? c16 : 0) * x_pitch + q * 128)
+                           : col_live ? lds_addr(xs) + (uint32_t)((c16 / JP) * x_pitch + q * 128 + (c16 % JP) * 16)
+                                      : lds_addr(xs) + (uint32_t)(M * x_pitch);
+    const uint32_t xstride = col_live ? 512u : 0u;
 
-    f4_t acc[R][2];
+    f4_t acc[R][kAcc];
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int a = 0; a < kAcc; a++) acc[r][a] = f4_t{0.f, 0.f, 0.f, 0.f};
 
     // publish this wave's partial sums of a finished row block, meet the other waves, add up
     // and store
     auto finish_block = [&](int blk) {
         f4_t *rp = red + (blk & 1) * red_par;
-        if (c16 < M) {
+        if constexpr (JP == 1) {
+            if (c16 < M) {
 #pragma unroll
-            for (int r = 0; r < R; r++) rp[(wave * R + r) * 4 * M + q * M + c16] = acc[r][0] + acc[r][1];
+                for (int r = 0; r < R; r++) rp[(wave * R + r) * 4 * M + q * M + c16] = acc[r][0] + acc[r][1];
+            }
+        } else {
+            // column 4 m + j of accumulator j, added over j into the lane of column 4 m
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                f4_t v = acc[r][0];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    v[e] = dpp_shl_add<1>(v[e], acc[r][1][e]);
+                    v[e] = dpp_shl_add<2>(v[e], acc[r][2][e]);
+                    v[e] = dpp_shl_add<3>(v[e], acc[r][3][e]);
+                }
+                if (c16 % JP == 0 && c16 / JP < M) rp[(wave * R + r) * 4 * M + q * M + c16 / JP] = v;
+            }
         }
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int a = 0; a < kAcc; a++) acc[r][a] = f4_t{0.f, 0.f, 0.f, 0.f};
         __syncthreads();
         // (row tile r, x row m) pairs go round the waves; lane (w = lane % 16, quarter lane / 16)
         // fetches ONE partial sum, wave w's, and the 16 of a row of lanes are added with DPP
@@ -564,9 +628,9 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
                 } else
 #endif
                 {
-                    const uint32_t xa = xlane + (uint32_t)((wave + j * W) * 512);
+                    const uint32_t xa = xlane + __umul24((uint32_t)(wave + j * W), xstride);
                     const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
-                    stream_step<R>(cw[d], xa, lane_base, quarter_bits, acc, nv);
+                    stream_step<R, JP>(cw[d], xa, lane_base, quarter_bits, acc, nv);
                 }
                 if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
                 if (++j >= n_sw) {
@@ -584,14 +648,14 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
     DMM_TRACE_DUMP();
 }
 
-template <int R, int W, int D, bool kPacked>
+template <int R, int W, int D, bool kPacked, int JP>
 __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__restrict__ x,
                                                              const uint16_t *__restrict__ codes,
                                                              const void *__restrict__ grid, float scale,
                                                              uint16_t *__restrict__ y, int M, int N, int K,
                                                              int tiles_q, int tiles_r)
 {
-    gemv_stream_body<R, W, D, kPacked>(x, codes, grid, scale, y, M, N, K, tiles_q, tiles_r);
+    gemv_stream_body<R, W, D, kPacked, JP>(x, codes, grid, scale, y, M, N, K, tiles_q, tiles_r);
 }
 
 // ------------------------------------------------------------------ streaming matrix-vector path, 8-bit operands
@@ -906,7 +970,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     if (__builtin_amdgcn_ballot_w64(votes[lane & (W - 1)] != 0) != 0) {
         // a grid value does not fit 8 bits, or x is not finite: the 16-bit kernel takes over (it
         // builds its own tables)
-        gemv_stream_body<R, W, 2, kPacked>(x, codes, grid, scale, y, M, N, K, tiles_q, tiles_r);
+        gemv_stream_body<R, W, 2, kPacked, 4>(x, codes, grid, scale, y, M, N, K, tiles_q, tiles_r);
         return;
     }
 
@@ -1937,13 +2001,20 @@ int launch_gemv_stream(const void *x, const void *codes, const void *grid, float
 #ifdef DMM_TRACE
     const size_t shmem = 160 * 1024;
 #else
-    const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)M * (2 * K + 16);
+    const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)stream_x_bytes(M, K);
 #endif
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemv_stream_kernel<R, W, D, kPacked>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_stream_kernel<R, W, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+    if (M <= 4) {   // four pieces of x per LDS read
+        static bool attr_done[kMaxDevices] = {};
+        if (int e = allow_dynamic_lds(gemv_stream_kernel<R, W, D, kPacked, 4>, 160 * 1024, attr_done)) return e;
+        return launch(gemv_stream_kernel<R, W, D, kPacked, 4>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                      (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N,
+                      (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    }
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(gemv_stream_kernel<R, W, D, kPacked, 1>, 160 * 1024, attr_done)) return e;
+    return launch(gemv_stream_kernel<R, W, D, kPacked, 1>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
@@ -1979,7 +2050,7 @@ int launch_gemv_q8(const void *x, const void *codes, const void *grid, float sca
 template <int R, int W>
 bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
 {
-    return M <= 16 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + M * (2 * K + 16) <= 160 * 1024 &&
+    return M <= 16 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + stream_x_bytes(M, K) <= 160 * 1024 &&
            N * (K >> 2) < (1LL << 31);
 }
 
@@ -2072,8 +2143,6 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
         if (gemv_q8_ok<R, 16>(M, N, K))                                                            \
             return launch_gemv_q8<R, 16, D>(x, codes, grid, scale, y, M, N, K, stream);            \
         break;
-        DMM_Q8_CASE(8, 2, 2)
-        DMM_Q8_CASE(8, 2, 3)
         DMM_Q8_CASE(9, 1, 2)
         DMM_Q8_CASE(9, 1, 3)
         DMM_Q8_CASE(9, 1, 4)
