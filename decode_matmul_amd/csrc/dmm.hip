@@ -813,17 +813,30 @@ __device__ __forceinline__ long q8_pack(uint32_t lo, uint32_t hi)
 // One 256-wide k step for the first nv (uniform, 1 <= nv <= R) of R row tiles; same item order
 // as stream_step.  xaddr: this lane's x terms of the step (16 bytes per word pair: the B
 // operands of its two codes), x8addr: the means of its 8 codes (8 halves: hi or lo, by column).
-template <int R>
+//
+// kOne (M = 1): the B operands of a step in two LDS reads instead of five.  A wave-wide read
+// costs the LDS the same whether one lane in 16 wants the bytes or all do, and at M = 1 only
+// the four term columns do.  So columns 0 .. 3 read the pieces of the first MFMA (32 bytes per
+// lane: two reads), columns 4 .. 7 those of the second in the same two reads, and columns 8 and 9
+// the means (hi, lo) in the first of them: every MFMA of the step takes the same registers, the
+// first looks at its columns 0 .. 3 only, the second at 4 .. 7, the shift term at 8 and 9 (what
+// the other columns make of bytes that are not theirs is never read).  xaddr is then the
+// lane's own address by column; x8addr is unused.
+template <int R, bool kOne>
 __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t x8addr, uint32_t lane_base,
                                         f4_t (&acc)[R][2], f4_t (&accd)[R], int nv)
 {
-    // All 16 table gathers of a tile's step and the 5 reads of x go out before the first MFMA
+    // All 16 table gathers of a tile's step and the reads of x go out before the first MFMA
     // (8-byte results: 48 registers), so the wave meets the LDS latency once per step and tile,
     // not once per word; with two tiles the reads of x serve both.
     u4_t xq[4];
-#pragma unroll
-    for (int t2 = 0; t2 < 4; t2++) xq[t2] = lds_read16(xaddr + t2 * 16);
-    const u4_t x8 = lds_read16(x8addr);
+    xq[0] = lds_read16(xaddr);
+    xq[1] = lds_read16(xaddr + 16);
+    if constexpr (!kOne) {
+        xq[2] = lds_read16(xaddr + 32);
+        xq[3] = lds_read16(xaddr + 48);
+    }
+    const u4_t x8 = kOne ? xq[0] : lds_read16(x8addr);
 #pragma unroll
     for (int r = 0; r < R; r++) {
         if (r > 0 && r >= nv) break;   // tiles past nv: nothing to do (uniform)
@@ -839,7 +852,7 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
             const i8_t a = i8_t{(int)(b0.g0[0] ^ b0.s0[0]), (int)(b0.g0[1] ^ b0.s0[1]), (int)(b0.g1[0] ^ b0.s1[0]),
                                 (int)(b0.g1[1] ^ b0.s1[1]), (int)(b1.g0[0] ^ b1.s0[0]), (int)(b1.g0[1] ^ b1.s0[1]),
                                 (int)(b1.g1[0] ^ b1.s1[0]), (int)(b1.g1[1] ^ b1.s1[1])};
-            const u4_t &x0 = xq[2 * h], &x1 = xq[2 * h + 1];
+            const u4_t &x0 = xq[kOne ? 0 : 2 * h], &x1 = xq[kOne ? 1 : 2 * h + 1];
             const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
             acc[r][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[r][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
         }
@@ -850,7 +863,7 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
     }
 }
 
-template <int R, int W, int D, bool kPacked>
+template <int R, int W, int D, bool kPacked, bool kOne>
 __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restrict__ x,
                                                          const uint16_t *__restrict__ codes,
                                                          const void *__restrict__ grid, float scale,
@@ -976,9 +989,16 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
 
     DMM_TRACE_MARK(4);
     // B operand addresses of this lane: column c16 = 4 m + term (column 0 for the idle ones)
+    // (kOne: columns 0 .. 7 = term c16 % 4 of the first or the second MFMA's 32 bytes, columns 8 and
+    // 9 = the means hi and lo, whose rows advance 64 bytes per step where a term row advances 256;
+    // the other columns repeat 2 .. 7)
     const int col = c16 < 4 * M ? c16 : 0;
     const int row8 = (c16 < 4 * M && (c16 & 3) < 2) ? 2 * (c16 >> 2) + (c16 & 3) : 0;   // hi or lo of x row c16 / 4
-    const uint32_t xlane = lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64);
+    const bool mean_col = kOne && (c16 == 8 || c16 == 9);
+    const uint32_t xlane = !kOne      ? lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64)
+                           : mean_col ? lds_addr(x8t) + (uint32_t)((c16 - 8) * x8_pitch + q * 16)
+                                      : lds_addr(xt) + (uint32_t)((c16 & 3) * xt_pitch + q * 64 + ((c16 >> 2) & 1) * 32);
+    const uint32_t xstride = mean_col ? 64u : 256u;
     const uint32_t x8lane = lds_addr(x8t) + (uint32_t)(row8 * x8_pitch + q * 16);
 
     f4_t acc[R][2];
@@ -994,13 +1014,17 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
 
     auto finish_block = [&](int blk) {
         f4_t *rp = red + (blk & 1) * red_par;
-        if (M == 1) {
-            // Batch 1: the wave only leaves its 4 columns (the shift term's columns 0 and 1 ride in
-            // the same slots, column 1 times 8 to meet the weight 1/8 it gets below) ...
+        if constexpr (kOne) {
+            // Batch 1: the wave only leaves 4 columns: term t of the first MFMAs (column t) plus
+            // term t of the second (column 4 + t); the shift term's columns 8 and 9 ride in slots
+            // 0 and 1, the second times 8 to meet the weight 1/8 it gets below ...
             const float d_scale = c16 == 0 ? 1.f : c16 == 1 ? 8.f : 0.f;
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const f4_t v = acc[r][0] + acc[r][1] + accd[r] * d_scale;
+                f4_t v;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    v[e] = dpp_shl_add<4>(acc[r][0][e], acc[r][1][e]) + dpp_shl_add<8>(0.f, accd[r][e]) * d_scale;
                 if (c16 < 4) rp[wave * (R * 16 + 1) + (r * 4 + q) * 4 + c16] = v;
                 acc[r][0] = acc[r][1] = accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
             }
@@ -1025,6 +1049,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             }
             return;
         }
+        (void)xstride;
 #pragma unroll
         for (int r = 0; r < R; r++) {
             // the four term columns of an x row are added first, each with the weight of its term:
@@ -1072,7 +1097,8 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
 #ifdef DMM_TRACE
                 if (i0 + d < 7) { asm volatile("" ::"v"(cw[d][0])); DMM_TRACE_MARK(8 + 2 * (i0 + d)); }
 #endif
-                q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 64u, lane_base, acc, accd, nv);
+                q8_step<R, kOne>(cw[d], kOne ? xlane + __umul24(step, xstride) : xlane + step * 256u, x8lane + step * 64u,
+                                 lane_base, acc, accd, nv);
                 if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
                 if (++j >= n_sw) {
                     j = 0;
@@ -2038,11 +2064,18 @@ int launch_gemv_q8(const void *x, const void *codes, const void *grid, float sca
 #else
     const size_t shmem = (size_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
 #endif
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemv_q8_kernel<R, W, D, kPacked>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_q8_kernel<R, W, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+    if (M == 1) {   // the B operands of a step in two LDS reads
+        static bool attr_done[kMaxDevices] = {};
+        if (int e = allow_dynamic_lds(gemv_q8_kernel<R, W, D, kPacked, true>, 160 * 1024, attr_done)) return e;
+        return launch(gemv_q8_kernel<R, W, D, kPacked, true>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                      (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N,
+                      (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    }
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(gemv_q8_kernel<R, W, D, kPacked, false>, 160 * 1024, attr_done)) return e;
+    return launch(gemv_q8_kernel<R, W, D, kPacked, false>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
