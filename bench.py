@@ -28,10 +28,10 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 # HBM bytes one GEMV launch moves, per kernel, averaged over the shapes of the step that kernel
 # serves: rocprofv3 FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter
 # reads for a plain 256 MiB device copy (x2.000 and x1.000).
-# gemv_stream_kernel (three of the step's launches): 15,892.7 KiB fetched, 19.7 KiB written per
-# dispatch (32,156,331 code bytes); gemv_q8_kernel (8192 -> 28672): 28,854.0 KiB and 56.7 KiB
+# gemv_stream_kernel (three of the step's launches): 15,891.7 KiB fetched, 19.8 KiB written per
+# dispatch (32,156,331 code bytes); gemv_q8_kernel (8192 -> 28672): 28,829.0 KiB and 56.7 KiB
 # (58,720,256 code bytes).
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_stream_kernel": 32565000, "dmm::gemv_q8_kernel": 59145000}
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_stream_kernel": 32565000, "dmm::gemv_q8_kernel": 59095000}
 
 
 def parse():
