@@ -1159,7 +1159,7 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
                                                            uint16_t *__restrict__ y, int M, int N, int K,
                                                            int tiles_q, int tiles_r)
 {
-    static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
+    static_assert(R >= 1 && R <= 4, "row tiles per block");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
     if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     typedef f4_t red_t[W][R * MT][kWave];
@@ -2144,6 +2144,28 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
     return kGemvRegx;
 }
 
+// The register-x kernel for M <= 16 reads the x slice of a k step once per row block, so the row
+// block should be the workgroup's whole share of tiles when that is 1 .. 4 tiles, and otherwise
+// the size that needs the fewest blocks (measured at M = 8 / 16, kernel us, two tiles per block
+// -> this choice: 4096 -> 11008 9.1 / 12.0 -> 8.4 / 10.0 (three); 8192 -> 28672 31.6 / 42.7 ->
+// 26.5 / 33.1 (four, then three); 11008 -> 4096 10.9 / 15.2 -> 10.6 / 14.8 (one)).
+template <bool kPacked>
+int run_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                  int64_t N, int64_t K, hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
+    int best = 1;
+    for (int r = 2; r <= 4; r++)
+        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
+    switch (best) {
+        case 1: return launch_gemv_regx<1, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case 2: return launch_gemv_regx<2, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case 3: return launch_gemv_regx<3, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return launch_gemv_regx<4, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    }
+}
+
 template <bool kPacked>
 int run_gemv_auto(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                   int64_t N, int64_t K, hipStream_t stream)
@@ -2151,7 +2173,7 @@ int run_gemv_auto(const void *x, const void *codes, const void *grid, float scal
     switch (pick_gemv(M, N, K)) {
         case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        default: return launch_gemv_regx<2, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return run_gemv_regx<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
     }
 }
 
@@ -2182,6 +2204,9 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
 #undef DMM_Q8_CASE
         case 20803: return launch_gemv_regx<2, 8, 1, 3>(x, codes, grid, scale, y, M, N, K, stream);
         case 20802: return launch_gemv_regx<2, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
+        case 10802: return launch_gemv_regx<1, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
+        case 40802: return launch_gemv_regx<4, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
+        case 30802: return launch_gemv_regx<3, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
         default: break;
     }
 #undef DMM_STREAM_CASE

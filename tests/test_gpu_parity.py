@@ -418,6 +418,33 @@ def test_full_size_against_decode_then_fp32_matmul(M, N, K):
     assert torch.allclose(y2.float(), 2 * y.float(), rtol=2e-3, atol=1e-3)
 
 
+# ----------------------------------------------------------------- small-batch kernel, row blocks
+@pytest.mark.parametrize("M,K", [(8, 4096), (16, 4096), (3, 28672), (12, 1024 * 5)])
+@pytest.mark.parametrize("share", [1, 2, 3, 4, 5, 7, 8])
+def test_small_batch_row_block_sizes(M, K, share):
+    """The register-x kernel takes one to four row tiles per block, chosen from the most tiles
+    a workgroup gets (`share`): every choice, with workgroups whose last block is partial and
+    an N that is no multiple of 16.  Reference: the library's own decode (pinned bit for bit
+    against the oracle above) times x in fp32 on the GPU, plus the oracle itself on the first
+    and last rows."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    N = 16 * (cus * share - 37) - 4
+    assert capi.lib().dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_regx_kernel"
+    x, _, grid, scale = workload.make_inputs(M, 8, K, seed=share)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(1000 * M + share)
+    codes = torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=DEV)
+    xd, gd = dev(x), dev(grid)
+    y = c_matmul(xd, codes, gd, scale, "gemv")
+    W = c_decode(codes, gd)
+    torch.cuda.synchronize()
+    ref = (xd.float() @ W.float().T) * scale
+    assert_close_to_oracle(y, ref.cpu().numpy(), "regx M=%d N=%d K=%d" % (M, N, K))
+    rows = torch.from_numpy(np.r_[0:24, N - 24:N]).to(DEV)
+    want = orc.matmul_f32(x.numpy(), orc.decode_f16(codes[rows].cpu().numpy(), grid.numpy()), scale)
+    assert_close_to_oracle(y[:, rows], want, "regx M=%d N=%d K=%d, oracle rows" % (M, N, K))
+
+
 # ----------------------------------------------------------------- seeded random shapes
 def _random_shapes(n, seed):
     rng = np.random.default_rng(seed)
