@@ -2166,6 +2166,17 @@ int run_gemv_regx(const void *x, const void *codes, const void *grid, float scal
     }
 }
 
+// M = 17 .. 32: two x tiles per wave leave registers for one or two row tiles (three spill)
+template <bool kPacked>
+int run_gemv_regx2(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                   int64_t N, int64_t K, hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;
+    if (share == 1) return launch_gemv_regx<1, 8, 2, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    return launch_gemv_regx<2, 8, 2, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+}
+
 template <bool kPacked>
 int run_gemv_auto(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                   int64_t N, int64_t K, hipStream_t stream)
@@ -2180,7 +2191,7 @@ int run_gemv_auto(const void *x, const void *codes, const void *grid, float scal
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
-    if (M > 16) return launch_gemv_regx<2, 8, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);
+    if (M > 16) return run_gemv_regx2<false>(x, codes, grid, scale, y, M, N, K, stream);
 #define DMM_STREAM_CASE(R, W, D)                                                                   \
     case R * 10000 + W * 100 + D:                                                                  \
         if (gemv_stream_ok<R, W>(M, N, K))                                                         \
@@ -2483,7 +2494,7 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
     // of kernel as for row-major codes
     if (!gemv_ok(x, packed, grid, y, M, N, K) || dmm_packed_bytes(N, K) >= (1LL << 31)) return DMM_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
-    if (M > 16) return launch_gemv_regx<2, 8, 2, 2, true>(x, packed, grid, scale, y, M, N, K, s);
+    if (M > 16) return run_gemv_regx2<true>(x, packed, grid, scale, y, M, N, K, s);
     return run_gemv_auto<true>(x, packed, grid, scale, y, M, N, K, s);
 }
 
