@@ -2130,9 +2130,9 @@ int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale,
 }
 
 // The choice among the matrix-vector kernels.  Launches of more than three row tiles per
-// workgroup: the 8-bit kernel where it applies (14 % faster at seven tiles, 2 % at two and a
-// half - below that its dearer prologue is not won back, and the 16-bit kernel's y is the
-// correctly rounded one).  Otherwise the 16-bit streaming kernel, one tile at a time (two at a
+// workgroup: the 8-bit kernel where it applies (13 % faster at seven tiles, 3 - 4 % at two to
+// three, slower at one - its prologue is the dearer one, a grid that does not fit fp8 costs it
+// a second table build, and the 16-bit kernel's y is the correctly rounded one).  Otherwise the 16-bit streaming kernel, one tile at a time (two at a
 // time is 6 - 10 % slower at K = 8192); the register-x kernel when x does not fit the LDS.
 enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
 
