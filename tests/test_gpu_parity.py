@@ -693,7 +693,9 @@ def test_graph_capture_and_replay():
     step can be captured in a HIP graph.  Every replay is checked against the eager result,
     with eager work and synchronisations between the replays, after x has been changed in
     place (a replay must read the current contents of its buffers)."""
-    shapes = [(1, 1024, 4096), (1, 4096, 1024), (8, 512, 2048), (160, 384, 512)]
+    shapes = [(1, 1024, 4096), (1, 4096, 1024), (8, 512, 2048), (160, 384, 512),
+              (1, 16384, 512), (3, 16400, 768),      # the 8-bit kernel, batch 1 and batch 3
+              (12, 4800, 5120)]                      # the register-x kernel
     probs = []
     for i, (M, N, K) in enumerate(shapes):
         x, codes, grid, scale = workload.make_inputs(M, N, K, seed=40 + i)
