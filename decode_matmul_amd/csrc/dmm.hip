@@ -1835,7 +1835,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 // (/root/reference/test_decode_matmul.py:101-109: 16-row x 4-column tiles of 64 codes ordered
 // [row % 8][column % 4][row / 8]) or plain row-major.  One wave per output row, integer
 // arithmetic throughout, so the result is exact for any K (the sum wraps in int32 like the
-// reference's accumulator).  A correctness path, not a tuned one.
+// reference's accumulator).  A correctness path, not a tuned one (no matrix unit).
 __device__ __forceinline__ int64_t tiled_code_index(int64_t n, int64_t j, int64_t kc)
 {
     return ((n >> 4) * (kc >> 2) + (j >> 2)) * 64 + (n & 7) * 8 + (j & 3) * 2 + ((n >> 3) & 1);
@@ -1848,42 +1848,75 @@ __device__ __forceinline__ int wave_sum_i32(int v)
     return v;
 }
 
-__global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
-                                                   const int64_t *__restrict__ codebook_abs,
-                                                   int32_t *__restrict__ out, int64_t M, int64_t N, int64_t K,
-                                                   int tiled)
+// Weights of one code, exactly as the reference's scalar decode: +-byte, then +1 or -1, kept in int8.
+__device__ __forceinline__ void int8_decode_exact(uint64_t abs, uint32_t c, int (&w)[8])
 {
-    __shared__ uint64_t table[256];
-    table[threadIdx.x] = (uint64_t)codebook_abs[threadIdx.x];
-    __syncthreads();
+    uint32_t s8 = (c >> 8) & 0x7Fu;
+    s8 |= (__builtin_popcount(s8) & 1u) << 7;
+    const int shift = (c >> 15) & 1;
+#pragma unroll
+    for (int d = 0; d < 8; d++) {
+        int8_t v = (int8_t)(abs & 0xFFu);
+        if ((s8 >> d) & 1u) v = (int8_t)(-v);
+        v = (int8_t)(shift ? v - 1 : v + 1);
+        w[d] = v;
+        abs >>= 8;
+    }
+}
+
+// kFast: every byte of the table is 2 mod 4 (the E8P table is: 4 x a half-odd value).  Then
+// negating a byte flips its upper six bits, adding 1 sets its lowest bit and subtracting 1
+// turns the low bits 10 into 01 - the whole decode is one exclusive or with a mask that depends
+// only on the code's high byte (/root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:45-65
+// uses the same property), and the 8 products of a code are two 4-way int8 dot products.
+// Otherwise (kFast false) the scalar decode above, byte by byte.  x8: x and K allow 8-byte loads.
+// Rows n_first, n_first + n_stride, ... below n_end, one wave each.
+template <bool kFast>
+__device__ __forceinline__ void int8_rows(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+                                          const uint64_t *table, const uint64_t *masks, int32_t *__restrict__ out,
+                                          int64_t M, int64_t N, int64_t K, int tiled, bool x8, int64_t n_first,
+                                          int64_t n_stride, int64_t n_end)
+{
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
     const int64_t kc = K >> 3;
-    constexpr int kMC = 4;
-    for (int64_t n = (int64_t)blockIdx.x * 4 + wave; n < N; n += (int64_t)gridDim.x * 4) {
+    constexpr int kMC = 8;
+    for (int64_t n = n_first; n < n_end; n += n_stride) {
         for (int64_t m0 = 0; m0 < M; m0 += kMC) {
             int acc[kMC] = {};
             for (int64_t j = lane; j < kc; j += kWave) {
                 const uint32_t c = codes[tiled ? tiled_code_index(n, j, kc) : n * kc + j];
-                uint64_t abs = table[c & 0xFFu];
-                uint32_t s8 = (c >> 8) & 0x7Fu;
-                s8 |= (__builtin_popcount(s8) & 1u) << 7;
-                const int shift = (c >> 15) & 1;
-                int w[8];
+                if (kFast) {
+                    const uint64_t w8 = table[c & 0xFFu] ^ masks[c >> 8];
+                    const int wlo = (int)(uint32_t)w8, whi = (int)(uint32_t)(w8 >> 32);
 #pragma unroll
-                for (int d = 0; d < 8; d++) {
-                    int8_t v = (int8_t)(abs & 0xFFu);
-                    if ((s8 >> d) & 1u) v = (int8_t)(-v);
-                    v = (int8_t)(shift ? v - 1 : v + 1);
-                    w[d] = v;
-                    abs >>= 8;
-                }
+                    for (int mm = 0; mm < kMC; mm++) {
+                        if (m0 + mm < M) {
+                            const int8_t *xr = x + (m0 + mm) * K + j * 8;
+                            int xlo, xhi;
+                            if (x8) {
+                                const u2_t v = *reinterpret_cast<const u2_t *>(xr);
+                                xlo = (int)v[0];
+                                xhi = (int)v[1];
+                            } else {
+                                xlo = (int)((uint32_t)(uint8_t)xr[0] | (uint32_t)(uint8_t)xr[1] << 8 |
+                                            (uint32_t)(uint8_t)xr[2] << 16 | (uint32_t)(uint8_t)xr[3] << 24);
+                                xhi = (int)((uint32_t)(uint8_t)xr[4] | (uint32_t)(uint8_t)xr[5] << 8 |
+                                            (uint32_t)(uint8_t)xr[6] << 16 | (uint32_t)(uint8_t)xr[7] << 24);
+                            }
+                            acc[mm] = __builtin_amdgcn_sdot4(xlo, wlo, acc[mm], false);
+                            acc[mm] = __builtin_amdgcn_sdot4(xhi, whi, acc[mm], false);
+                        }
+                    }
+                } else {
+                    int w[8];
+                    int8_decode_exact(table[c & 0xFFu], c, w);
 #pragma unroll
-                for (int mm = 0; mm < kMC; mm++) {
-                    if (m0 + mm < M) {
-                        const int8_t *xr = x + (m0 + mm) * K + j * 8;
+                    for (int mm = 0; mm < kMC; mm++) {
+                        if (m0 + mm < M) {
+                            const int8_t *xr = x + (m0 + mm) * K + j * 8;
 #pragma unroll
-                        for (int d = 0; d < 8; d++) acc[mm] += (int)xr[d] * w[d];
+                            for (int d = 0; d < 8; d++) acc[mm] += (int)xr[d] * w[d];
+                        }
                     }
                 }
             }
@@ -1895,6 +1928,239 @@ __global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x,
         }
     }
 }
+
+__global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+                                                   const int64_t *__restrict__ codebook_abs,
+                                                   int32_t *__restrict__ out, int64_t M, int64_t N, int64_t K,
+                                                   int tiled, int x8)
+{
+    __shared__ uint64_t table[256];
+    __shared__ uint64_t masks[256];
+    __shared__ int slow[4];
+    const uint64_t abs = (uint64_t)codebook_abs[threadIdx.x];
+    table[threadIdx.x] = abs;
+    {
+        // mask of high byte t: sign bits t & 0x7F (the eighth by parity), shift t >> 7
+        uint32_t s8 = threadIdx.x & 0x7Fu;
+        s8 |= (__builtin_popcount(s8) & 1u) << 7;
+        uint64_t mk = (threadIdx.x >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
+#pragma unroll
+        for (int d = 0; d < 8; d++)
+            if ((s8 >> d) & 1u) mk ^= 0xFCull << (8 * d);
+        masks[threadIdx.x] = mk;
+    }
+    const bool bad = (abs & 0x0303030303030303ull) != 0x0202020202020202ull;
+    const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
+    if ((threadIdx.x & 63) == 0) slow[threadIdx.x >> 6] = wave_bad ? 1 : 0;
+    __syncthreads();
+    const int64_t n_first = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), n_stride = (int64_t)gridDim.x * 4;
+    if (slow[0] | slow[1] | slow[2] | slow[3])
+        int8_rows<false>(x, codes, table, masks, out, M, N, K, tiled, false, n_first, n_stride, N);
+    else
+        int8_rows<true>(x, codes, table, masks, out, M, N, K, tiled, x8 != 0, n_first, n_stride, N);
+}
+
+// ------------------------------------------------------------------ the integer operator on the matrix unit
+// M <= 16, K a multiple of 256, a table whose bytes are all 2 mod 4 (see int8_rows): the
+// small-batch kernel's structure (persistent workgroups over contiguous ranges of 16-row tiles,
+// k steps of 256 dealt to 8 waves, x fetched from L2 into registers with the codes as one
+// prefetch unit, partial sums through LDS) with the decode done in bytes - one 8-byte gather of
+// the table entry by the code's low byte, one of the mask by its high byte, exclusive or - and
+// v_mfma_i32_16x16x64_i8: a lane's 8 codes of a step are the A operands of four MFMAs (two codes =
+// 16 k each), B is 16 bytes of x per lane and MFMA.  Both tables hold 32 copies of every 8-byte
+// row (row pitch 256 B, lane reads copy lane % 32: no bank conflicts for any codes).  Exact:
+// int8 products, int32 sums (which wrap like the reference's accumulator).
+// Codes row-major, or in the reference's tile order (/root/reference/test_decode_matmul.py:101-109):
+// there 16 bytes hold codes (row g, columns c .. c + 3) interleaved with row g + 8's, so lanes g
+// and g + 8 load the same two pieces and each keeps its halves (one v_perm per two codes).
+// A table with any other byte is found while the tables are built, and the workgroup then does
+// its rows with the scalar decode instead.
+typedef int i4_t __attribute__((ext_vector_type(4)));
+constexpr int kI8TableBytes = 256 * 256;   // one table: 256 rows x 32 copies x 8 bytes
+
+template <int R, int W, int D, bool kTiled>
+__global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+                                                       const int64_t *__restrict__ codebook_abs,
+                                                       int32_t *__restrict__ out, int M, int N, int K, int tiles_q,
+                                                       int tiles_r)
+{
+    static_assert(W == 8, "the table staging below assumes 512 threads");
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
+    typedef i4_t red_t[W][R][kWave];
+    red_t *red = reinterpret_cast<red_t *>(smem_raw + 2 * kI8TableBytes);   // red[parity]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c16 = lane & 15;
+    const int q = lane >> 4;
+    const int n_steps = K >> 8;
+    const int row_bytes = K >> 2;
+    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;          // grid rows: [0, 64K)
+    const uint32_t lane_base2 = lane_base | 0x10000u;               // mask rows: [64K, 128K)
+
+    uint64_t entry = 0;
+    if (tid < 256) entry = (uint64_t)codebook_abs[tid];
+
+    const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;
+    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
+    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
+    const int nb_wg = (t1 - t0 + R - 1) / R;
+
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kTiled ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(x), 0, M * K, 0x00020000);
+    constexpr int kOut = (int)0x80000000;
+    // per-lane byte offsets inside a row block.  Row-major: row 16 r + c16, 16 bytes at quarter q.
+    // Tiled: the tile row of the block is 16 rows x K / 4 bytes as well, a tile (4 code columns) is
+    // 128 bytes, and lane (g = c16 % 8, quarter q) reads 16 bytes at g * 16 of tiles 2 q and 2 q + 1
+    // of the step's 8.
+    int voff[R];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        voff[r] = kTiled ? r * 16 * row_bytes + q * 256 + (c16 & 7) * 16 : (16 * r + c16) * row_bytes + q * 16;
+    const int xoff = c16 < M ? c16 * K + 64 * q : kOut;   // columns past M: zeros, no memory access
+    const uint32_t half_sel = (c16 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
+
+    struct Unit {
+        u4_t cw[R][kTiled ? 2 : 1];
+        u4_t xb[4];
+    };
+    int pf_blk = 0, pf_j = 0;
+    auto issue = [&](Unit &u) {
+        const bool ok = pf_blk < nb_wg && n_sw > 0;
+        const int step = wave + pf_j * W;
+        const int xs_off = ok ? step * 256 : kOut;
+        const int tb = t0 + pf_blk * R;
+        const int soff = !ok ? kOut : kTiled ? tb * 16 * row_bytes + step * 1024 : tb * 16 * row_bytes + step * 64;
+#pragma unroll
+        for (int t = 0; t < 4; t++) u.xb[t] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff + t * 16, xs_off, 0);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int so = (r == 0 || tb + r < t1) ? soff : kOut;
+            u.cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], so, 0);
+            if (kTiled) u.cw[r][kTiled ? 1 : 0] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r] + 128, so, 0);
+        }
+        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
+    };
+
+    Unit ring[D];
+#pragma unroll
+    for (int d = 0; d < D; d++) issue(ring[d]);
+
+    // tables: threads 0 .. 255 write the 32 copies of table entry tid (16 slots of two copies),
+    // threads 256 .. 511 those of the mask of high byte tid - 256
+    bool bad = false;
+    {
+        uint64_t v = entry;
+        if (tid < 256) {
+            bad = (entry & 0x0303030303030303ull) != 0x0202020202020202ull;
+        } else {
+            const uint32_t t = (uint32_t)tid - 256u;
+            uint32_t s8 = t & 0x7Fu;
+            s8 |= (__builtin_popcount(s8) & 1u) << 7;
+            v = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
+#pragma unroll
+            for (int d = 0; d < 8; d++)
+                if ((s8 >> d) & 1u) v ^= 0xFCull << (8 * d);
+        }
+        const uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+        u4_t *rowp = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;   // tid >= 256 lands in the mask table
+#pragma unroll
+        for (int i = 0; i < 16; i++) rowp[(i + tid) & 15] = u4_t{lo, hi, lo, hi};   // 16 lanes, 16 bank groups
+    }
+    // the vote on the table: one word per wave in the partial-sum area, read by everybody after the barrier
+    uint32_t *votes = reinterpret_cast<uint32_t *>(smem_raw + 2 * kI8TableBytes);
+    const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
+    if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
+    __syncthreads();
+    const bool any_bad = __builtin_amdgcn_ballot_w64(votes[lane & (W - 1)] != 0) != 0;
+    __syncthreads();   // the votes are read before partial sums overwrite them
+    if (any_bad) {
+        // scalar decode for this workgroup's rows; the raw table goes where the partial sums would
+        uint64_t *table = reinterpret_cast<uint64_t *>(smem_raw + 2 * kI8TableBytes);
+        if (tid < 256) table[tid] = entry;
+        __syncthreads();
+        const int64_t n_end = (int64_t)t1 * 16 < N ? (int64_t)t1 * 16 : N;
+        int8_rows<false>(x, codes, table, table, out, M, N, K, kTiled ? 1 : 0, false, (int64_t)t0 * 16 + wave, W, n_end);
+        return;
+    }
+
+    i4_t acc[R][2];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = i4_t{0, 0, 0, 0};
+
+    auto finish_block = [&](int blk) {
+        const int par = blk & 1;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            red[par][wave][r][lane] = acc[r][0] + acc[r][1];
+            acc[r][0] = acc[r][1] = i4_t{0, 0, 0, 0};
+        }
+        __syncthreads();
+        for (int r = wave; r < R; r += W) {
+            i4_t sacc = red[par][0][r][lane];
+#pragma unroll
+            for (int w = 1; w < W; w++) sacc += red[par][w][r][lane];
+            const int rt = t0 + blk * R + r;
+            const int n = rt * 16 + 4 * q;
+            if (c16 < M && rt < t1 && n < N)   // N % 4 == 0, so the four rows are in range together
+                *reinterpret_cast<i4_t *>(out + (int64_t)c16 * N + n) = sacc;
+        }
+    };
+
+    if (n_sw == 0) {
+        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
+        return;
+    }
+    const int n_items = nb_wg * n_sw;
+    int blk = 0, j = 0;
+    for (int i0 = 0; i0 < n_items; i0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (i0 + d < n_items) {
+                const Unit &u = ring[d];
+                const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    if (r > 0 && r >= nv) break;
+                    u4_t cw;   // the lane's 8 codes of the step, two per word
+                    if (kTiled) {
+                        const u4_t &a = u.cw[r][0], &b = u.cw[r][kTiled ? 1 : 0];
+                        cw = u4_t{__builtin_amdgcn_perm(a[1], a[0], half_sel), __builtin_amdgcn_perm(a[3], a[2], half_sel),
+                                  __builtin_amdgcn_perm(b[1], b[0], half_sel), __builtin_amdgcn_perm(b[3], b[2], half_sel)};
+                    } else {
+                        cw = u.cw[r][0];
+                    }
+                    u2_t g[8], m[8];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const uint32_t w = cw[i];
+                        g[2 * i] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
+                        m[2 * i] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
+                        g[2 * i + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
+                        m[2 * i + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const i4_t a = i4_t{(int)(g[2 * i][0] ^ m[2 * i][0]), (int)(g[2 * i][1] ^ m[2 * i][1]),
+                                            (int)(g[2 * i + 1][0] ^ m[2 * i + 1][0]), (int)(g[2 * i + 1][1] ^ m[2 * i + 1][1])};
+                        acc[r][i & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, __builtin_bit_cast(i4_t, u.xb[i]), acc[r][i & 1], 0, 0, 0);
+                    }
+                }
+                if (++j >= n_sw) {
+                    j = 0;
+                    finish_block(blk);
+                    blk++;
+                }
+            }
+            issue(ring[d]);
+        }
+    }
+}
+
 
 __global__ void zero_i32_kernel(int32_t *y, int64_t n)
 {
@@ -2361,6 +2627,49 @@ int run_generic(const void *x, const void *codes, const void *grid, float scale,
                   (const uint16_t *)codes, grid, scale, (uint16_t *)y, M, N, K);
 }
 
+// DMM_INT8_MFMA=0 in the environment keeps the integer operator on the scalar kernel (for
+// comparisons)
+bool int8x_enabled()
+{
+    static const bool on = [] {
+        const char *e = getenv("DMM_INT8_MFMA");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+template <int R, bool kTiled, bool kFirst, bool kLast>
+int launch_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+                 hipStream_t stream)
+{
+    constexpr int W = 8, D = 2;
+    const size_t shmem = (size_t)2 * kI8TableBytes + 2 * W * R * kWave * 16;
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(int8x_kernel<R, W, D, kTiled>, 160 * 1024, attr_done)) return e;
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch<kFirst, kLast>(int8x_kernel<R, W, D, kTiled>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                                 (const int8_t *)x, (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M,
+                                 (int)N, (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+// one launch for up to 16 rows of x; first / last: position in the operator call's sequence of
+// launches, for the timing events
+template <bool kTiled>
+int run_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+              bool first, bool last, hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const bool one = n_tiles <= cus;   // a workgroup with a single tile takes it alone
+#define DMM_I8X(RR)                                                                                         \
+    (first ? (last ? launch_int8x<RR, kTiled, true, true>(x, codes, cb, out, M, N, K, stream)               \
+                   : launch_int8x<RR, kTiled, true, false>(x, codes, cb, out, M, N, K, stream))              \
+           : (last ? launch_int8x<RR, kTiled, false, true>(x, codes, cb, out, M, N, K, stream)              \
+                   : launch_int8x<RR, kTiled, false, false>(x, codes, cb, out, M, N, K, stream)))
+    return one ? DMM_I8X(1) : DMM_I8X(2);
+#undef DMM_I8X
+}
+
 }  // namespace dmm
 
 using namespace dmm;
@@ -2543,10 +2852,24 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
         const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
         return launch(zero_i32_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (int32_t *)out, n);
     }
+    // the matrix-unit kernel takes up to 16 rows of x per launch
+    if ((K & 255) == 0 && (N & 3) == 0 && N * (K >> 2) < (1LL << 31) && K <= (1 << 23) && aligned(x, 16) &&
+        aligned(codes, 16) && aligned(out, 16) && int8x_enabled()) {
+        for (int64_t m0 = 0; m0 < M; m0 += 16) {
+            const int64_t mc = M - m0 < 16 ? M - m0 : 16;
+            const int8_t *xs = (const int8_t *)x + m0 * K;
+            int32_t *os = (int32_t *)out + m0 * N;
+            const int e = tiled ? run_int8x<true>(xs, codes, codebook_abs, os, mc, N, K, m0 == 0, m0 + 16 >= M, (hipStream_t)stream)
+                                : run_int8x<false>(xs, codes, codebook_abs, os, mc, N, K, m0 == 0, m0 + 16 >= M, (hipStream_t)stream);
+            if (e) return e;
+        }
+        return DMM_OK;
+    }
     int64_t blocks = (N + 3) / 4;
     if (blocks > 65535 * 16) blocks = 65535 * 16;
     return launch(int8_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const int8_t *)x,
-                  (const uint16_t *)codes, (const int64_t *)codebook_abs, (int32_t *)out, M, N, K, tiled ? 1 : 0);
+                  (const uint16_t *)codes, (const int64_t *)codebook_abs, (int32_t *)out, M, N, K, tiled ? 1 : 0,
+                  aligned(x, 8) ? 1 : 0);
 }
 
 int64_t dmm_workspace_bytes(int64_t M, int64_t N, int64_t K)

@@ -369,6 +369,53 @@ def test_integer_operator_row_major_any_shape(M, N, K):
     assert np.array_equal(out.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("M,N,K,tiled,x_off", [(1, 37, 1000, False, 0), (8, 48, 1024, True, 0), (13, 48, 1024, True, 3),
+                                               (9, 37, 1000, False, 1), (20, 16, 4096, True, 8)])
+def test_integer_operator_table_bytes_2_mod_4(M, N, K, tiled, x_off):
+    """Any table whose bytes are all 2 mod 4 takes the one-exclusive-or decode (the E8P table is
+    such a table; so is this random one, with bytes from -126 to 126): batches above the 8 rows
+    one pass covers, x at byte offsets that rule out 8-byte loads, both code layouts."""
+    rng = np.random.default_rng(M * 131 + N)
+    by = (rng.integers(0, 256, size=(256, 8)).astype(np.uint8) & 0xFC) | 2
+    by[0] = [0x82, 0x7E, 0x02, 0xFE, 0x06, 0xFA, 0x7E, 0x82]
+    cb = by.view(np.int64).reshape(256).copy()
+    xbuf = rng.integers(-128, 128, size=M * K + 16).astype(np.int8)
+    xs = xbuf[x_off:x_off + M * K].reshape(M, K)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    want = orc.decode_matmul_i32(xs, codes, cb)
+    xd = dev(xbuf)[x_off:x_off + M * K].view(M, K)
+    cd = dev(orc.transpose_tile(codes)) if tiled else dev(codes)
+    out = c_matmul_i8(xd, cd, dev(cb), tiled)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M,N,K,tiled,table", [
+    (8, 16, 4096, True, "e8p"), (1, 4100, 256, False, "e8p"), (16, 16 * 300, 512, True, "e8p"),
+    (17, 16 * (256 * 2 + 5), 256, True, "e8p"), (40, 1000, 768, False, "mod4"), (8, 16 * 1000, 1024, True, "mod4"),
+    (5, 8192 + 16, 1024, True, "any"), (3, 52, 2048, False, "any"), (16, 4096, 4096, False, "e8p")])
+def test_integer_operator_matrix_unit(M, N, K, tiled, table):
+    """K a multiple of 256 with 16-byte aligned buffers runs on v_mfma_i32_16x16x64_i8: one or
+    several tiles per workgroup with partial last blocks, more than 16 rows of x (several
+    launches), both code layouts, N no multiple of 16 (row-major), and a table with bytes that are
+    not 2 mod 4, which every workgroup must notice and serve with the scalar decode.  Exact
+    against the oracle's restatement of /root/reference/test_decode_matmul.py:58-71."""
+    rng = np.random.default_rng(M * 977 + N + K)
+    if table == "e8p":
+        cb = orc.build_codebook_abs()
+    elif table == "mod4":
+        cb = ((rng.integers(0, 256, size=(256, 8)).astype(np.uint8) & 0xFC) | 2).view(np.int64).reshape(256).copy()
+    else:
+        cb = rng.integers(-2 ** 63, 2 ** 63, size=256, dtype=np.int64)
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    want = orc.decode_matmul_i32(x, codes, cb)
+    cd = dev(orc.transpose_tile(codes)) if tiled else dev(codes)
+    out = c_matmul_i8(dev(x), cd, dev(cb), tiled)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
 def test_integer_operator_golden_cases_and_edges():
     case = np.load(os.path.join(GOLDEN_DIR, "int8_case.npz"))
     x, codes, yi, cb = case["x"], case["codes"], case["y"], case["codebook_abs"]
