@@ -241,6 +241,7 @@ def main():
         out["gemv_packed"] = gemv_packed(torch, lib, capi, workload, probs, copies, stream, args.steps)
         out["gemv_7b_shapes"] = gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes)
         out["small_batch"] = small_batch(torch, lib, capi, workload, dev, stream, rand_codes)
+        out["integer_operator"] = integer_operator(torch, lib, capi, workload, dev, stream, rand_codes)
         out["prefill"] = prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes)
         out["cpu_baseline"] = cpu_baseline(torch, workload)
     else:
@@ -377,6 +378,37 @@ def small_batch(torch, lib, capi, workload, dev, stream, rand_codes):
             rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3), "workspace_MB": round(ws_bytes / 1e6, 1),
                          "GBps_code": round(workload.code_bytes(N, K) / t / 1e9, 1),
                          "TFLOPs": round(workload.flops(M, N, K) / t / 1e12, 2)})
+    return rows
+
+
+def integer_operator(torch, lib, capi, workload, dev, stream, rand_codes):
+    """The reference's own operator (int8 x, int16 codes in its tile order, int64 table -> int32,
+    dmm_decode_matmul_i8) at the headline shapes, M = 1 and M = 8 (the reference asks for M % 8
+    == 0).  Kernel durations by events; every launch reads the next of enough code buffers to
+    stay out of the Infinity Cache.  Random 16-bit codes are equally random in either layout."""
+    from decode_matmul_amd import codebook
+    cb = codebook.build_codebook_abs().to(dev)
+    rows = []
+    for K, N in workload.LLAMA2_70B:
+        copies = max(2, -(-320 * 1000000 // workload.code_bytes(N, K)))
+        codes = rand_codes(N, K, copies, 11)
+        for M in (1, 8):
+            g = torch.Generator(device=dev)
+            g.manual_seed(5)
+            x = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8, device=dev)
+            out = torch.empty(M, N, dtype=torch.int32, device=dev)
+
+            def fn(i):
+                st = lib.dmm_decode_matmul_i8(x.data_ptr(), codes[i % copies].data_ptr(), cb.data_ptr(), out.data_ptr(),
+                                              M, N, K, 1, stream)
+                assert st == 0, st
+            for i in range(3):
+                fn(i)
+            t = timed_kernel(torch, lib, fn, 40)
+            rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3),
+                         "GBps_code": round(workload.code_bytes(N, K) / t / 1e9, 1),
+                         "frac_hbm": round(workload.code_bytes(N, K) / t / 1e9 / HBM_PEAK_GBS, 4)})
+        del codes
     return rows
 
 

@@ -168,7 +168,11 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
  * /root/reference/test_decode_matmul.py:101-109 (needs N % 16 == 0 and K % 32 == 0, as
  * decode_matmul_cuda.cu:196-197 does); tiled == 0: plain row-major [N, K/8].  None of the
  * reference's other shape demands (M % 8, K % 2048, K >= 4096) apply.  Exact integer
- * arithmetic; `out` is fully overwritten.  A correctness path (one wave per output row). */
+ * arithmetic (int32 sums wrap); `out` is fully overwritten.  With K % 256 == 0, N % 4 == 0 and
+ * 16-byte aligned x, codes and out the call runs on the int8 matrix unit, 16 rows of x per
+ * launch (a table with a byte that is not 2 mod 4 - the E8P table has none - is noticed inside
+ * the launch and served by the scalar decode); anything else takes the scalar kernel, one wave
+ * per output row.  DMM_INT8_MFMA=0 in the environment keeps every call on the scalar kernel. */
 int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_abs, void *out,
                          int64_t M, int64_t N, int64_t K, int tiled, void *stream);
 
