@@ -2852,8 +2852,10 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
         const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
         return launch(zero_i32_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (int32_t *)out, n);
     }
-    // the matrix-unit kernel takes up to 16 rows of x per launch
-    if ((K & 255) == 0 && (N & 3) == 0 && N * (K >> 2) < (1LL << 31) && K <= (1 << 23) && aligned(x, 16) &&
+    // the matrix-unit kernel takes up to 16 rows of x per launch; K <= 2^17: its weights are odd,
+    // so |w| <= 127 and no sum of K products leaves int32 - nothing depends on what the matrix
+    // unit does on overflow
+    if ((K & 255) == 0 && (N & 3) == 0 && N * (K >> 2) < (1LL << 31) && K <= (1 << 17) && aligned(x, 16) &&
         aligned(codes, 16) && aligned(out, 16) && int8x_enabled()) {
         for (int64_t m0 = 0; m0 < M; m0 += 16) {
             const int64_t mc = M - m0 < 16 ? M - m0 : 16;
