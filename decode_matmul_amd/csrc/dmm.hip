@@ -1987,6 +1987,9 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
     static_assert(W == 8, "the table staging below assumes 512 threads");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
     if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
+    // partial sums: two buffers taken in turn while they fit beside the tables (R <= 2), else one
+    // and a second barrier per row block
+    constexpr bool kTwoBuffers = R <= 2;
     typedef i4_t red_t[W][R][kWave];
     red_t *red = reinterpret_cast<red_t *>(smem_raw + 2 * kI8TableBytes);   // red[parity]
 
@@ -2093,7 +2096,7 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
     for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = i4_t{0, 0, 0, 0};
 
     auto finish_block = [&](int blk) {
-        const int par = blk & 1;
+        const int par = kTwoBuffers ? blk & 1 : 0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
             red[par][wave][r][lane] = acc[r][0] + acc[r][1];
@@ -2109,6 +2112,7 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
             if (c16 < M && rt < t1 && n < N)   // N % 4 == 0, so the four rows are in range together
                 *reinterpret_cast<i4_t *>(out + (int64_t)c16 * N + n) = sacc;
         }
+        if (!kTwoBuffers) __syncthreads();   // the next block's sums go to the same buffer
     };
 
     if (n_sw == 0) {
@@ -2643,7 +2647,7 @@ int launch_int8x(const void *x, const void *codes, const void *cb, void *out, in
                  hipStream_t stream)
 {
     constexpr int W = 8, D = 2;
-    const size_t shmem = (size_t)2 * kI8TableBytes + 2 * W * R * kWave * 16;
+    const size_t shmem = (size_t)2 * kI8TableBytes + (R <= 2 ? 2 : 1) * W * R * kWave * 16;
     static bool attr_done[kMaxDevices] = {};
     if (int e = allow_dynamic_lds(int8x_kernel<R, W, D, kTiled>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
@@ -2659,14 +2663,19 @@ template <bool kTiled>
 int run_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
               bool first, bool last, hipStream_t stream)
 {
+    // row block = the workgroup's share of tiles when that is one to four, else the size that needs
+    // the fewest blocks (x is fetched once per row block), as for the half-precision kernel
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const bool one = n_tiles <= cus;   // a workgroup with a single tile takes it alone
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;
+    int best = 1;
+    for (int r = 2; r <= 4; r++)
+        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
 #define DMM_I8X(RR)                                                                                         \
     (first ? (last ? launch_int8x<RR, kTiled, true, true>(x, codes, cb, out, M, N, K, stream)               \
                    : launch_int8x<RR, kTiled, true, false>(x, codes, cb, out, M, N, K, stream))              \
            : (last ? launch_int8x<RR, kTiled, false, true>(x, codes, cb, out, M, N, K, stream)              \
                    : launch_int8x<RR, kTiled, false, false>(x, codes, cb, out, M, N, K, stream)))
-    return one ? DMM_I8X(1) : DMM_I8X(2);
+    return best == 1 ? DMM_I8X(1) : best == 2 ? DMM_I8X(2) : best == 3 ? DMM_I8X(3) : DMM_I8X(4);
 #undef DMM_I8X
 }
 

@@ -393,7 +393,10 @@ def test_integer_operator_table_bytes_2_mod_4(M, N, K, tiled, x_off):
 @pytest.mark.parametrize("M,N,K,tiled,table", [
     (8, 16, 4096, True, "e8p"), (1, 4100, 256, False, "e8p"), (16, 16 * 300, 512, True, "e8p"),
     (17, 16 * (256 * 2 + 5), 256, True, "e8p"), (40, 1000, 768, False, "mod4"), (8, 16 * 1000, 1024, True, "mod4"),
-    (5, 8192 + 16, 1024, True, "any"), (3, 52, 2048, False, "any"), (16, 4096, 4096, False, "e8p")])
+    (5, 8192 + 16, 1024, True, "any"), (3, 52, 2048, False, "any"), (16, 4096, 4096, False, "e8p"),
+    # workgroup shares of 3, 4, 7 and 5 tiles: row blocks of three and four tiles, partial last blocks
+    (8, 16 * (256 * 3 - 10), 256, True, "e8p"), (16, 16 * (256 * 4 - 3), 256, False, "mod4"),
+    (8, 28672, 256, True, "e8p"), (4, 16 * (256 * 5 - 1), 512, True, "any")])
 def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     """K a multiple of 256 with 16-byte aligned buffers runs on v_mfma_i32_16x16x64_i8: one or
     several tiles per workgroup with partial last blocks, more than 16 rows of x (several
