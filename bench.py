@@ -45,6 +45,8 @@ def parse():
                     help="steps per HIP graph replay (rounded down to whole turns of the code-buffer sets)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the M = 2048 leg and print its object (for profiling the matrix-matrix kernel)")
+    ap.add_argument("--integer-only", action="store_true",
+                    help="run only the integer-operator leg and print its object (for profiling that kernel)")
     ap.add_argument("--rotate-mb", type=int, default=400, help="distinct code bytes to rotate through, at least")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch 8 plain device copies of 256 MiB first (a known-size reference for scaling "
@@ -96,6 +98,10 @@ def main():
 
     if args.prefill_only:
         print(json.dumps({"prefill": prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes)}))
+        return
+
+    if args.integer_only:
+        print(json.dumps({"integer_operator": integer_operator(torch, lib, capi, workload, dev, stream, rand_codes)}))
         return
 
     # ---------------------------------------------------------------- headline: 70B GEMV
