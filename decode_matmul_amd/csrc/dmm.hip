@@ -2166,6 +2166,220 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 }
 
 
+// ------------------------------------------------------------------ the integer operator, many rows of x
+// Block tile 256 (n) x 128 (m) x 64 (k), four waves, each 64 rows of W x all 128 rows of x = 8
+// accumulators of v_mfma_i32_32x32x32_i8.  Like the half-precision gemm_reg_kernel, every wave
+// decodes its own rows straight into A operands - here that is two 8-byte gathers and two
+// exclusive ors per code (int8x_kernel's tables), four codes per lane and k tile - and only x goes
+// through the LDS (rows 80 bytes apart: the 16 lanes the LDS serves per clock, 16 consecutive
+// rows, hit 16 different bank groups).  Lane (row, half h = lane / 32) takes codes 4 h .. 4 h + 3
+// of its row's 8 in the k tile (8 consecutive bytes; in the reference's tile order, the 16 bytes
+// of the pair of rows, of which one v_perm per two codes keeps ours) and pairs them with bytes
+// 32 h .. 32 h + 31 of the x rows.  Global loads run four k tiles ahead in a ring of registers;
+// one barrier per k tile.  A table with a byte that is not 2 mod 4: the workgroup does its tile
+// with the scalar decode.
+typedef int i16_t __attribute__((ext_vector_type(16)));
+constexpr int kI8gBN = 256, kI8gBM = 128, kI8gBK = 64, kI8gLd = 80;
+constexpr int kI8gSmem = 2 * kI8TableBytes + 2 * kI8gBM * kI8gLd;
+
+template <bool kTiled>
+__global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+                                                    const int64_t *__restrict__ codebook_abs,
+                                                    int32_t *__restrict__ out, int M, int N, int K)
+{
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
+    unsigned char *xs = smem_raw + 2 * kI8TableBytes;   // two x tiles of 128 rows x 80 bytes
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, kq = lane >> 5;
+    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;   // grid rows: [0, 64K)
+    const uint32_t lane_base2 = lane_base | 0x10000u;        // mask rows: [64K, 128K)
+    const int m0 = blockIdx.x * kI8gBM;
+    const int n0 = blockIdx.y * kI8gBN;
+    const int row_bytes = K >> 2;
+    const int k_tiles = K / kI8gBK;
+    constexpr int kOut = (int)0x80000000;
+
+    // tables: thread tid writes the 32 copies of table entry tid and of the mask of high byte tid
+    const uint64_t entry = (uint64_t)codebook_abs[tid];
+    {
+        uint32_t s8 = (uint32_t)tid & 0x7Fu;
+        s8 |= (__builtin_popcount(s8) & 1u) << 7;
+        uint64_t mk = (tid >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
+#pragma unroll
+        for (int d = 0; d < 8; d++)
+            if ((s8 >> d) & 1u) mk ^= 0xFCull << (8 * d);
+        u4_t *grow = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;
+        u4_t *mrow = reinterpret_cast<u4_t *>(smem_raw + kI8TableBytes) + tid * 16;
+        const u4_t gv = u4_t{(uint32_t)entry, (uint32_t)(entry >> 32), (uint32_t)entry, (uint32_t)(entry >> 32)};
+        const u4_t mv = u4_t{(uint32_t)mk, (uint32_t)(mk >> 32), (uint32_t)mk, (uint32_t)(mk >> 32)};
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            grow[(i + tid) & 15] = gv;   // 16 lanes, 16 bank groups
+            mrow[(i + tid) & 15] = mv;
+        }
+    }
+    // the vote on the table (one word per wave in the x area, read by everybody after the barrier)
+    {
+        uint32_t *votes = reinterpret_cast<uint32_t *>(xs);
+        const bool bad = (entry & 0x0303030303030303ull) != 0x0202020202020202ull;
+        const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
+        if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
+        __syncthreads();
+        const bool any_bad = (votes[0] | votes[1] | votes[2] | votes[3]) != 0;
+        __syncthreads();   // the votes are read before x overwrites them
+        if (any_bad) {
+            uint64_t *table = reinterpret_cast<uint64_t *>(xs);
+            table[tid] = entry;
+            __syncthreads();
+            const int64_t n_end = (int64_t)n0 + kI8gBN < N ? (int64_t)n0 + kI8gBN : N;
+            const int64_t mc = M - m0 < kI8gBM ? M - m0 : kI8gBM;
+            int8_rows<false>(x + (int64_t)m0 * K, codes, table, table, out + (int64_t)m0 * N, mc, N, K, kTiled ? 1 : 0,
+                             false, (int64_t)n0 + wave, 4, n_end);
+            return;
+        }
+    }
+
+    // global sources, as raw buffer loads (rows past N / M and tiles past the end: zeros, no access)
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kTiled ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(x), 0, (int)((int64_t)M * K), 0x00020000);
+    // codes of row group i (32 rows): row-major 8 bytes at row * K / 4 + kt * 16 + 8 h; tiled: tile
+    // (row / 16, 2 kt + h) of 128 bytes, 16 bytes at (row % 8) * 16
+    int cvoff[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int n = n0 + wave * 64 + i * 32 + l32;
+        if (kTiled) cvoff[i] = n < N ? (n >> 4) * 16 * row_bytes + kq * 128 + (n & 7) * 16 : kOut;
+        else cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
+    }
+    const uint32_t half_sel = (l32 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
+    // x: load p of thread tid is piece tid % 4 (16 bytes) of row 64 p + tid / 4 of the tile
+    int xvoff[2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const int m = m0 + 64 * p + (tid >> 2);
+        xvoff[p] = m < M ? m * K + (tid & 3) * 16 : kOut;
+    }
+    unsigned char *xw_ptr = xs + (tid >> 2) * kI8gLd + (tid & 3) * 16;
+    const uint32_t xr_addr = lds_addr(xs) + (uint32_t)(l32 * kI8gLd + kq * 32);
+
+    struct Stage {
+        u4_t cw[2];   // row-major: only the low 8 bytes are loaded
+        u4_t xv[2];
+    };
+    auto load = [&](Stage &st, int kt) {
+        const int ok = kt < k_tiles;
+        const int coff = ok ? (kTiled ? kt * 256 : kt * 16) : kOut;
+        const int xoff = ok ? kt * kI8gBK : kOut;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (kTiled) {
+                st.cw[i] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, cvoff[i], coff, 0);
+            } else {
+                const u2_t v = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
+                st.cw[i] = u4_t{v[0], v[1], 0u, 0u};
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 2; p++) st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
+    };
+    auto stage_x = [&](const Stage &st, int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++)
+            *reinterpret_cast<u4_t *>(xw_ptr + buf * kI8gBM * kI8gLd + p * 64 * kI8gLd) = st.xv[p];
+    };
+
+    i16_t acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
+
+    // k tile kt out of LDS buffer kt % 2 with the codes of ring slot `cur`; then the x of tile
+    // kt + 1 (slot `nxt`, loaded three tiles ago) goes to the other buffer, slot `cur` is refilled
+    // with tile kt + 4, and the barrier hands the buffers over
+    auto tile = [&](int kt, Stage &cur, const Stage &nxt) {
+        const uint32_t xb_addr = xr_addr + (uint32_t)((kt & 1) * kI8gBM * kI8gLd);
+        u4_t b[4][2];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) b[j][s2] = lds_read16(xb_addr + (uint32_t)(j * 32 * kI8gLd + s2 * 16));
+        uint32_t cwi[2][2];   // [row group][MFMA step]: two codes each
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (kTiled) {
+                cwi[i][0] = __builtin_amdgcn_perm(cur.cw[i][1], cur.cw[i][0], half_sel);
+                cwi[i][1] = __builtin_amdgcn_perm(cur.cw[i][3], cur.cw[i][2], half_sel);
+            } else {
+                cwi[i][0] = cur.cw[i][0];
+                cwi[i][1] = cur.cw[i][1];
+            }
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const uint32_t w = cwi[i][s2];
+                const u2_t g0 = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
+                const u2_t k0 = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
+                const u2_t g1 = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
+                const u2_t k1 = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
+                const i4_t a = i4_t{(int)(g0[0] ^ k0[0]), (int)(g0[1] ^ k0[1]), (int)(g1[0] ^ k1[0]), (int)(g1[1] ^ k1[1])};
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, __builtin_bit_cast(i4_t, b[j][s2]), acc[i][j], 0, 0, 0);
+            }
+        stage_x(nxt, (kt + 1) & 1);
+        load(cur, kt + 4);
+        __syncthreads();
+    };
+
+    Stage ring[4];
+#pragma unroll
+    for (int d = 0; d < 4; d++) load(ring[d], d);
+    stage_x(ring[0], 0);
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 4 <= k_tiles; kt += 4) {
+        tile(kt, ring[0], ring[1]);
+        tile(kt + 1, ring[1], ring[2]);
+        tile(kt + 2, ring[2], ring[3]);
+        tile(kt + 3, ring[3], ring[0]);
+    }
+    if (kt < k_tiles) tile(kt, ring[0], ring[1]);
+    if (kt + 1 < k_tiles) tile(kt + 1, ring[1], ring[2]);
+    if (kt + 2 < k_tiles) tile(kt + 2, ring[2], ring[3]);
+
+    // D layout of 32x32: element e of lane: row (n) = 8 * (e / 4) + 4 * (lane / 32) + e % 4, column (m) = lane % 32
+    const bool n_vec = (N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int m = m0 + j * 32 + l32;
+            if (m >= M) continue;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; e4++) {
+                const int n = n0 + wave * 64 + i * 32 + 8 * e4 + 4 * kq;
+                int32_t *dst = out + (int64_t)m * N + n;
+                if (n_vec && n + 3 < N) {
+                    *reinterpret_cast<i4_t *>(dst) = i4_t{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < N) dst[e] = acc[i][j][4 * e4 + e];
+                }
+            }
+        }
+}
+
 __global__ void zero_i32_kernel(int32_t *y, int64_t n)
 {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -2657,6 +2871,38 @@ int launch_int8x(const void *x, const void *codes, const void *cb, void *out, in
                                  (int)N, (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
 
+// Which kernel the integer operator takes for 16-byte aligned buffers.  Many rows of x: the
+// matrix-matrix kernel costs about K * 11.5 ns per round of one 256 x 128 tile per CU (47 us at
+// K = 4096) however few of its tiles exist, the matrix-vector kernel about 3 us plus its code
+// bytes at 3.5 TB/s per 16 rows of x; the cheaper estimate wins (M = 64 at 4096 x 4096: four
+// matrix-vector launches, 20 us; M = 256: one matrix-matrix launch, 47 us against 75).
+enum Int8Kind { kInt8Scalar, kInt8Gemv, kInt8Gemm };
+Int8Kind pick_int8(int64_t M, int64_t N, int64_t K)
+{
+    if (M < 1 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31) || K > (1 << 17) ||
+        !int8x_enabled())
+        return kInt8Scalar;
+    if (M > 16 && M * K < (1LL << 31)) {
+        const int64_t cus = cu_count();
+        const int64_t tiles = ((M + kI8gBM - 1) / kI8gBM) * ((N + kI8gBN - 1) / kI8gBN);
+        const double t_gemm = 3.0 + (double)((tiles + cus - 1) / cus) * (double)K * 0.0115;
+        const double t_gemv = (double)((M + 15) / 16) * (3.0 + (double)N * (double)(K >> 2) / 3.5e6);
+        if (t_gemm < t_gemv) return kInt8Gemm;
+    }
+    return kInt8Gemv;
+}
+
+template <bool kTiled>
+int launch_int8g(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+                 hipStream_t stream)
+{
+    static bool attr_done[kMaxDevices] = {};
+    if (int e = allow_dynamic_lds(int8g_kernel<kTiled>, kI8gSmem, attr_done)) return e;
+    dim3 g((unsigned)((M + kI8gBM - 1) / kI8gBM), (unsigned)((N + kI8gBN - 1) / kI8gBN));
+    return launch(int8g_kernel<kTiled>, g, dim3(256), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
+                  (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
+}
+
 // one launch for up to 16 rows of x; first / last: position in the operator call's sequence of
 // launches, for the timing events
 template <bool kTiled>
@@ -2763,6 +3009,15 @@ int dmm_set_gemv_8bit(int enabled)
     return before;
 }
 
+const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K)
+{
+    switch (pick_int8(M, N, K)) {
+        case kInt8Gemm: return "dmm::int8g_kernel";
+        case kInt8Gemv: return "dmm::int8x_kernel";
+        default: return "dmm::int8_kernel";
+    }
+}
+
 const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K)
 {
     if (M < 1 || M > 32 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31)) return "";
@@ -2861,12 +3116,14 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
         const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
         return launch(zero_i32_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (int32_t *)out, n);
     }
-    // the matrix-unit kernel takes up to 16 rows of x per launch; K <= 2^17: its weights are odd,
-    // so |w| <= 127 and no sum of K products leaves int32 - nothing depends on what the matrix
-    // unit does on overflow
-    if ((K & 255) == 0 && (N & 3) == 0 && N * (K >> 2) < (1LL << 31) && K <= (1 << 17) && aligned(x, 16) &&
-        aligned(codes, 16) && aligned(out, 16) && int8x_enabled()) {
-        for (int64_t m0 = 0; m0 < M; m0 += 16) {
+    // the matrix-unit kernels (K <= 2^17: their weights are odd, so |w| <= 127 and no sum of K
+    // products leaves int32 - nothing depends on what the matrix unit does on overflow)
+    const Int8Kind kind = aligned(x, 16) && aligned(codes, 16) && aligned(out, 16) ? pick_int8(M, N, K) : kInt8Scalar;
+    if (kind == kInt8Gemm)
+        return tiled ? launch_int8g<true>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream)
+                     : launch_int8g<false>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream);
+    if (kind == kInt8Gemv) {
+        for (int64_t m0 = 0; m0 < M; m0 += 16) {   // up to 16 rows of x per launch
             const int64_t mc = M - m0 < 16 ? M - m0 : 16;
             const int8_t *xs = (const int8_t *)x + m0 * K;
             int32_t *os = (int32_t *)out + m0 * N;

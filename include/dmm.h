@@ -176,6 +176,12 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
 int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_abs, void *out,
                          int64_t M, int64_t N, int64_t K, int tiled, void *stream);
 
+/* Which kernel dmm_decode_matmul_i8 takes for this shape when x, codes and out are 16-byte
+ * aligned: "dmm::int8g_kernel" (matrix-matrix, many rows of x), "dmm::int8x_kernel"
+ * (matrix-vector, 16 rows of x per launch) or "dmm::int8_kernel" (scalar).  For tests and
+ * benchmarks; no counterpart in the reference. */
+const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K);
+
 /* Kernel timing hook for benchmarks.  While a (start, stop) pair of hipEvent_t handles is
  * set on the calling thread, the dominant kernel of each operator call records `start`
  * immediately before and `stop` immediately after itself on the GPU timeline, so

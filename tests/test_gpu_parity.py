@@ -403,6 +403,7 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     launches), both code layouts, N no multiple of 16 (row-major), and a table with bytes that are
     not 2 mod 4, which every workgroup must notice and serve with the scalar decode.  Exact
     against the oracle's restatement of /root/reference/test_decode_matmul.py:58-71."""
+    assert capi.lib().dmm_integer_kernel_name(M, N, K) in (b"dmm::int8x_kernel", b"dmm::int8g_kernel")
     rng = np.random.default_rng(M * 977 + N + K)
     if table == "e8p":
         cb = orc.build_codebook_abs()
@@ -417,6 +418,36 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     out = c_matmul_i8(dev(x), cd, dev(cb), tiled)
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M,N,K,tiled,table", [
+    (128, 32768, 256, True, "e8p"), (300, 16 * 1030, 512, False, "mod4"), (64, 40000, 256, False, "any"),
+    (2048, 4096, 512, True, "e8p"), (200, 16 * 1030, 1280, True, "mod4"), (129, 16 * 1030, 256, True, "any"),
+    (256, 4096, 4096, True, "e8p"), (512, 2048, 8192, False, "mod4")])
+def test_integer_operator_matrix_matrix(M, N, K, tiled, table):
+    """Many rows of x run on the int8 matrix-matrix kernel: partial tiles in M and N, both code layouts, 4 to 20 k tiles, and a
+    table with bytes that are not 2 mod 4 (scalar decode per workgroup, with x rows and output
+    rows offset by the workgroup's m block).  Exact against the oracle's decode times x in
+    float64 (every sum is far below 2^53, so that product is the integer one)."""
+    assert capi.lib().dmm_integer_kernel_name(M, N, K) == b"dmm::int8g_kernel"
+    rng = np.random.default_rng(M * 31 + N + K)
+    if table == "e8p":
+        cb = orc.build_codebook_abs()
+    elif table == "mod4":
+        cb = ((rng.integers(0, 256, size=(256, 8)).astype(np.uint8) & 0xFC) | 2).view(np.int64).reshape(256).copy()
+    else:
+        cb = rng.integers(-2 ** 63, 2 ** 63, size=256, dtype=np.int64)
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    W = orc.decode_i8(codes, cb)
+    want = (x.astype(np.float64) @ W.astype(np.float64).T).astype(np.int64).astype(np.int32)
+    cd = dev(orc.transpose_tile(codes)) if tiled else dev(codes)
+    out = c_matmul_i8(dev(x), cd, dev(cb), tiled)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+    # a few rows against the integer oracle itself
+    rows = np.r_[0:2, M - 2:M]
+    assert np.array_equal(out.cpu().numpy()[rows], orc.decode_matmul_i32(x[rows], codes, cb))
 
 
 def test_integer_operator_golden_cases_and_edges():
