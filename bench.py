@@ -25,6 +25,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
+MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 # HBM bytes one GEMV launch moves, per kernel, averaged over the shapes of the step that kernel
 # serves: rocprofv3 FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter
 # reads for a plain 256 MiB device copy (x2.000 and x1.000).
@@ -413,8 +414,29 @@ def integer_operator(torch, lib, capi, workload, dev, stream, rand_codes):
             t = timed_kernel(torch, lib, fn, 40)
             rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3),
                          "GBps_code": round(workload.code_bytes(N, K) / t / 1e9, 1),
-                         "frac_hbm": round(workload.code_bytes(N, K) / t / 1e9 / HBM_PEAK_GBS, 4)})
+                         "frac_hbm": round(workload.code_bytes(N, K) / t / 1e9 / HBM_PEAK_GBS, 4),
+                         "kernel": lib.dmm_integer_kernel_name(M, N, K).decode()})
         del codes
+    # M = 2048 at the prefill shapes: the int8 matrix-matrix kernel (2 M N K integer operations)
+    M = 2048
+    for K, N in workload.PREFILL:
+        codes = rand_codes(N, K, 2, 13)
+        g = torch.Generator(device=dev)
+        g.manual_seed(6)
+        x = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8, device=dev)
+        out = torch.empty(M, N, dtype=torch.int32, device=dev)
+
+        def fn(i):
+            st = lib.dmm_decode_matmul_i8(x.data_ptr(), codes[i % 2].data_ptr(), cb.data_ptr(), out.data_ptr(),
+                                          M, N, K, 1, stream)
+            assert st == 0, st
+        for i in range(3):
+            fn(i)
+        t = timed_kernel(torch, lib, fn, 20)
+        rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 2),
+                     "TOPs": round(workload.flops(M, N, K) / t / 1e12, 1),
+                     "frac_mfma_i8": round(workload.flops(M, N, K) / t / 1e12 / MFMA_I8_PEAK_TOPS, 4),
+                     "kernel": lib.dmm_integer_kernel_name(M, N, K).decode()})
     return rows
 
 

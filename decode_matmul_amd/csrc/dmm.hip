@@ -2167,8 +2167,8 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 
 
 // ------------------------------------------------------------------ the integer operator, many rows of x
-// Block tile 256 (n) x 128 (m) x 64 (k), four waves, each 64 rows of W x all 128 rows of x = 8
-// accumulators of v_mfma_i32_32x32x32_i8.  Like the half-precision gemm_reg_kernel, every wave
+// Block tile 256 (n) x 128 (m) x 64 (k), eight waves (two per SIMD, to hide the table gathers),
+// each 32 rows of W x all 128 rows of x = 4 accumulators of v_mfma_i32_32x32x32_i8.  Like the half-precision gemm_reg_kernel, every wave
 // decodes its own rows straight into A operands - here that is two 8-byte gathers and two
 // exclusive ors per code (int8x_kernel's tables), four codes per lane and k tile - and only x goes
 // through the LDS (rows 80 bytes apart: the 16 lanes the LDS serves per clock, 16 consecutive
@@ -2183,7 +2183,7 @@ constexpr int kI8gBN = 256, kI8gBM = 128, kI8gBK = 64, kI8gLd = 80;
 constexpr int kI8gSmem = 2 * kI8TableBytes + 2 * kI8gBM * kI8gLd;
 
 template <bool kTiled>
-__global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+__global__ __launch_bounds__(512) void int8g_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
                                                     const int64_t *__restrict__ codebook_abs,
                                                     int32_t *__restrict__ out, int M, int N, int K)
 {
@@ -2202,24 +2202,24 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
     const int k_tiles = K / kI8gBK;
     constexpr int kOut = (int)0x80000000;
 
-    // tables: thread tid writes the 32 copies of table entry tid and of the mask of high byte tid
-    const uint64_t entry = (uint64_t)codebook_abs[tid];
+    // tables: threads 0 .. 255 write the 32 copies of table entry tid, threads 256 .. 511 those of
+    // the mask of high byte tid - 256 (the mask table follows the grid table: row tid either way)
+    const uint64_t entry = tid < 256 ? (uint64_t)codebook_abs[tid] : 0x0202020202020202ull;
     {
-        uint32_t s8 = (uint32_t)tid & 0x7Fu;
-        s8 |= (__builtin_popcount(s8) & 1u) << 7;
-        uint64_t mk = (tid >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
+        uint64_t v = entry;
+        if (tid >= 256) {
+            const uint32_t t = (uint32_t)tid - 256u;
+            uint32_t s8 = t & 0x7Fu;
+            s8 |= (__builtin_popcount(s8) & 1u) << 7;
+            v = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
 #pragma unroll
-        for (int d = 0; d < 8; d++)
-            if ((s8 >> d) & 1u) mk ^= 0xFCull << (8 * d);
-        u4_t *grow = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;
-        u4_t *mrow = reinterpret_cast<u4_t *>(smem_raw + kI8TableBytes) + tid * 16;
-        const u4_t gv = u4_t{(uint32_t)entry, (uint32_t)(entry >> 32), (uint32_t)entry, (uint32_t)(entry >> 32)};
-        const u4_t mv = u4_t{(uint32_t)mk, (uint32_t)(mk >> 32), (uint32_t)mk, (uint32_t)(mk >> 32)};
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            grow[(i + tid) & 15] = gv;   // 16 lanes, 16 bank groups
-            mrow[(i + tid) & 15] = mv;
+            for (int d = 0; d < 8; d++)
+                if ((s8 >> d) & 1u) v ^= 0xFCull << (8 * d);
         }
+        u4_t *rowp = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;
+        const u4_t vv = u4_t{(uint32_t)v, (uint32_t)(v >> 32), (uint32_t)v, (uint32_t)(v >> 32)};
+#pragma unroll
+        for (int i = 0; i < 16; i++) rowp[(i + tid) & 15] = vv;   // 16 lanes, 16 bank groups
     }
     // the vote on the table (one word per wave in the x area, read by everybody after the barrier)
     {
@@ -2228,16 +2228,16 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
         const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
         if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
         __syncthreads();
-        const bool any_bad = (votes[0] | votes[1] | votes[2] | votes[3]) != 0;
+        const bool any_bad = (votes[0] | votes[1] | votes[2] | votes[3]) != 0;   // the table is in waves 0 - 3
         __syncthreads();   // the votes are read before x overwrites them
         if (any_bad) {
             uint64_t *table = reinterpret_cast<uint64_t *>(xs);
-            table[tid] = entry;
+            if (tid < 256) table[tid] = entry;
             __syncthreads();
             const int64_t n_end = (int64_t)n0 + kI8gBN < N ? (int64_t)n0 + kI8gBN : N;
             const int64_t mc = M - m0 < kI8gBM ? M - m0 : kI8gBM;
             int8_rows<false>(x + (int64_t)m0 * K, codes, table, table, out + (int64_t)m0 * N, mc, N, K, kTiled ? 1 : 0,
-                             false, (int64_t)n0 + wave, 4, n_end);
+                             false, (int64_t)n0 + wave, 8, n_end);
             return;
         }
     }
@@ -2249,57 +2249,47 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
         __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(x), 0, (int)((int64_t)M * K), 0x00020000);
     // codes of row group i (32 rows): row-major 8 bytes at row * K / 4 + kt * 16 + 8 h; tiled: tile
     // (row / 16, 2 kt + h) of 128 bytes, 16 bytes at (row % 8) * 16
-    int cvoff[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int n = n0 + wave * 64 + i * 32 + l32;
-        if (kTiled) cvoff[i] = n < N ? (n >> 4) * 16 * row_bytes + kq * 128 + (n & 7) * 16 : kOut;
-        else cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
+    int cvoff;
+    {
+        const int n = n0 + wave * 32 + l32;
+        if (kTiled) cvoff = n < N ? (n >> 4) * 16 * row_bytes + kq * 128 + (n & 7) * 16 : kOut;
+        else cvoff = n < N ? n * row_bytes + kq * 8 : kOut;
     }
     const uint32_t half_sel = (l32 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
-    // x: load p of thread tid is piece tid % 4 (16 bytes) of row 64 p + tid / 4 of the tile
-    int xvoff[2];
-#pragma unroll
-    for (int p = 0; p < 2; p++) {
-        const int m = m0 + 64 * p + (tid >> 2);
-        xvoff[p] = m < M ? m * K + (tid & 3) * 16 : kOut;
+    // x: thread tid loads piece tid % 4 (16 bytes) of row tid / 4 of the tile
+    int xvoff;
+    {
+        const int m = m0 + (tid >> 2);
+        xvoff = m < M ? m * K + (tid & 3) * 16 : kOut;
     }
     unsigned char *xw_ptr = xs + (tid >> 2) * kI8gLd + (tid & 3) * 16;
     const uint32_t xr_addr = lds_addr(xs) + (uint32_t)(l32 * kI8gLd + kq * 32);
 
     struct Stage {
-        u4_t cw[2];   // row-major: only the low 8 bytes are loaded
-        u4_t xv[2];
+        u4_t cw;   // row-major: only the low 8 bytes are loaded
+        u4_t xv;
     };
     auto load = [&](Stage &st, int kt) {
         const int ok = kt < k_tiles;
         const int coff = ok ? (kTiled ? kt * 256 : kt * 16) : kOut;
         const int xoff = ok ? kt * kI8gBK : kOut;
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            if (kTiled) {
-                st.cw[i] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, cvoff[i], coff, 0);
-            } else {
-                const u2_t v = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
-                st.cw[i] = u4_t{v[0], v[1], 0u, 0u};
-            }
+        if (kTiled) {
+            st.cw = __builtin_amdgcn_raw_buffer_load_b128(crsrc, cvoff, coff, 0);
+        } else {
+            const u2_t v = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff, coff, 0);
+            st.cw = u4_t{v[0], v[1], 0u, 0u};
         }
-#pragma unroll
-        for (int p = 0; p < 2; p++) st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
+        st.xv = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff, xoff, 0);
     };
     auto stage_x = [&](const Stage &st, int buf) {
-#pragma unroll
-        for (int p = 0; p < 2; p++)
-            *reinterpret_cast<u4_t *>(xw_ptr + buf * kI8gBM * kI8gLd + p * 64 * kI8gLd) = st.xv[p];
+        *reinterpret_cast<u4_t *>(xw_ptr + buf * kI8gBM * kI8gLd) = st.xv;
     };
 
-    i16_t acc[2][4];
+    i16_t acc[4];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int j = 0; j < 4; j++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
+        for (int e = 0; e < 16; e++) acc[j][e] = 0;
 
     // k tile kt out of LDS buffer kt % 2 with the codes of ring slot `cur`; then the x of tile
     // kt + 1 (slot `nxt`, loaded three tiles ago) goes to the other buffer, slot `cur` is refilled
@@ -2311,31 +2301,31 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
         for (int j = 0; j < 4; j++)
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) b[j][s2] = lds_read16(xb_addr + (uint32_t)(j * 32 * kI8gLd + s2 * 16));
-        uint32_t cwi[2][2];   // [row group][MFMA step]: two codes each
+        uint32_t cwi[2];   // [MFMA step]: two codes each
+        if (kTiled) {
+            cwi[0] = __builtin_amdgcn_perm(cur.cw[1], cur.cw[0], half_sel);
+            cwi[1] = __builtin_amdgcn_perm(cur.cw[3], cur.cw[2], half_sel);
+        } else {
+            cwi[0] = cur.cw[0];
+            cwi[1] = cur.cw[1];
+        }
+        u2_t g[4], k[4];   // all 8 gathers of the tile go out before the first MFMA
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            if (kTiled) {
-                cwi[i][0] = __builtin_amdgcn_perm(cur.cw[i][1], cur.cw[i][0], half_sel);
-                cwi[i][1] = __builtin_amdgcn_perm(cur.cw[i][3], cur.cw[i][2], half_sel);
-            } else {
-                cwi[i][0] = cur.cw[i][0];
-                cwi[i][1] = cur.cw[i][1];
-            }
+        for (int s2 = 0; s2 < 2; s2++) {
+            const uint32_t w = cwi[s2];
+            g[2 * s2] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
+            k[2 * s2] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
+            g[2 * s2 + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
+            k[2 * s2 + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
         }
 #pragma unroll
-        for (int s2 = 0; s2 < 2; s2++)
+        for (int s2 = 0; s2 < 2; s2++) {
+            const i4_t a = i4_t{(int)(g[2 * s2][0] ^ k[2 * s2][0]), (int)(g[2 * s2][1] ^ k[2 * s2][1]),
+                                (int)(g[2 * s2 + 1][0] ^ k[2 * s2 + 1][0]), (int)(g[2 * s2 + 1][1] ^ k[2 * s2 + 1][1])};
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const uint32_t w = cwi[i][s2];
-                const u2_t g0 = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
-                const u2_t k0 = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
-                const u2_t g1 = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
-                const u2_t k1 = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
-                const i4_t a = i4_t{(int)(g0[0] ^ k0[0]), (int)(g0[1] ^ k0[1]), (int)(g1[0] ^ k1[0]), (int)(g1[1] ^ k1[1])};
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, __builtin_bit_cast(i4_t, b[j][s2]), acc[i][j], 0, 0, 0);
-            }
+            for (int j = 0; j < 4; j++)
+                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, __builtin_bit_cast(i4_t, b[j][s2]), acc[j], 0, 0, 0);
+        }
         stage_x(nxt, (kt + 1) & 1);
         load(cur, kt + 4);
         __syncthreads();
@@ -2360,24 +2350,22 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
     // D layout of 32x32: element e of lane: row (n) = 8 * (e / 4) + 4 * (lane / 32) + e % 4, column (m) = lane % 32
     const bool n_vec = (N & 3) == 0;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int j = 0; j < 4; j++) {
+        const int m = m0 + j * 32 + l32;
+        if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int m = m0 + j * 32 + l32;
-            if (m >= M) continue;
+        for (int e4 = 0; e4 < 4; e4++) {
+            const int n = n0 + wave * 32 + 8 * e4 + 4 * kq;
+            int32_t *dst = out + (int64_t)m * N + n;
+            if (n_vec && n + 3 < N) {
+                *reinterpret_cast<i4_t *>(dst) = i4_t{acc[j][4 * e4], acc[j][4 * e4 + 1], acc[j][4 * e4 + 2], acc[j][4 * e4 + 3]};
+            } else {
 #pragma unroll
-            for (int e4 = 0; e4 < 4; e4++) {
-                const int n = n0 + wave * 64 + i * 32 + 8 * e4 + 4 * kq;
-                int32_t *dst = out + (int64_t)m * N + n;
-                if (n_vec && n + 3 < N) {
-                    *reinterpret_cast<i4_t *>(dst) = i4_t{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (n + e < N) dst[e] = acc[i][j][4 * e4 + e];
-                }
+                for (int e = 0; e < 4; e++)
+                    if (n + e < N) dst[e] = acc[j][4 * e4 + e];
             }
         }
+    }
 }
 
 __global__ void zero_i32_kernel(int32_t *y, int64_t n)
@@ -2899,7 +2887,7 @@ int launch_int8g(const void *x, const void *codes, const void *cb, void *out, in
     static bool attr_done[kMaxDevices] = {};
     if (int e = allow_dynamic_lds(int8g_kernel<kTiled>, kI8gSmem, attr_done)) return e;
     dim3 g((unsigned)((M + kI8gBM - 1) / kI8gBM), (unsigned)((N + kI8gBN - 1) / kI8gBN));
-    return launch(int8g_kernel<kTiled>, g, dim3(256), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
+    return launch(int8g_kernel<kTiled>, g, dim3(512), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
                   (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
 }
 

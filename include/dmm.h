@@ -169,8 +169,9 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
  * decode_matmul_cuda.cu:196-197 does); tiled == 0: plain row-major [N, K/8].  None of the
  * reference's other shape demands (M % 8, K % 2048, K >= 4096) apply.  Exact integer
  * arithmetic (int32 sums wrap); `out` is fully overwritten.  With K % 256 == 0, N % 4 == 0 and
- * 16-byte aligned x, codes and out the call runs on the int8 matrix unit, 16 rows of x per
- * launch (a table with a byte that is not 2 mod 4 - the E8P table has none - is noticed inside
+ * 16-byte aligned x, codes and out the call runs on the int8 matrix unit - 16 rows of x per
+ * launch of a matrix-vector kernel, or one launch of a matrix-matrix kernel when x has many rows
+ * (a table with a byte that is not 2 mod 4 - the E8P table has none - is noticed inside
  * the launch and served by the scalar decode); anything else takes the scalar kernel, one wave
  * per output row.  DMM_INT8_MFMA=0 in the environment keeps every call on the scalar kernel. */
 int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_abs, void *out,
