@@ -66,11 +66,24 @@ __all__ = [
 ]
 
 
-def decode_matmul(x, codes, grid, scale):
-    """y[M,N] = half(scale * x @ decode(codes, grid).T), fp32 accumulation, on x's device and
-    the current stream, asynchronously.  Same role as the reference's `decode_matmul`
-    (decode_matmul_cuda.cu:178-234); raises RuntimeError on bad inputs like its TORCH_CHECKs."""
-    return _ext().decode_matmul(x, codes, grid, float(scale))
+def decode_matmul(x, codes, table, scale=None):
+    """The operator under the reference's name, dispatching on the dtype of x.
+
+    Half x: `decode_matmul(x, codes, grid, scale)` -> half y[M,N] = half(scale * x @
+    decode(codes, grid).T), fp32 accumulation; codes row-major [N, K/8], grid half [256,8].
+    int8 x: the reference's own call `decode_matmul(x, weights_compressed, codebook_abs)`
+    (decode_matmul_cuda.cu:178-181, test_decode_matmul.py:136) -> int32 [M,N], exact; codes in the
+    reference's tile order (`transpose_tile`), table int64[256]; no scale.
+
+    Runs on x's device and the current stream, asynchronously; raises RuntimeError on bad
+    inputs like the reference's TORCH_CHECKs (decode_matmul_cuda.cu:182-207)."""
+    if x.dtype == _torch.int8:
+        if scale is not None:
+            raise TypeError("decode_matmul: the integer form (int8 x) takes no scale")
+        return _ext().decode_matmul_int8(x, codes, table, True)
+    if scale is None:
+        raise TypeError("decode_matmul: the half-precision form needs a scale")
+    return _ext().decode_matmul(x, codes, table, float(scale))
 
 
 def decode_matmul_path(x, codes, grid, scale, path="auto"):

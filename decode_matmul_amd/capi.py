@@ -14,6 +14,7 @@ _OP = [_P, _P, _P, _F, _P, _I64, _I64, _I64, _P]
 SYMBOLS = {
     "dmm_version": (ctypes.c_int, []),
     "dmm_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "dmm_init": (ctypes.c_int, [ctypes.c_int]),
     "dmm_decode_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "dmm_decode_matmul_f16": (ctypes.c_int, _OP),
     "dmm_gemv_f16": (ctypes.c_int, _OP),

@@ -13,6 +13,8 @@
 // matrix-vector path.
 #include <hip/hip_runtime.h>
 #include <atomic>
+#include <mutex>
+#include <vector>
 #include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -259,28 +261,6 @@ __device__ __forceinline__ uint32_t pk_fma_bcast(uint32_t g, uint32_t s, uint32_
 //     the lane's copy offset.
 // LDS map: [0, 32K) sign rows (128 x 256 B), [32K, 96K) grid rows (256 x 256 B),
 //          then 2 x (W x R x 4 x M) float4 partial sums (double-buffered per row block), then x.
-#ifdef DMM_TRACE
-// Experiment build only: per-wave timestamps kept in the last 4 KB of LDS and copied out
-// when the wave ends, so that marking does not disturb the vector-memory queue.
-__device__ unsigned long long *dmm_trace_buf = nullptr;
-__device__ int dmm_exp_mode = 0;   // 1: loads only (no decode), 2: decode only (no HBM traffic)
-#define DMM_TRACE_SLOTS 32
-#define DMM_TRACE_LDS(smem) (reinterpret_cast<unsigned long long *>((smem) + 160 * 1024 - 16 * DMM_TRACE_SLOTS * 8))
-#define DMM_TRACE_MARK(slot)                                                                         \
-    do {                                                                                             \
-        if ((threadIdx.x & 63) == 0)                                                                 \
-            DMM_TRACE_LDS(smem_raw)[(threadIdx.x >> 6) * DMM_TRACE_SLOTS + (slot)] = __builtin_amdgcn_s_memrealtime(); \
-    } while (0)
-#define DMM_TRACE_DUMP()                                                                             \
-    do {                                                                                             \
-        if (dmm_trace_buf && (threadIdx.x & 63) < DMM_TRACE_SLOTS)                                   \
-            dmm_trace_buf[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * DMM_TRACE_SLOTS + (threadIdx.x & 63)] = \
-                DMM_TRACE_LDS(smem_raw)[(threadIdx.x >> 6) * DMM_TRACE_SLOTS + (threadIdx.x & 63)];  \
-    } while (0)
-#else
-#define DMM_TRACE_MARK(slot) do { } while (0)
-#define DMM_TRACE_DUMP() do { } while (0)
-#endif
 
 constexpr int kSSignBytes = 128 * 256;
 constexpr int kSGridBytes = 256 * 256;
@@ -448,8 +428,6 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
 {
     static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
-    DMM_TRACE_MARK(0);
     f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // [2][W][R][4 * M]
     const int red_par = W * R * 4 * M;                                 // float4 per parity
     unsigned char *xs = smem_raw + kSTablesBytes + stream_red_bytes(R, W, M);
@@ -503,13 +481,8 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
     int pf_blk = 0, pf_j = 0;
     auto issue = [&](u4_t (&cwd)[R]) {
         const bool ok = pf_blk < nb_wg && n_sw > 0;
-#ifdef DMM_TRACE
-        const bool ok2 = ok && dmm_exp_mode != 2;
-#else
-        const bool ok2 = ok;
-#endif
         const int tb = t0 + pf_blk * R;
-        const int soff = !ok2 ? kOut
+        const int soff = !ok ? kOut
                          : kPacked ? (tb * n_steps + wave + pf_j * W) * 1024
                                    : tb * 16 * row_bytes + (wave + pf_j * W) * 64;
 #pragma unroll
@@ -521,7 +494,6 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
     u4_t cw[D][R];
 #pragma unroll
     for (int d = 0; d < D; d++) issue(cw[d]);
-    DMM_TRACE_MARK(1);
     stream_stage_signs<64 * W>(smem_raw, tid);
     __builtin_amdgcn_sched_barrier(0);   // keep the sign rows ahead of the waits for the loads
 
@@ -537,11 +509,8 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
         for (int c = tid; c < row_chunks; c += 64 * W)
             reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = reinterpret_cast<const u4_t *>(x + (int64_t)m * K)[c];
     if (tid >= 64 * W - 8) reinterpret_cast<u4_t *>(xs + M * x_pitch)[tid - (64 * W - 8)] = u4_t{0u, 0u, 0u, 0u};
-    DMM_TRACE_MARK(2);
     stream_stage_grid<64 * W>(smem_raw, grow, tid);
-    DMM_TRACE_MARK(3);
     __syncthreads();
-    DMM_TRACE_MARK(4);
 
     // B operand address of this lane.  JP = 1: row m = c16 (row 0 for columns past M), quarter
     // q.  JP = 4: column c16 = 4 m + j reads piece j (and 4 + j) of row m's quarter; columns past
@@ -620,32 +589,20 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
 #pragma unroll
         for (int d = 0; d < D; d++) {
             if (i0 + d < n_items) {
-#ifdef DMM_TRACE
-                if (i0 + d < 7) { asm volatile("" ::"v"(cw[d][0])); DMM_TRACE_MARK(8 + 2 * (i0 + d)); }
-                if (dmm_exp_mode == 1) {
-#pragma unroll
-                    for (int r = 0; r < R; r++) acc[r][0][0] += __builtin_bit_cast(float, cw[d][r][0] ^ cw[d][r][1] ^ cw[d][r][2] ^ cw[d][r][3]);
-                } else
-#endif
                 {
                     const uint32_t xa = xlane + __umul24((uint32_t)(wave + j * W), xstride);
                     const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
                     stream_step<R, JP>(cw[d], xa, lane_base, quarter_bits, acc, nv);
                 }
-                if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
                 if (++j >= n_sw) {
                     j = 0;
-                    if (blk == 0) DMM_TRACE_MARK(5);
                     finish_block(blk);
-                    if (blk == 0) DMM_TRACE_MARK(6);
                     blk++;
                 }
             }
             issue(cw[d]);
         }
     }
-    DMM_TRACE_MARK(7);
-    DMM_TRACE_DUMP();
 }
 
 template <int R, int W, int D, bool kPacked, int JP>
@@ -873,8 +830,6 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
     static_assert(W == 16, "the table staging below assumes 1024 threads");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
-    DMM_TRACE_MARK(0);
     f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // two parities, see q8_red_bytes
     const int red_par = q8_red_bytes(R, W, M) / 32;                    // float4 per parity
     unsigned char *xt = smem_raw + kSTablesBytes + q8_red_bytes(R, W, M);
@@ -931,7 +886,6 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     u4_t cw[D][R];
 #pragma unroll
     for (int d = 0; d < D; d++) issue(cw[d]);
-    DMM_TRACE_MARK(1);
 
     bool fits = true;   // stays true while x is finite and the grid fits fp8
     if (wave >= 4 && wave < 8) {
@@ -963,7 +917,6 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             c += 64 * W;
         }
     }
-    DMM_TRACE_MARK(2);
     if (wave < 4) {
         // grid rows: thread tid converts row tid and writes its 16 slots (two copies each)
         bool exact;
@@ -973,7 +926,6 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
 #pragma unroll
         for (int i = 0; i < 16; i++) gg[(i + tid) & 15] = u4_t{g8[0], g8[1], g8[0], g8[1]};
     }
-    DMM_TRACE_MARK(3);
     // the vote: every wave publishes whether one of its rows or pieces failed, in a word of its own (so
     // nothing needs clearing first), and after the barrier every wave reads all of them
     uint32_t *votes = reinterpret_cast<uint32_t *>(x8t + 2 * M * x8_pitch);
@@ -987,7 +939,6 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
         return;
     }
 
-    DMM_TRACE_MARK(4);
     // B operand addresses of this lane: column c16 = 4 m + term (column 0 for the idle ones)
     // (kOne: columns 0 .. 7 = term c16 % 4 of the first or the second MFMA's 32 bytes, columns 8 and
     // 9 = the means hi and lo, whose rows advance 64 bytes per step where a term row advances 256;
@@ -1094,25 +1045,17 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             if (i0 + d < n_items) {
                 const uint32_t step = (uint32_t)(wave + j * W);
                 const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
-#ifdef DMM_TRACE
-                if (i0 + d < 7) { asm volatile("" ::"v"(cw[d][0])); DMM_TRACE_MARK(8 + 2 * (i0 + d)); }
-#endif
                 q8_step<R, kOne>(cw[d], kOne ? xlane + __umul24(step, xstride) : xlane + step * 256u, x8lane + step * 64u,
                                  lane_base, acc, accd, nv);
-                if (i0 + d < 7) DMM_TRACE_MARK(9 + 2 * (i0 + d));
                 if (++j >= n_sw) {
                     j = 0;
-                    if (blk == 0) DMM_TRACE_MARK(5);
                     finish_block(blk);
-                    if (blk == 0) DMM_TRACE_MARK(6);
                     blk++;
                 }
             }
             issue(cw[d]);
         }
     }
-    DMM_TRACE_MARK(7);
-    DMM_TRACE_DUMP();
 }
 
 // ------------------------------------------------------------------ small-batch matrix-vector path
@@ -1161,7 +1104,6 @@ __global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__res
 {
     static_assert(R >= 1 && R <= 4, "row tiles per block");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     typedef f4_t red_t[W][R * MT][kWave];
     red_t *red = reinterpret_cast<red_t *>(smem_raw + kSTablesBytes);   // red[parity]
 
@@ -1346,7 +1288,7 @@ template <int WN, int WM, int TN, int TM>
 __global__ __launch_bounds__(64 * WN * WM) void gemm_kernel(const uint16_t *__restrict__ x,
                                                             const uint16_t *__restrict__ codes,
                                                             const void *__restrict__ grid, float scale,
-                                                            uint16_t *__restrict__ y, int M, int N, int K)
+                                                            uint16_t *__restrict__ y, int M, int N, int K, int y_vec)
 {
     typedef GemmCfg<WN, WM, TN, TM> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
@@ -1496,7 +1438,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_kernel(const uint16_t *__re
     }
 
     // D layout of 32x32: element e of lane: row (n) = 8*(e/4) + 4*(lane/32) + e%4, column (m) = lane%32
-    const bool n_vec = (N & 3) == 0;
+    const bool n_vec = (N & 3) == 0 && y_vec != 0;   // 8-byte stores need an 8-byte aligned y
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
@@ -1568,11 +1510,10 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
                                                        const uint16_t *__restrict__ codes,
                                                        const void *__restrict__ grid, float scale,
                                                        uint16_t *__restrict__ y, float *__restrict__ part,
-                                                       int M, int N, int K, int splits)
+                                                       int M, int N, int K, int splits, int y_vec)
 {
     constexpr int kBM = 32 * TM;
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1762,7 +1703,7 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
 
     // D layout of 32x32: element e of lane: row (n) = 8*(e/4) + 4*(lane/32) + e%4, column (m) = lane%32
-    const bool n_vec = (N & 3) == 0;
+    const bool n_vec = (N & 3) == 0 && (kSplit || y_vec != 0);   // 8-byte stores need an 8-byte aligned y
 #pragma unroll
     for (int i = 0; i < kGrTN; i++)
 #pragma unroll
@@ -1986,7 +1927,6 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 {
     static_assert(W == 8, "the table staging below assumes 512 threads");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     // partial sums: two buffers taken in turn while they fit beside the tables (R <= 2), else one
     // and a second barrier per row block
     constexpr bool kTwoBuffers = R <= 2;
@@ -2188,7 +2128,6 @@ __global__ __launch_bounds__(512) void int8g_kernel(const int8_t *__restrict__ x
                                                     int32_t *__restrict__ out, int M, int N, int K)
 {
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    if (lds_addr(smem_raw) != 0) return;   // the table addressing assumes LDS offset 0 (no static LDS here)
     unsigned char *xs = smem_raw + 2 * kI8TableBytes;   // two x tiles of 128 rows x 80 bytes
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -2395,20 +2334,139 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ 
 thread_local hipEvent_t tls_start = nullptr;
 thread_local hipEvent_t tls_stop = nullptr;
 
-// kFirst / kLast: whether this launch opens / closes the span the timing events bracket (an
-// operator call that takes two kernels records start before the first and stop after the second)
-template <bool kFirst = true, bool kLast = true, typename Kern, typename... Args>
-int launch(Kern kernel, dim3 grid, dim3 block, size_t shmem, hipStream_t stream, Args... args)
+template <typename T>
+struct same_type { typedef T type; };
+
+// Enqueue one kernel; the status is what the launch call itself returns (no look at the
+// thread's last-error state, which may hold somebody else's stale error).  kFirst / kLast:
+// whether this launch opens / closes the span the timing events bracket (an operator call
+// that takes two kernels records start before the first and stop after the second).
+template <bool kFirst = true, bool kLast = true, typename... KArgs>
+int launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStream_t stream,
+           typename same_type<KArgs>::type... args)
 {
+    void *argv[] = {(void *)&args...};
     if (tls_start && tls_stop)
-        hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, kFirst ? tls_start : nullptr,
-                              kLast ? tls_stop : nullptr, 0, args...);
-    else
-        hipLaunchKernelGGL(kernel, grid, block, shmem, stream, args...);
-    return (int)hipGetLastError();
+        return (int)hipExtLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream,
+                                       kFirst ? tls_start : nullptr, kLast ? tls_stop : nullptr, 0);
+    return (int)hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream);
 }
 
 inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---- per-device state, set up by dmm_init --------------------------------------------------
+constexpr int kMaxDevices = 64;
+constexpr int kLdsMax = 160 * 1024;
+
+struct DeviceState {
+    std::atomic<int> ready{0};
+    int cus = 256;
+};
+DeviceState g_dev[kMaxDevices];
+std::mutex g_init_mutex;
+
+// Every kernel that needs more dynamic LDS than the default limit, or whose table addressing
+// assumes that its dynamic LDS starts at LDS address 0 (true exactly when the kernel has no
+// static LDS, which dmm_init verifies from the function's attributes).
+struct KernelInfo {
+    const void *fn;
+    int dynamic_lds;   // bytes to allow; 0 = default limit is enough
+    bool lds_base0;
+};
+
+template <typename... KArgs>
+KernelInfo kinfo(void (*k)(KArgs...), int lds, bool base0) { return KernelInfo{reinterpret_cast<const void *>(k), lds, base0}; }
+
+const std::vector<KernelInfo> &kernel_table()
+{
+    static const std::vector<KernelInfo> t = {
+#define DMM_BOTH_LAYOUTS(X) X(false), X(true)
+#define DMM_K_STREAM(P) kinfo(gemv_stream_kernel<1, 16, 2, P, 4>, kLdsMax, true), kinfo(gemv_stream_kernel<1, 16, 2, P, 1>, kLdsMax, true)
+        DMM_BOTH_LAYOUTS(DMM_K_STREAM),
+#define DMM_K_Q8(P)                                                                                          \
+    kinfo(gemv_q8_kernel<1, 16, 2, P, true>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 2, P, false>, kLdsMax, true), \
+        kinfo(gemv_q8_kernel<1, 16, 3, P, true>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P, false>, kLdsMax, true)
+        DMM_BOTH_LAYOUTS(DMM_K_Q8),
+#define DMM_K_REGX(P)                                                                                        \
+    kinfo(gemv_regx_kernel<1, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 1, 2, P>, kLdsMax, true),     \
+        kinfo(gemv_regx_kernel<3, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 1, 2, P>, kLdsMax, true), \
+        kinfo(gemv_regx_kernel<1, 8, 2, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, 2, P>, kLdsMax, true)
+        DMM_BOTH_LAYOUTS(DMM_K_REGX),
+#define DMM_K_GREG(P)                                                                                        \
+    kinfo(gemm_reg_kernel<1, false, P>, gr_smem_bytes(1), true), kinfo(gemm_reg_kernel<2, false, P>, gr_smem_bytes(2), true), \
+        kinfo(gemm_reg_kernel<4, false, P>, gr_smem_bytes(4), true), kinfo(gemm_reg_kernel<1, true, P>, gr_smem_bytes(1), true), \
+        kinfo(gemm_reg_kernel<2, true, P>, gr_smem_bytes(2), true), kinfo(gemm_reg_kernel<4, true, P>, gr_smem_bytes(4), true)
+        DMM_BOTH_LAYOUTS(DMM_K_GREG),
+        kinfo(gemm_kernel<4, 2, 2, 2>, (int)sizeof(GemmCfg<4, 2, 2, 2>::Shared), false),
+#define DMM_K_I8X(T)                                                                                         \
+    kinfo(int8x_kernel<1, 8, 2, T>, kLdsMax, true), kinfo(int8x_kernel<2, 8, 2, T>, kLdsMax, true),                    \
+        kinfo(int8x_kernel<3, 8, 2, T>, kLdsMax, true), kinfo(int8x_kernel<4, 8, 2, T>, kLdsMax, true),                \
+        kinfo(int8g_kernel<T>, kI8gSmem, true)
+        DMM_BOTH_LAYOUTS(DMM_K_I8X),
+#undef DMM_K_I8X
+#undef DMM_K_GREG
+#undef DMM_K_REGX
+#undef DMM_K_Q8
+#undef DMM_K_STREAM
+#undef DMM_BOTH_LAYOUTS
+    };
+    return t;
+}
+
+// One-time set-up of a device (the current one must be `dev`): compute-unit count, dynamic-LDS
+// limits and the check that the table kernels have no static LDS.
+int init_current_device(int dev)
+{
+    DeviceState &ds = g_dev[dev];
+    if (ds.ready.load(std::memory_order_acquire)) return DMM_OK;
+    std::lock_guard<std::mutex> lock(g_init_mutex);
+    if (ds.ready.load(std::memory_order_acquire)) return DMM_OK;
+    int v = 0;
+    hipError_t e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return (int)e;
+    ds.cus = v > 0 ? v : 256;
+    for (const KernelInfo &k : kernel_table()) {
+        if (k.lds_base0) {
+            hipFuncAttributes attr;
+            e = hipFuncGetAttributes(&attr, k.fn);
+            if (e != hipSuccess) return (int)e;
+            if (attr.sharedSizeBytes != 0) return DMM_ERR_INTERNAL;
+        }
+        if (k.dynamic_lds > 0) {
+            e = hipFuncSetAttribute(k.fn, hipFuncAttributeMaxDynamicSharedMemorySize, k.dynamic_lds);
+            if (e != hipSuccess) return (int)e;
+        }
+    }
+    ds.ready.store(1, std::memory_order_release);
+    return DMM_OK;
+}
+
+// Called by every entry point that launches, after its argument checks.  A first call on a
+// device does the set-up unless the stream is being captured into a graph, where host-side
+// set-up has no business: such a caller runs dmm_init beforehand.
+int ensure_ready(hipStream_t stream, const DeviceState **out = nullptr)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return DMM_ERR_TOO_LARGE;
+    if (!g_dev[dev].ready.load(std::memory_order_acquire)) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (stream && hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+            return DMM_ERR_NOT_INITIALIZED;
+        if (int st = init_current_device(dev)) return st;
+    }
+    if (out) *out = &g_dev[dev];
+    return DMM_OK;
+}
+
+// compute units of the current device (after ensure_ready)
+int cu_count()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    return g_dev[dev].cus;
+}
 
 int check_common(const void *x, const void *codes, const void *grid, const void *y, int64_t M,
                  int64_t N, int64_t K)
@@ -2437,81 +2495,17 @@ bool gemm_ok(const void *x, const void *codes, const void *grid, const void *, i
            aligned(grid, 16) && M <= 65535LL * 128;
 }
 
-// Tuning override for experiments: DMM_GEMV_CFG="R,W,D" picks the kernel instance (rows per
-// block = 16 R, W waves, D prefetched steps per wave); unset or unknown -> the default choice.
-int gemv_cfg_override()
-{
-    static int cfg = -1;
-    if (cfg < 0) {
-        cfg = 0;
-        if (const char *e = getenv("DMM_GEMV_CFG")) {
-            int r = 0, w = 0, d = 0;
-            const int n = sscanf(e, "%d,%d,%d", &r, &w, &d);
-            if (n >= 2) cfg = r * 10000 + w * 100 + (n == 3 ? d : 0);
-        }
-    }
-    return cfg;
-}
-
-// State that depends on the device (CU count, per-function attributes) is kept per device
-// ordinal: a process may drive several GPUs, each through its own calls.
-constexpr int kMaxDevices = 64;
-
-inline int current_device()
-{
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
-    return dev;
-}
-
-int cu_count()
-{
-    static int n[kMaxDevices] = {};
-    const int dev = current_device();
-    if (n[dev] == 0) {
-        hipDeviceProp_t prop;
-        int v = 0;
-        if (hipGetDeviceProperties(&prop, dev) == hipSuccess) v = prop.multiProcessorCount;
-        n[dev] = v > 0 ? v : 256;
-    }
-    return n[dev];
-}
-
-// Allow `bytes` of dynamic LDS for a kernel, once per device (benign race: every thread sets
-// the same value).  Returns 0 or the hipError_t.
-template <typename Kern>
-int allow_dynamic_lds(Kern kernel, int bytes, bool (&done)[kMaxDevices])
-{
-    const int dev = current_device();
-    if (!done[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        if (e != hipSuccess) return (int)e;
-        done[dev] = true;
-    }
-    return 0;
-}
-
 template <int R, int W, int D, bool kPacked = false>
 int launch_gemv_stream(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                        int64_t N, int64_t K, hipStream_t stream)
 {
-#ifdef DMM_TRACE
-    const size_t shmem = 160 * 1024;
-#else
     const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)stream_x_bytes(M, K);
-#endif
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    if (M <= 4) {   // four pieces of x per LDS read
-        static bool attr_done[kMaxDevices] = {};
-        if (int e = allow_dynamic_lds(gemv_stream_kernel<R, W, D, kPacked, 4>, 160 * 1024, attr_done)) return e;
+    if (M <= 4)   // four pieces of x per LDS read
         return launch(gemv_stream_kernel<R, W, D, kPacked, 4>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                       (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N,
                       (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
-    }
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemv_stream_kernel<R, W, D, kPacked, 1>, 160 * 1024, attr_done)) return e;
     return launch(gemv_stream_kernel<R, W, D, kPacked, 1>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
@@ -2522,7 +2516,7 @@ int launch_gemv_stream(const void *x, const void *codes, const void *grid, float
 template <int R, int W>
 bool gemv_q8_ok(int64_t M, int64_t N, int64_t K)
 {
-    return M <= 4 && (int64_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + q8_x_bytes(M, K) <= 160 * 1024 &&
+    return M <= 4 && (int64_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + q8_x_bytes(M, K) <= kLdsMax &&
            N * (K >> 2) < (1LL << 31);
 }
 
@@ -2531,22 +2525,13 @@ int launch_gemv_q8(const void *x, const void *codes, const void *grid, float sca
                    int64_t N, int64_t K, hipStream_t stream)
 {
     // the 8-bit layout is the larger one, so the 16-bit kernel it may hand over to fits as well
-#ifdef DMM_TRACE
-    const size_t shmem = 160 * 1024;
-#else
     const size_t shmem = (size_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
-#endif
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    if (M == 1) {   // the B operands of a step in two LDS reads
-        static bool attr_done[kMaxDevices] = {};
-        if (int e = allow_dynamic_lds(gemv_q8_kernel<R, W, D, kPacked, true>, 160 * 1024, attr_done)) return e;
+    if (M == 1)   // the B operands of a step in two LDS reads
         return launch(gemv_q8_kernel<R, W, D, kPacked, true>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                       (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N,
                       (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
-    }
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemv_q8_kernel<R, W, D, kPacked, false>, 160 * 1024, attr_done)) return e;
     return launch(gemv_q8_kernel<R, W, D, kPacked, false>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
@@ -2555,7 +2540,7 @@ int launch_gemv_q8(const void *x, const void *codes, const void *grid, float sca
 template <int R, int W>
 bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
 {
-    return M <= 16 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + stream_x_bytes(M, K) <= 160 * 1024 &&
+    return M <= 16 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + stream_x_bytes(M, K) <= kLdsMax &&
            N * (K >> 2) < (1LL << 31);
 }
 
@@ -2564,8 +2549,6 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
                      int64_t N, int64_t K, hipStream_t stream)
 {
     const size_t shmem = (size_t)kSTablesBytes + 2 * W * R * MT * kWave * 16;
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemv_regx_kernel<R, W, MT, D, kPacked>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     return launch(gemv_regx_kernel<R, W, MT, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
@@ -2602,10 +2585,10 @@ int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale,
 }
 
 // The choice among the matrix-vector kernels.  Launches of more than three row tiles per
-// workgroup: the 8-bit kernel where it applies (13 % faster at seven tiles, 3 - 4 % at two to
-// three, slower at one - its prologue is the dearer one, a grid that does not fit fp8 costs it
-// a second table build, and the 16-bit kernel's y is the correctly rounded one).  Otherwise the 16-bit streaming kernel, one tile at a time (two at a
-// time is 6 - 10 % slower at K = 8192); the register-x kernel when x does not fit the LDS.
+// workgroup: the 8-bit kernel where it applies (its prologue is the dearer one, a grid that does
+// not fit fp8 costs it a second table build, and the 16-bit kernel's y is the correctly rounded
+// one).  Otherwise the 16-bit streaming kernel, one tile at a time; the register-x kernel when x
+// does not fit the LDS.
 enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
 
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
@@ -2618,9 +2601,7 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 
 // The register-x kernel for M <= 16 reads the x slice of a k step once per row block, so the row
 // block should be the workgroup's whole share of tiles when that is 1 .. 4 tiles, and otherwise
-// the size that needs the fewest blocks (measured at M = 8 / 16, kernel us, two tiles per block
-// -> this choice: 4096 -> 11008 9.1 / 12.0 -> 8.4 / 10.0 (three); 8192 -> 28672 31.6 / 42.7 ->
-// 26.5 / 33.1 (four, then three); 11008 -> 4096 10.9 / 15.2 -> 10.6 / 14.8 (one)).
+// the size that needs the fewest blocks.
 template <bool kPacked>
 int run_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                   int64_t N, int64_t K, hipStream_t stream)
@@ -2650,9 +2631,10 @@ int run_gemv_regx2(const void *x, const void *codes, const void *grid, float sca
 }
 
 template <bool kPacked>
-int run_gemv_auto(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                  int64_t N, int64_t K, hipStream_t stream)
+int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+             int64_t N, int64_t K, hipStream_t stream)
 {
+    if (M > 16) return run_gemv_regx2<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
     switch (pick_gemv(M, N, K)) {
         case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
@@ -2660,64 +2642,14 @@ int run_gemv_auto(const void *x, const void *codes, const void *grid, float scal
     }
 }
 
-int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-             int64_t N, int64_t K, hipStream_t stream)
-{
-    if (M > 16) return run_gemv_regx2<false>(x, codes, grid, scale, y, M, N, K, stream);
-#define DMM_STREAM_CASE(R, W, D)                                                                   \
-    case R * 10000 + W * 100 + D:                                                                  \
-        if (gemv_stream_ok<R, W>(M, N, K))                                                         \
-            return launch_gemv_stream<R, W, D>(x, codes, grid, scale, y, M, N, K, stream);         \
-        break;
-    switch (gemv_cfg_override()) {
-        DMM_STREAM_CASE(2, 8, 4)
-        DMM_STREAM_CASE(1, 16, 4)
-        DMM_STREAM_CASE(1, 16, 3)
-        DMM_STREAM_CASE(1, 16, 2)
-        DMM_STREAM_CASE(2, 16, 2)
-        DMM_STREAM_CASE(2, 16, 3)
-#define DMM_Q8_CASE(TAG, R, D)                                                                     \
-    case TAG * 10000 + 1600 + D:                                                                   \
-        if (gemv_q8_ok<R, 16>(M, N, K))                                                            \
-            return launch_gemv_q8<R, 16, D>(x, codes, grid, scale, y, M, N, K, stream);            \
-        break;
-        DMM_Q8_CASE(9, 1, 2)
-        DMM_Q8_CASE(9, 1, 3)
-        DMM_Q8_CASE(9, 1, 4)
-#undef DMM_Q8_CASE
-        case 20803: return launch_gemv_regx<2, 8, 1, 3>(x, codes, grid, scale, y, M, N, K, stream);
-        case 20802: return launch_gemv_regx<2, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
-        case 10802: return launch_gemv_regx<1, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
-        case 40802: return launch_gemv_regx<4, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
-        case 30802: return launch_gemv_regx<3, 8, 1, 2>(x, codes, grid, scale, y, M, N, K, stream);
-        default: break;
-    }
-#undef DMM_STREAM_CASE
-    return run_gemv_auto<false>(x, codes, grid, scale, y, M, N, K, stream);
-}
-
-template <int WN, int WM, int TN, int TM>
-int launch_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                int64_t N, int64_t K, hipStream_t stream)
-{
-    typedef GemmCfg<WN, WM, TN, TM> C;
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemm_kernel<WN, WM, TN, TM>, (int)sizeof(typename C::Shared), attr_done)) return e;
-    dim3 g((unsigned)((N + C::kBN - 1) / C::kBN), (unsigned)((M + C::kBM - 1) / C::kBM));
-    return launch(gemm_kernel<WN, WM, TN, TM>, g, dim3(C::kThreads), sizeof(typename C::Shared), stream,
-                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K);
-}
-
 template <int TM, bool kSplit, bool kPacked>
 int launch_gemm_reg_tm(const void *x, const void *codes, const void *grid, float scale, void *y, float *part,
                        int64_t M, int64_t N, int64_t K, int splits, hipStream_t stream)
 {
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(gemm_reg_kernel<TM, kSplit, kPacked>, gr_smem_bytes(TM), attr_done)) return e;
     dim3 g((unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)((N + kGrBN - 1) / kGrBN), (unsigned)splits);
     return launch<true, !kSplit>(gemm_reg_kernel<TM, kSplit, kPacked>, g, dim3(256), gr_smem_bytes(TM), stream,
                                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, part, (int)M,
-                                 (int)N, (int)K, splits);
+                                 (int)N, (int)K, splits, aligned(y, 8) ? 1 : 0);
 }
 
 // rows of x per block: 32, 64 or 128
@@ -2737,11 +2669,11 @@ int launch_gemm_reg(const void *x, const void *codes, const void *grid, float sc
 // How many ways to split K so that the blocks about fill the chip: as many as fit the CU count
 // without starting a second round, each with at least 4 k tiles, and no more than the
 // workspace holds partial sums for.  1 = no split.
-int splitk_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes)
+int splitk_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, int cus)
 {
     const int tm = gemm_reg_tm(M);
     const int64_t tiles = ((M + 32 * tm - 1) / (32 * tm)) * ((N + kGrBN - 1) / kGrBN);
-    int64_t splits = cu_count() / tiles;
+    int64_t splits = cus / tiles;
     const int64_t k_tiles = K / kGrBK;
     if (splits > k_tiles / 4) splits = k_tiles / 4;
     if (splits > 64) splits = 64;
@@ -2775,41 +2707,25 @@ bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
 }
 
 // Smallest M that takes the split-K path when a workspace is given (up to M = 16 the
-// matrix-vector kernels are as fast or faster).  DMM_SPLITK_MIN_M overrides for experiments.
-int splitk_min_m()
-{
-    static int v = -1;
-    if (v < 0) {
-        const char *e = getenv("DMM_SPLITK_MIN_M");
-        v = e ? atoi(e) : 17;
-        if (v < 1) v = 1;
-    }
-    return v;
-}
+// matrix-vector kernels are as fast or faster).
+constexpr int kSplitKMinM = 17;
 
 bool splitk_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
                int64_t K)
 {
-    return M >= splitk_min_m() && gemm_ok(x, codes, grid, y, M, N, K) && gemm_reg_ok(M, N, K) && aligned(y, 8);
+    return M >= kSplitKMinM && gemm_ok(x, codes, grid, y, M, N, K) && gemm_reg_ok(M, N, K) && aligned(y, 8);
 }
 
-// Tuning override for experiments: DMM_GEMM_CFG=a|b|g picks a tile configuration of the
-// LDS-staged kernel, r (the default where its offsets fit) the register-operand kernel.
+// The register-operand kernel where its offsets fit, else the LDS-staged one (256 x 128, 8 waves)
 int run_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
-    static int cfg = -1;
-    if (cfg < 0) {
-        const char *e = getenv("DMM_GEMM_CFG");
-        cfg = e ? e[0] : 0;
-    }
-    if ((cfg == 'r' || cfg == 0) && gemm_reg_ok(M, N, K)) return launch_gemm_reg(x, codes, grid, scale, y, M, N, K, stream);
-    switch (cfg) {
-        case 'b': return launch_gemm<2, 2, 4, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 256 x 128, 4 waves
-        case 'g': return launch_gemm<2, 2, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);   // 128 x 128, 4 waves, 2 per CU
-        default: break;
-    }
-    return launch_gemm<4, 2, 2, 2>(x, codes, grid, scale, y, M, N, K, stream);                 // 256 x 128, 8 waves
+    if (gemm_reg_ok(M, N, K)) return launch_gemm_reg(x, codes, grid, scale, y, M, N, K, stream);
+    typedef GemmCfg<4, 2, 2, 2> C;
+    dim3 g((unsigned)((N + C::kBN - 1) / C::kBN), (unsigned)((M + C::kBM - 1) / C::kBM));
+    return launch(gemm_kernel<4, 2, 2, 2>, g, dim3(C::kThreads), sizeof(typename C::Shared), stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  aligned(y, 8) ? 1 : 0);
 }
 
 // y = 0 when K == 0 (empty sum), any M, N.
@@ -2833,25 +2749,12 @@ int run_generic(const void *x, const void *codes, const void *grid, float scale,
                   (const uint16_t *)codes, grid, scale, (uint16_t *)y, M, N, K);
 }
 
-// DMM_INT8_MFMA=0 in the environment keeps the integer operator on the scalar kernel (for
-// comparisons)
-bool int8x_enabled()
-{
-    static const bool on = [] {
-        const char *e = getenv("DMM_INT8_MFMA");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
-
 template <int R, bool kTiled, bool kFirst, bool kLast>
 int launch_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
                  hipStream_t stream)
 {
     constexpr int W = 8, D = 2;
     const size_t shmem = (size_t)2 * kI8TableBytes + (R <= 2 ? 2 : 1) * W * R * kWave * 16;
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(int8x_kernel<R, W, D, kTiled>, 160 * 1024, attr_done)) return e;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     return launch<kFirst, kLast>(int8x_kernel<R, W, D, kTiled>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
@@ -2865,13 +2768,11 @@ int launch_int8x(const void *x, const void *codes, const void *cb, void *out, in
 // bytes at 3.5 TB/s per 16 rows of x; the cheaper estimate wins (M = 64 at 4096 x 4096: four
 // matrix-vector launches, 20 us; M = 256: one matrix-matrix launch, 47 us against 75).
 enum Int8Kind { kInt8Scalar, kInt8Gemv, kInt8Gemm };
-Int8Kind pick_int8(int64_t M, int64_t N, int64_t K)
+Int8Kind pick_int8(int64_t M, int64_t N, int64_t K, int cus)
 {
-    if (M < 1 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31) || K > (1 << 17) ||
-        !int8x_enabled())
+    if (M < 1 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31) || K > (1 << 17))
         return kInt8Scalar;
     if (M > 16 && M * K < (1LL << 31)) {
-        const int64_t cus = cu_count();
         const int64_t tiles = ((M + kI8gBM - 1) / kI8gBM) * ((N + kI8gBN - 1) / kI8gBN);
         const double t_gemm = 3.0 + (double)((tiles + cus - 1) / cus) * (double)K * 0.0115;
         const double t_gemv = (double)((M + 15) / 16) * (3.0 + (double)N * (double)(K >> 2) / 3.5e6);
@@ -2884,8 +2785,6 @@ template <bool kTiled>
 int launch_int8g(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
                  hipStream_t stream)
 {
-    static bool attr_done[kMaxDevices] = {};
-    if (int e = allow_dynamic_lds(int8g_kernel<kTiled>, kI8gSmem, attr_done)) return e;
     dim3 g((unsigned)((M + kI8gBM - 1) / kI8gBM), (unsigned)((N + kI8gBN - 1) / kI8gBN));
     return launch(int8g_kernel<kTiled>, g, dim3(512), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
                   (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
@@ -2913,24 +2812,35 @@ int run_int8x(const void *x, const void *codes, const void *cb, void *out, int64
 #undef DMM_I8X
 }
 
+// CU count for the pure queries (kernel names, workspace size), which must answer without a
+// device: the current device's if it has been set up, else the MI355X's 256
+int cu_count_or_default()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    return g_dev[dev].ready.load(std::memory_order_acquire) ? g_dev[dev].cus : 256;
+}
+
+// the operator's dispatch once the arguments are checked and the device is ready
+int dispatch_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M, int64_t N,
+                 int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K)) {
+        const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
+        if (splits >= 2) return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, s);
+    }
+    if (gemv_ok(x, codes, grid, y, M, N, K)) return run_gemv<false>(x, codes, grid, scale, y, M, N, K, s);
+    if (gemm_ok(x, codes, grid, y, M, N, K)) return run_gemm(x, codes, grid, scale, y, M, N, K, s);
+    return run_generic(x, codes, grid, scale, y, M, N, K, s);
+}
+
 }  // namespace dmm
 
 using namespace dmm;
 
 extern "C" {
 
-#ifdef DMM_TRACE
-int dmm_debug_set_trace(void *buf)
-{
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(dmm::dmm_trace_buf), &buf, sizeof(buf));
-}
-int dmm_debug_set_mode(int mode)
-{
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(dmm::dmm_exp_mode), &mode, sizeof(mode));
-}
-#endif
-
-int dmm_version(void) { return (0 << 16) | 1; }
+int dmm_version(void) { return (0 << 16) | 2; }
 
 const char *dmm_status_string(int status)
 {
@@ -2941,10 +2851,29 @@ const char *dmm_status_string(int status)
         case DMM_ERR_MISALIGNED: return "a pointer does not meet the required alignment";
         case DMM_ERR_TOO_LARGE: return "a dimension is too large for the launch";
         case DMM_ERR_UNSUPPORTED: return "this explicit path does not support the given shape or alignment";
+        case DMM_ERR_NOT_INITIALIZED:
+            return "first call on this device while its stream is being captured: call dmm_init before capturing";
+        case DMM_ERR_INTERNAL: return "a table kernel was built with static LDS (library build error)";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
     return "unknown status";
+}
+
+int dmm_init(int device)
+{
+    int cur = 0;
+    hipError_t e = hipGetDevice(&cur);
+    if (e != hipSuccess) return (int)e;
+    if (device < 0) device = cur;
+    if (device >= kMaxDevices) return DMM_ERR_TOO_LARGE;
+    if (device != cur) {
+        e = hipSetDevice(device);
+        if (e != hipSuccess) return (int)e;
+    }
+    const int st = init_current_device(device);
+    if (device != cur) (void)hipSetDevice(cur);
+    return st;
 }
 
 int dmm_set_kernel_events(void *start_event, void *stop_event)
@@ -2962,6 +2891,7 @@ int dmm_decode_f16(const void *codes, const void *grid, void *W, int64_t N, int6
     if (n_codes == 0) return DMM_OK;
     if (!codes || !grid || !W) return DMM_ERR_NULL_POINTER;
     if (!aligned(codes, 2) || !aligned(grid, 2) || !aligned(W, 2)) return DMM_ERR_MISALIGNED;
+    if (int st = ensure_ready((hipStream_t)stream)) return st;
     const bool wide = aligned(codes, 4) && aligned(grid, 16) && aligned(W, 16);
     const int64_t work = wide ? (n_codes + 1) / 2 : n_codes;
     int64_t blocks = (work + 255) / 256;
@@ -2978,6 +2908,7 @@ int dmm_generic_f16(const void *x, const void *codes, const void *grid, float sc
 {
     int st = check_common(x, codes, grid, y, M, N, K);
     if (st != DMM_OK || M == 0 || N == 0) return st;
+    if ((st = ensure_ready((hipStream_t)stream))) return st;
     return run_generic(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
 }
 
@@ -2987,7 +2918,8 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
     int st = check_common(x, codes, grid, y, M, N, K);
     if (st != DMM_OK || M == 0 || N == 0) return st;
     if (!gemv_ok(x, codes, grid, y, M, N, K)) return DMM_ERR_UNSUPPORTED;
-    return run_gemv(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
+    if ((st = ensure_ready((hipStream_t)stream))) return st;
+    return run_gemv<false>(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
 }
 
 int dmm_set_gemv_8bit(int enabled)
@@ -2999,7 +2931,7 @@ int dmm_set_gemv_8bit(int enabled)
 
 const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K)
 {
-    switch (pick_int8(M, N, K)) {
+    switch (pick_int8(M, N, K, cu_count_or_default())) {
         case kInt8Gemm: return "dmm::int8g_kernel";
         case kInt8Gemv: return "dmm::int8x_kernel";
         default: return "dmm::int8_kernel";
@@ -3023,6 +2955,7 @@ int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float 
     int st = check_common(x, codes, grid, y, M, N, K);
     if (st != DMM_OK || M == 0 || N == 0) return st;
     if (!gemv_ok(x, codes, grid, y, M, N, K) || !gemv_q8_ok<1, 16>(M, N, K)) return DMM_ERR_UNSUPPORTED;
+    if ((st = ensure_ready((hipStream_t)stream))) return st;
     return run_gemv_q8<false>(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
 }
 
@@ -3039,6 +2972,7 @@ int dmm_pack_codes(const void *codes, void *packed, int64_t N, int64_t K, void *
     if (N == 0) return DMM_OK;
     if (!codes || !packed) return DMM_ERR_NULL_POINTER;
     if (!aligned(codes, 16) || !aligned(packed, 16)) return DMM_ERR_MISALIGNED;
+    if (int st = ensure_ready((hipStream_t)stream)) return st;
     const int64_t pieces = dmm_packed_bytes(N, K) / 16;
     int64_t blocks = (pieces + 255) / 256;
     if (blocks > 65535 * 16) blocks = 65535 * 16;
@@ -3054,9 +2988,8 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
     // the matrix-vector kernels' domain, with the padded size in place of N * K / 4; same choice
     // of kernel as for row-major codes
     if (!gemv_ok(x, packed, grid, y, M, N, K) || dmm_packed_bytes(N, K) >= (1LL << 31)) return DMM_ERR_UNSUPPORTED;
-    hipStream_t s = (hipStream_t)stream;
-    if (M > 16) return run_gemv_regx2<true>(x, packed, grid, scale, y, M, N, K, s);
-    return run_gemv_auto<true>(x, packed, grid, scale, y, M, N, K, s);
+    if ((st = ensure_ready((hipStream_t)stream))) return st;
+    return run_gemv<true>(x, packed, grid, scale, y, M, N, K, (hipStream_t)stream);
 }
 
 int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *grid, float scale, void *y,
@@ -3071,14 +3004,15 @@ int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *
     if (pbytes == 0 || pbytes >= (1LL << 31)) return DMM_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     const bool mm_ok = gemm_ok(x, packed, grid, y, M, N, K) && gemm_reg_ok(M, ((N + 15) / 16) * 16, K);
-    if (workspace && workspace_bytes > 0 && mm_ok && M >= splitk_min_m() && aligned(y, 8)) {
-        const int splits = splitk_plan(M, N, K, workspace_bytes);
+    const bool mv_ok = gemv_ok(x, packed, grid, y, M, N, K);
+    if (!mm_ok && !mv_ok) return DMM_ERR_UNSUPPORTED;
+    if ((st = ensure_ready(s))) return st;
+    if (workspace && workspace_bytes > 0 && mm_ok && M >= kSplitKMinM && aligned(y, 8)) {
+        const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
         if (splits >= 2) return launch_gemm_splitk<true>(x, packed, grid, scale, y, workspace, splits, M, N, K, s);
     }
-    if (gemv_ok(x, packed, grid, y, M, N, K))
-        return dmm_gemv_packed_f16(x, packed, grid, scale, y, M, N, K, stream);
-    if (mm_ok) return launch_gemm_reg<true>(x, packed, grid, scale, y, M, N, K, s);
-    return DMM_ERR_UNSUPPORTED;
+    if (mv_ok) return run_gemv<true>(x, packed, grid, scale, y, M, N, K, s);
+    return launch_gemm_reg<true>(x, packed, grid, scale, y, M, N, K, s);
 }
 
 int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
@@ -3087,6 +3021,7 @@ int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale
     int st = check_common(x, codes, grid, y, M, N, K);
     if (st != DMM_OK || M == 0 || N == 0) return st;
     if (!gemm_ok(x, codes, grid, y, M, N, K)) return DMM_ERR_UNSUPPORTED;
+    if ((st = ensure_ready((hipStream_t)stream))) return st;
     return run_gemm(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
 }
 
@@ -3099,6 +3034,7 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
     if (!out || !codebook_abs) return DMM_ERR_NULL_POINTER;
     if (K > 0 && (!x || !codes)) return DMM_ERR_NULL_POINTER;
     if (!aligned(codes, 2) || !aligned(codebook_abs, 8) || !aligned(out, 4)) return DMM_ERR_MISALIGNED;
+    if (int st = ensure_ready((hipStream_t)stream)) return st;
     if (K == 0) {
         const int64_t n = M * N;
         const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
@@ -3106,7 +3042,8 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
     }
     // the matrix-unit kernels (K <= 2^17: their weights are odd, so |w| <= 127 and no sum of K
     // products leaves int32 - nothing depends on what the matrix unit does on overflow)
-    const Int8Kind kind = aligned(x, 16) && aligned(codes, 16) && aligned(out, 16) ? pick_int8(M, N, K) : kInt8Scalar;
+    const Int8Kind kind =
+        aligned(x, 16) && aligned(codes, 16) && aligned(out, 16) ? pick_int8(M, N, K, cu_count()) : kInt8Scalar;
     if (kind == kInt8Gemm)
         return tiled ? launch_int8g<true>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream)
                      : launch_int8g<false>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream);
@@ -3130,9 +3067,9 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
 
 int64_t dmm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 {
-    if (M < 1 || N < 1 || K < kGrBK || (K & 63) || M < splitk_min_m() || M > 65535LL * 128 || !gemm_reg_ok(M, N, K))
+    if (M < 1 || N < 1 || K < kGrBK || (K & 63) || M < kSplitKMinM || M > 65535LL * 128 || !gemm_reg_ok(M, N, K))
         return 0;
-    const int splits = splitk_plan(M, N, K, INT64_MAX);
+    const int splits = splitk_plan(M, N, K, INT64_MAX, cu_count_or_default());
     return splits >= 2 ? (int64_t)splits * M * N * 4 : 0;
 }
 
@@ -3144,12 +3081,8 @@ int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid,
     if (st != DMM_OK || M == 0 || N == 0) return st;
     if (workspace_bytes < 0) return DMM_ERR_BAD_SHAPE;
     if (workspace && workspace_bytes > 0 && !aligned(workspace, 16)) return DMM_ERR_MISALIGNED;
-    if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K)) {
-        const int splits = splitk_plan(M, N, K, workspace_bytes);
-        if (splits >= 2)
-            return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, (hipStream_t)stream);
-    }
-    return dmm_decode_matmul_f16(x, codes, grid, scale, y, M, N, K, stream);
+    if ((st = ensure_ready((hipStream_t)stream))) return st;
+    return dispatch_f16(x, codes, grid, scale, y, M, N, K, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, float scale, void *y,
@@ -3157,10 +3090,8 @@ int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, fl
 {
     int st = check_common(x, codes, grid, y, M, N, K);
     if (st != DMM_OK || M == 0 || N == 0) return st;
-    hipStream_t s = (hipStream_t)stream;
-    if (gemv_ok(x, codes, grid, y, M, N, K)) return run_gemv(x, codes, grid, scale, y, M, N, K, s);
-    if (gemm_ok(x, codes, grid, y, M, N, K)) return run_gemm(x, codes, grid, scale, y, M, N, K, s);
-    return run_generic(x, codes, grid, scale, y, M, N, K, s);
+    if ((st = ensure_ready((hipStream_t)stream))) return st;
+    return dispatch_f16(x, codes, grid, scale, y, M, N, K, nullptr, 0, (hipStream_t)stream);
 }
 
 }  // extern "C"

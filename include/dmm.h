@@ -7,6 +7,13 @@
  * synchronises the device and never terminates the process: every entry point enqueues
  * its kernels on the caller's stream and returns a status code.
  *
+ * Host work outside the launches happens once per device, in dmm_init: the compute-unit
+ * count is read and the kernels' dynamic-LDS limits are raised (hipFuncSetAttribute).  An entry point called on a device that has not
+ * been initialised does this itself first - except when its stream is being captured into
+ * a HIP graph, where it returns DMM_ERR_NOT_INITIALIZED instead: call dmm_init (or make one
+ * eager call) before capturing.  After that every entry point only enqueues kernels and
+ * can be captured.
+ *
  * Code format (one 16-bit code per 8 consecutive weights along K), as defined by
  * /root/reference/test_decode_matmul.py:29-55 and
  * /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:45-65:
@@ -33,7 +40,10 @@ enum {
                                    shape constraint of the entry point is violated      */
     DMM_ERR_MISALIGNED = -3,    /* a pointer misses the alignment the entry point asks  */
     DMM_ERR_TOO_LARGE = -4,     /* a dimension exceeds what the launch can index        */
-    DMM_ERR_UNSUPPORTED = -5    /* explicit-path entry point called outside its domain  */
+    DMM_ERR_UNSUPPORTED = -5,   /* explicit-path entry point called outside its domain  */
+    DMM_ERR_NOT_INITIALIZED = -6, /* first call on a device made under stream capture     */
+    DMM_ERR_INTERNAL = -7       /* the library was built wrongly (a table kernel has
+                                   static LDS); no kernel was launched                  */
 };
 
 /* Library version, (major << 16) | minor. */
@@ -41,6 +51,12 @@ int dmm_version(void);
 
 /* Human-readable text for a status code returned by this library (static storage). */
 const char *dmm_status_string(int status);
+
+/* One-time set-up of a device (device < 0: the current one); see the note on host work
+ * above.  Idempotent and thread-safe; restores the current device before it returns.  The
+ * reference does the corresponding host work on every call
+ * (cudaGetDeviceProperties, /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:217-218). */
+int dmm_init(int device);
 
 /* Standalone decoder: codes [N, K/8] row-major -> W half [N, K] row-major.
  * Replaces the decode half of the fused reference kernel
@@ -173,7 +189,7 @@ int dmm_gemv_packed_f16(const void *x, const void *packed, const void *grid, flo
  * launch of a matrix-vector kernel, or one launch of a matrix-matrix kernel when x has many rows
  * (a table with a byte that is not 2 mod 4 - the E8P table has none - is noticed inside
  * the launch and served by the scalar decode); anything else takes the scalar kernel, one wave
- * per output row.  DMM_INT8_MFMA=0 in the environment keeps every call on the scalar kernel. */
+ * per output row. */
 int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_abs, void *out,
                          int64_t M, int64_t N, int64_t K, int tiled, void *stream);
 

@@ -475,7 +475,8 @@ def test_integer_operator_golden_cases_and_edges():
 
 # ----------------------------------------------------------------- full benchmark sizes
 FULL = [(1, N, K) for (K, N) in workload.LLAMA2_70B + workload.LLAMA2_7B] + \
-       [(16, 11008, 4096), (32, 4096, 11008), (2048, 4096, 4096), (2048, 11008, 4096), (2048, 4096, 11008)]
+       [(M, N, K) for M in (4, 8, 16, 32) for (K, N) in workload.SMALL_BATCH] + \
+       [(2048, 4096, 4096), (2048, 11008, 4096), (2048, 4096, 11008)]
 
 
 @pytest.mark.parametrize("M,N,K", FULL)
@@ -497,6 +498,39 @@ def test_full_size_against_decode_then_fp32_matmul(M, N, K):
     y2 = c_matmul(xd * 2, cd, gd, scale, "auto")
     torch.cuda.synchronize()
     assert torch.allclose(y2.float(), 2 * y.float(), rtol=2e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("K,N", workload.SMALL_BATCH)
+def test_full_size_m32_through_the_workspace_entry(K, N):
+    """M = 32 at the small-batch shapes the way the benchmark calls them: through
+    dmm_decode_matmul_ws_f16 with the workspace dmm_workspace_bytes asks for (split-K)."""
+    M = 32
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=0)
+    xd, cd, gd = dev(x), dev(codes), dev(grid)
+    y, want = c_matmul_ws(xd, cd, gd, scale)
+    assert want > 0, "this shape is meant to split"
+    W = c_decode(cd, gd)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(W), bits(orc.decode_f16(codes.numpy(), grid.numpy())))
+    ref = (xd.float() @ W.float().T) * scale
+    assert_close_to_oracle(y, ref.cpu().numpy(), "full, workspace, M=32 N=%d K=%d" % (N, K))
+
+
+@pytest.mark.parametrize("M,N,K", [(40, 256, 512), (130, 260, 1024), (33, 64, 64)])
+def test_matrix_matrix_with_y_only_2_byte_aligned(M, N, K):
+    """x, codes and grid 16-byte aligned (so the register-operand MFMA kernel runs), y at an odd
+    2-byte offset: the kernel must fall back to 2-byte stores and stay inside y."""
+    x, codes, grid, scale = workload.make_inputs(M, N, K, seed=M)
+    ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+    buf = torch.full((M * N + 64,), -7.0, dtype=torch.float16, device=DEV)
+    y = buf[17:17 + M * N].view(M, N)
+    assert y.data_ptr() % 8 == 2
+    for path in ("gemm", "auto"):
+        buf.fill_(-7.0)
+        c_matmul(dev(x), dev(codes), dev(grid), scale, path, out=y)
+        torch.cuda.synchronize()
+        assert_close_to_oracle(y, ref, "y misaligned, %s" % path)
+        assert torch.all(buf[:17] == -7.0) and torch.all(buf[17 + M * N:] == -7.0)
 
 
 # ----------------------------------------------------------------- small-batch kernel, row blocks
@@ -788,7 +822,7 @@ def test_graph_capture_and_replay():
             c_matmul(xd, cd, gd, scale, "auto", out=y)
         c_decode(probs[0][1], probs[0][2], out=W)
 
-    step()                                   # warm-up outside the capture (kernel attributes are set here)
+    assert capi.lib().dmm_init(-1) == 0     # the once-per-device host work, outside the capture
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
@@ -808,6 +842,30 @@ def test_graph_capture_and_replay():
         want = [p[4] for p in probs] + [W]
         for g, w in zip(got, want):
             assert torch.equal(g, w), rep
+
+
+def test_reference_call_under_the_reference_name():
+    """`decode_matmul(x int8, weights_compressed int16 tiled, codebook_abs int64) -> int32`, the
+    reference's three-argument call (test_decode_matmul.py:136), works under the reference's
+    function name, also through a module alias as `from decode_matmul_cuda import decode_matmul`."""
+    import sys
+    M, N, K = 8, 16, 4096                        # the reference's own test shape
+    rng = np.random.default_rng(5)
+    x = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8), dtype=np.int16)
+    cb = orc.build_codebook_abs()
+    want = orc.decode_matmul_i32(x, codes, cb)
+    sys.modules.setdefault("decode_matmul_cuda", dmm)
+    from decode_matmul_cuda import decode_matmul
+    tiled = dmm.transpose_tile(torch.from_numpy(codes))
+    out = decode_matmul(dev(torch.from_numpy(x)), dev(tiled), dev(torch.from_numpy(cb)))
+    torch.cuda.synchronize()
+    assert out.dtype == torch.int32 and np.array_equal(out.cpu().numpy(), want)
+    with pytest.raises(TypeError):
+        decode_matmul(dev(torch.from_numpy(x)), dev(tiled), dev(torch.from_numpy(cb)), 0.5)
+    xh, ch, gh, scale = workload.make_inputs(1, 64, 512, seed=9)
+    with pytest.raises(TypeError):
+        decode_matmul(dev(xh), dev(ch), dev(gh))     # the half-precision form needs its scale
 
 
 def test_kernel_event_hook_times_the_kernel():
