@@ -15,6 +15,8 @@ SYMBOLS = {
     "dmm_version": (ctypes.c_int, []),
     "dmm_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "dmm_init": (ctypes.c_int, [ctypes.c_int]),
+    "dmm_noalloc_scratch_bytes": (ctypes.c_int64, []),
+    "dmm_decode_matmul_noalloc_f16": (ctypes.c_int, _OP),
     "dmm_decode_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "dmm_decode_matmul_f16": (ctypes.c_int, _OP),
     "dmm_gemv_f16": (ctypes.c_int, _OP),

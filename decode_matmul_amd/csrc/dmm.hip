@@ -2330,6 +2330,13 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ 
     }
 }
 
+// ------------------------------------------------------------------ scratch memory of the library
+// The one buffer the library owns: split-K partial sums for dmm_decode_matmul_noalloc_f16, whose
+// callers cannot allocate.  In host code the array's name is a stand-in, not a device address;
+// dmm_init asks the runtime for the address once per device and the launches pass that.
+constexpr int64_t kScratchBytes = 16ll << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
 // ------------------------------------------------------------------ host side
 thread_local hipEvent_t tls_start = nullptr;
 thread_local hipEvent_t tls_stop = nullptr;
@@ -2361,6 +2368,7 @@ constexpr int kLdsMax = 160 * 1024;
 struct DeviceState {
     std::atomic<int> ready{0};
     int cus = 256;
+    void *scratch = nullptr;   // this device's copy of `scratch`
 };
 DeviceState g_dev[kMaxDevices];
 std::mutex g_init_mutex;
@@ -2414,7 +2422,7 @@ const std::vector<KernelInfo> &kernel_table()
 }
 
 // One-time set-up of a device (the current one must be `dev`): compute-unit count, dynamic-LDS
-// limits and the check that the table kernels have no static LDS.
+// limits, the check that the table kernels have no static LDS, and the address of `scratch`.
 int init_current_device(int dev)
 {
     DeviceState &ds = g_dev[dev];
@@ -2437,6 +2445,10 @@ int init_current_device(int dev)
             if (e != hipSuccess) return (int)e;
         }
     }
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    ds.scratch = p;
     ds.ready.store(1, std::memory_order_release);
     return DMM_OK;
 }
@@ -2854,6 +2866,9 @@ const char *dmm_status_string(int status)
         case DMM_ERR_NOT_INITIALIZED:
             return "first call on this device while its stream is being captured: call dmm_init before capturing";
         case DMM_ERR_INTERNAL: return "a table kernel was built with static LDS (library build error)";
+        case DMM_ERR_SCRATCH_TOO_SMALL:
+            return "the split-K partial sums of this shape exceed the library's 16 MiB scratch buffer: use "
+                   "dmm_decode_matmul_ws_f16 with a workspace of dmm_workspace_bytes, or dmm_decode_matmul_f16";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -3083,6 +3098,21 @@ int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid,
     if (workspace && workspace_bytes > 0 && !aligned(workspace, 16)) return DMM_ERR_MISALIGNED;
     if ((st = ensure_ready((hipStream_t)stream))) return st;
     return dispatch_f16(x, codes, grid, scale, y, M, N, K, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int64_t dmm_noalloc_scratch_bytes(void) { return kScratchBytes; }
+
+int dmm_decode_matmul_noalloc_f16(const void *x, const void *codes, const void *grid, float scale, void *y,
+                                  int64_t M, int64_t N, int64_t K, void *stream)
+{
+    int st = check_common(x, codes, grid, y, M, N, K);
+    if (st != DMM_OK || M == 0 || N == 0) return st;
+    // what dmm_decode_matmul_ws_f16 would like as a workspace must fit the library's buffer
+    const int64_t want = splitk_ok(x, codes, grid, y, M, N, K) ? dmm_workspace_bytes(M, N, K) : 0;
+    if (want > kScratchBytes) return DMM_ERR_SCRATCH_TOO_SMALL;
+    const DeviceState *ds = nullptr;
+    if ((st = ensure_ready((hipStream_t)stream, &ds))) return st;
+    return dispatch_f16(x, codes, grid, scale, y, M, N, K, want > 0 ? ds->scratch : nullptr, want, (hipStream_t)stream);
 }
 
 int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, float scale, void *y,

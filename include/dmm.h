@@ -8,7 +8,8 @@
  * its kernels on the caller's stream and returns a status code.
  *
  * Host work outside the launches happens once per device, in dmm_init: the compute-unit
- * count is read and the kernels' dynamic-LDS limits are raised (hipFuncSetAttribute).  An entry point called on a device that has not
+ * count is read, the kernels' dynamic-LDS limits are raised (hipFuncSetAttribute) and the
+ * library's one device buffer is located.  An entry point called on a device that has not
  * been initialised does this itself first - except when its stream is being captured into
  * a HIP graph, where it returns DMM_ERR_NOT_INITIALIZED instead: call dmm_init (or make one
  * eager call) before capturing.  After that every entry point only enqueues kernels and
@@ -42,8 +43,10 @@ enum {
     DMM_ERR_TOO_LARGE = -4,     /* a dimension exceeds what the launch can index        */
     DMM_ERR_UNSUPPORTED = -5,   /* explicit-path entry point called outside its domain  */
     DMM_ERR_NOT_INITIALIZED = -6, /* first call on a device made under stream capture     */
-    DMM_ERR_INTERNAL = -7       /* the library was built wrongly (a table kernel has
+    DMM_ERR_INTERNAL = -7,      /* the library was built wrongly (a table kernel has
                                    static LDS); no kernel was launched                  */
+    DMM_ERR_SCRATCH_TOO_SMALL = -8 /* dmm_decode_matmul_noalloc_f16: the shape's partial
+                                   sums exceed the library's scratch buffer             */
 };
 
 /* Library version, (major << 16) | minor. */
@@ -96,6 +99,21 @@ int64_t dmm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid, float scale,
                              void *y, int64_t M, int64_t N, int64_t K, void *workspace,
                              int64_t workspace_bytes, void *stream);
+
+/* The operator for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same result as dmm_decode_matmul_ws_f16 with a workspace of dmm_workspace_bytes(M, N, K),
+ * bit for bit, but the split-K partial sums go to a buffer inside the library: a 16 MiB
+ * static device array (dmm_noalloc_scratch_bytes), one copy per GPU the library runs on,
+ * held until the process ends.  The call allocates nothing and frees nothing.  A shape whose
+ * preferred workspace exceeds the buffer is rejected with DMM_ERR_SCRATCH_TOO_SMALL (nothing is
+ * launched); shapes that use no workspace (M <= 16, or too few k tiles to split) run exactly
+ * as dmm_decode_matmul_f16.  Every partial sum is written before it is read, so the buffer
+ * needs no clearing between calls; but all calls on one GPU share it: two such calls that
+ * may overlap (different streams, or graphs replayed concurrently) race. */
+int64_t dmm_noalloc_scratch_bytes(void);
+int dmm_decode_matmul_noalloc_f16(const void *x, const void *codes, const void *grid, float scale,
+                                  void *y, int64_t M, int64_t N, int64_t K, void *stream);
 
 /* Explicit paths of the operator, for tests and measurement.  Same arguments.  Each
  * returns DMM_ERR_UNSUPPORTED outside its domain instead of falling back:
