@@ -33,6 +33,10 @@ MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 # dispatch (32,156,331 code bytes); gemv_q8_kernel (8192 -> 28672): 28,829.0 KiB and 56.7 KiB
 # (58,720,256 code bytes).
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_stream_kernel": 32565000, "dmm::gemv_q8_kernel": 59095000}
+GEMV_TRAFFIC_SOURCE = {"dmm::gemv_stream_kernel": "profiles/gemv_stream_kernel_llama70b_batch1.md (rocprofv3 --pmc, an earlier run; "
+                                                  "not measured by this run)",
+                       "dmm::gemv_q8_kernel": "profiles/gemv_q8_kernel_llama70b_batch1.md (rocprofv3 --pmc, an earlier run; not "
+                                              "measured by this run)"}
 
 
 def parse():
@@ -40,6 +44,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="how many times the region of exactly --steps steps is timed; the median region is reported")
     ap.add_argument("--quick", action="store_true", help="skip prefill / small-batch / CPU legs")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
     ap.add_argument("--graph-steps", type=int, default=12,
@@ -115,6 +121,9 @@ def main():
         probs.append(dict(K=K, N=N, x=x.to(dev), grid=grid.to(dev), scale=scale,
                           codes=rand_codes(N, K, copies, 100 + i),
                           y=torch.empty(1, N, dtype=torch.float16, device=dev)))
+    st = lib.dmm_init(-1)                # the once-per-device host work, before anything is captured
+    if st != 0:
+        raise capi.DmmError("dmm_init", st)
 
     def step(i):
         for p in probs:
@@ -126,52 +135,66 @@ def main():
     # layers of these four projections at this size), not one of four: with a graph per step the
     # GPU sat idle for about 15 us between replays, a fifth of the step, and with four ctypes
     # calls per 56 us step the eager loop sits close to being bound by the host.
-    def run_steps(n):
-        for i in range(n):
-            step(i)
-    launch_mode = "eager"
-    if not args.no_graph:
-        try:
-            for i in range(copies):
-                step(i)                      # kernel attributes are set outside the capture
+    def timed_steps(tag):
+        """Wall time of exactly args.steps steps, `--repeats` times over (each region bracketed by
+        synchronisation; the median region is reported), with the kernel choice as it stands."""
+        def run_steps(n):
+            for i in range(n):
+                step(i)
+        mode = "eager"
+        if not args.no_graph:
+            try:
+                chunk = max(copies, args.graph_steps // copies * copies)   # whole turns of the buffer sets
+                graphs = {}
+
+                def graph_of(n):                 # n consecutive steps, starting on buffer set 0
+                    if n not in graphs:
+                        g = torch.cuda.CUDAGraph()
+                        with torch.cuda.graph(g):
+                            cap = torch.cuda.current_stream().cuda_stream
+                            for i in range(n):
+                                for p in probs:
+                                    st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][i % copies].data_ptr(),
+                                                                   p["grid"].data_ptr(), p["scale"], p["y"].data_ptr(),
+                                                                   1, p["N"], p["K"], cap)
+                                    if st != 0:
+                                        raise capi.DmmError("dmm_decode_matmul_f16", st)
+                        graphs[n] = g
+                    return graphs[n]
+
+                for n in {chunk, args.steps % chunk, args.warmup % chunk} - {0}:
+                    graph_of(n)
+
+                def run_steps(n):                # exactly n steps: whole chunks, then the rest
+                    for _ in range(n // chunk):
+                        graphs[chunk].replay()
+                    if n % chunk:
+                        graphs[n % chunk].replay()
+                mode = "hip graph, %d steps (%d launches) per replay" % (chunk, chunk * len(probs))
+            except Exception as e:   # capture unavailable: time the eager loop
+                print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
+        run_steps(args.warmup)
+        torch.cuda.synchronize()
+        regions = []
+        for _ in range(max(1, args.repeats)):
+            t0 = time.perf_counter()
+            run_steps(args.steps)
             torch.cuda.synchronize()
-            chunk = max(copies, args.graph_steps // copies * copies)   # whole turns of the buffer sets
-            graphs = {}
+            regions.append(time.perf_counter() - t0)
+        return sorted(regions)[len(regions) // 2], regions, mode
 
-            def graph_of(n):                 # n consecutive steps, starting on buffer set 0
-                if n not in graphs:
-                    g = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(g):
-                        cap = torch.cuda.current_stream().cuda_stream
-                        for i in range(n):
-                            for p in probs:
-                                st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][i % copies].data_ptr(),
-                                                               p["grid"].data_ptr(), p["scale"], p["y"].data_ptr(),
-                                                               1, p["N"], p["K"], cap)
-                                if st != 0:
-                                    raise capi.DmmError("dmm_decode_matmul_f16", st)
-                    graphs[n] = g
-                return graphs[n]
-
-            for n in {chunk, args.steps % chunk, args.warmup % chunk} - {0}:
-                graph_of(n)
-
-            def run_steps(n):                # exactly n steps: whole chunks, then the rest
-                for _ in range(n // chunk):
-                    graphs[chunk].replay()
-                if n % chunk:
-                    graphs[n % chunk].replay()
-            launch_mode = "hip graph, %d steps (%d launches) per replay" % (chunk, chunk * len(probs))
-        except Exception as e:   # capture unavailable: time the eager loop
-            print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
-    run_steps(args.warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_steps(args.steps)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    wall, regions, launch_mode = timed_steps("operator's choice")
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes * args.steps / wall / 1e9
+    # the same steps with the 8-bit kernels switched off: every launch in 16-bit arithmetic (half x half
+    # products, fp32 sums), the arithmetic the operator's definition states
+    was = lib.dmm_set_gemv_8bit(0)
+    try:
+        wall16, _, _ = timed_steps("16-bit kernels only")
+        names16 = sorted({lib.dmm_gemv_kernel_name(1, N, K).decode() for K, N in shapes})
+    finally:
+        lib.dmm_set_gemv_8bit(was)
+    value_f16_only = step_bytes * args.steps / wall16 / 1e9
 
     # same region again with the kernel's own begin/end events
     n_launch = args.steps * len(probs)
@@ -225,6 +248,14 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
+        "dtype_note": "x, grid, y and the decoded weights are halves, sums fp32; launches of three or more row tiles "
+                      "per compute unit multiply fp8 weights (exact for this grid) by x split into four bf8 terms "
+                      "(exact) on the 8-bit matrix unit; value_f16_only is the same step with every launch on "
+                      "half x half products",
+        "value_f16_only": round(value_f16_only, 2),
+        "ms_per_step_f16_only": round(wall16 * 1e3 / args.steps, 5),
+        "kernels_f16_only": names16,
+        "timed_regions_ms": [round(r * 1e3, 4) for r in regions],
         "data": "synthetic",
         "config": {"workload": "configs[2]: batch-1 decode-GEMV, 8192->10240, 8192->8192, 8192->28672, 28672->8192",
                    "M": 1, "code_buffers_rotated": copies, "distinct_code_MB": round(copies * step_bytes / 1e6, 1),
@@ -232,6 +263,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+                     "traffic_source": GEMV_TRAFFIC_SOURCE.get(dom),
                      "kernel": dom, "launches": kd["launches"],
                      "avg_launch_us": round(kd["seconds"] / kd["launches"] * 1e6, 3),
                      "algorithmic_bytes_per_launch": kd["bytes"] / kd["launches"]},
@@ -245,7 +277,9 @@ def main():
     }
 
     if not args.quick:
+        out["hbm_read_probe"] = hbm_read_probe(torch, lib, probs, copies, stream, args.steps)
         out["gemv_packed"] = gemv_packed(torch, lib, capi, workload, probs, copies, stream, args.steps)
+        out["gemv_7b_step"] = gemv_7b_step(torch, lib, capi, workload, dev, rand_codes)
         out["gemv_7b_shapes"] = gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes)
         out["small_batch"] = small_batch(torch, lib, capi, workload, dev, stream, rand_codes)
         out["integer_operator"] = integer_operator(torch, lib, capi, workload, dev, stream, rand_codes)
@@ -269,6 +303,86 @@ def timed_kernel(torch, lib, fn, reps):
     torch.cuda.synchronize()
     t = [a.elapsed_time(b) * 1e-3 for a, b in ev]
     return sum(t) / len(t)
+
+
+def hbm_read_probe(torch, lib, probs, copies, stream, steps):
+    """What a kernel that only reads gets out of the memory system at the headline shapes: the
+    library's read probe (same launch shape and access pattern as the batch-1 kernels, no decode)
+    over the same rotating code buffers, the four shapes taking turns, durations by events."""
+    sink = torch.zeros(16, dtype=torch.int32, device=probs[0]["x"].device)
+
+    def fn(k, i):
+        p = probs[k]
+        st = lib.dmm_read_probe(p["codes"][i % copies].data_ptr(), sink.data_ptr(), p["N"], p["K"], stream)
+        assert st == 0, st
+    for i in range(3):
+        for k in range(len(probs)):
+            fn(k, i)
+    n = steps * len(probs)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for a, b in ev:
+        a.record(); b.record()
+    torch.cuda.synchronize()
+    j = 0
+    for i in range(steps):
+        for k in range(len(probs)):
+            lib.dmm_set_kernel_events(ev[j][0].cuda_event, ev[j][1].cuda_event)
+            fn(k, i)
+            j += 1
+    lib.dmm_set_kernel_events(None, None)
+    torch.cuda.synchronize()
+    rows = []
+    for k, p in enumerate(probs):
+        v = [ev[i * len(probs) + k][0].elapsed_time(ev[i * len(probs) + k][1]) * 1e-3 for i in range(steps)]
+        t = sum(v) / len(v)
+        b = p["N"] * p["K"] // 4
+        rows.append({"K": p["K"], "N": p["N"], "code_bytes": b, "kernel_us": round(t * 1e6, 3),
+                     "GBps": round(b / t / 1e9, 1), "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBS, 4)})
+    return {"kernel": "dmm::read_probe_kernel", "shapes": rows}
+
+
+def gemv_7b_step(torch, lib, capi, workload, dev, rand_codes):
+    """One decode step's projections of a Llama-2-7B layer as the caller would issue them: fused QKV
+    (4096 -> 12288), o_proj (4096 -> 4096), gate and up as ONE call on their concatenated code rows (4096 ->
+    22016), down (11008 -> 4096); 12 layers' worth of distinct code buffers (590 MB) captured as one HIP graph
+    of 48 launches.  Wall time per layer step and code bytes per second, beside the eager per-shape figures."""
+    layer = ((4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096))
+    layers = 12
+    probs = []
+    for j, (K, N) in enumerate(layer):
+        x, _, grid, scale = workload.make_inputs(1, 8, K, seed=0)
+        probs.append(dict(K=K, N=N, x=x.to(dev), grid=grid.to(dev), scale=scale, codes=rand_codes(N, K, layers, 300 + j),
+                          y=torch.empty(1, N, dtype=torch.float16, device=dev)))
+    layer_bytes = sum(workload.code_bytes(N, K) for K, N in layer)
+
+    def enqueue(stream):
+        for i in range(layers):
+            for p in probs:
+                st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][i].data_ptr(), p["grid"].data_ptr(), p["scale"],
+                                               p["y"].data_ptr(), 1, p["N"], p["K"], stream)
+                if st != 0:
+                    raise capi.DmmError("dmm_decode_matmul_f16", st)
+    enqueue(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        enqueue(torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    reps, times = 10, []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            g.replay()
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) / (reps * layers))
+    t = sorted(times)[len(times) // 2]
+    return {"launches_per_step": len(layer), "shapes": [{"K": K, "N": N} for K, N in layer],
+            "graph": "%d layer steps (%d launches) per replay" % (layers, layers * len(layer)),
+            "us_per_step": round(t * 1e6, 3), "code_bytes_per_step": layer_bytes,
+            "GBps": round(layer_bytes / t / 1e9, 1), "frac_hbm": round(layer_bytes / t / 1e9 / HBM_PEAK_GBS, 4),
+            "kernels": [lib.dmm_gemv_kernel_name(1, N, K).decode() for K, N in layer]}
 
 
 def gemv_packed(torch, lib, capi, workload, probs, copies, stream, steps):

@@ -14,6 +14,7 @@
 #include <hip/hip_runtime.h>
 #include <atomic>
 #include <mutex>
+#include <type_traits>
 #include <vector>
 #include <hip/hip_ext.h>
 #include <stdint.h>
@@ -35,6 +36,7 @@ typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
 typedef int i8_t __attribute__((ext_vector_type(8)));
 
 constexpr int kWave = 64;
+
 
 // ------------------------------------------------------------------ decode tables in LDS
 struct DecodeTables {
@@ -589,11 +591,9 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
 #pragma unroll
         for (int d = 0; d < D; d++) {
             if (i0 + d < n_items) {
-                {
-                    const uint32_t xa = xlane + __umul24((uint32_t)(wave + j * W), xstride);
-                    const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
-                    stream_step<R, JP>(cw[d], xa, lane_base, quarter_bits, acc, nv);
-                }
+                const uint32_t xa = xlane + __umul24((uint32_t)(wave + j * W), xstride);
+                const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
+                stream_step<R, JP>(cw[d], xa, lane_base, quarter_bits, acc, nv);
                 if (++j >= n_sw) {
                     j = 0;
                     finish_block(blk);
@@ -657,14 +657,9 @@ __device__ __forceinline__ u2_t lds_read8(uint32_t byte_addr)
     return *reinterpret_cast<lds_u2_t *>(byte_addr);
 }
 
-// Partial sums of a row block, two parities.  M > 1: one float4 per (wave, tile, quarter, x row), the
-// term columns already added by the wave.  M == 1: the 4 columns per (wave, tile, quarter), added
-// (with their weights) by the one wave that sums the block up; a wave's slots are padded by one
-// float4 so that the 16 waves' slots fall in 16 different bank groups.
-__host__ __device__ constexpr int q8_red_bytes(int R, int W, int M)
-{
-    return M == 1 ? 2 * W * (R * 4 * 4 + 1) * 16 : 2 * W * R * 4 * M * 16;
-}
+// Partial sums of a row block, two parities: one float4 per (wave, tile, quarter, x row), the term
+// columns already added by the wave.
+__host__ __device__ constexpr int q8_red_bytes(int R, int W, int M) { return 2 * W * R * 4 * M * 16; }
 // terms of x (4 rows of K bytes per x row), the per-code means of x as two halves each (hi + lo:
 // 2 rows of K / 8 halves per x row), and one word per wave for the vote on the grid
 __host__ __device__ constexpr int64_t q8_x_bytes(int64_t M, int64_t K)
@@ -770,16 +765,7 @@ __device__ __forceinline__ long q8_pack(uint32_t lo, uint32_t hi)
 // One 256-wide k step for the first nv (uniform, 1 <= nv <= R) of R row tiles; same item order
 // as stream_step.  xaddr: this lane's x terms of the step (16 bytes per word pair: the B
 // operands of its two codes), x8addr: the means of its 8 codes (8 halves: hi or lo, by column).
-//
-// kOne (M = 1): the B operands of a step in two LDS reads instead of five.  A wave-wide read
-// costs the LDS the same whether one lane in 16 wants the bytes or all do, and at M = 1 only
-// the four term columns do.  So columns 0 .. 3 read the pieces of the first MFMA (32 bytes per
-// lane: two reads), columns 4 .. 7 those of the second in the same two reads, and columns 8 and 9
-// the means (hi, lo) in the first of them: every MFMA of the step takes the same registers, the
-// first looks at its columns 0 .. 3 only, the second at 4 .. 7, the shift term at 8 and 9 (what
-// the other columns make of bytes that are not theirs is never read).  xaddr is then the
-// lane's own address by column; x8addr is unused.
-template <int R, bool kOne>
+template <int R>
 __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t x8addr, uint32_t lane_base,
                                         f4_t (&acc)[R][2], f4_t (&accd)[R], int nv)
 {
@@ -789,11 +775,9 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
     u4_t xq[4];
     xq[0] = lds_read16(xaddr);
     xq[1] = lds_read16(xaddr + 16);
-    if constexpr (!kOne) {
-        xq[2] = lds_read16(xaddr + 32);
-        xq[3] = lds_read16(xaddr + 48);
-    }
-    const u4_t x8 = kOne ? xq[0] : lds_read16(x8addr);
+    xq[2] = lds_read16(xaddr + 32);
+    xq[3] = lds_read16(xaddr + 48);
+    const u4_t x8 = lds_read16(x8addr);
 #pragma unroll
     for (int r = 0; r < R; r++) {
         if (r > 0 && r >= nv) break;   // tiles past nv: nothing to do (uniform)
@@ -809,7 +793,7 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
             const i8_t a = i8_t{(int)(b0.g0[0] ^ b0.s0[0]), (int)(b0.g0[1] ^ b0.s0[1]), (int)(b0.g1[0] ^ b0.s1[0]),
                                 (int)(b0.g1[1] ^ b0.s1[1]), (int)(b1.g0[0] ^ b1.s0[0]), (int)(b1.g0[1] ^ b1.s0[1]),
                                 (int)(b1.g1[0] ^ b1.s1[0]), (int)(b1.g1[1] ^ b1.s1[1])};
-            const u4_t &x0 = xq[kOne ? 0 : 2 * h], &x1 = xq[kOne ? 1 : 2 * h + 1];
+            const u4_t &x0 = xq[2 * h], &x1 = xq[2 * h + 1];
             const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
             acc[r][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[r][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
         }
@@ -820,7 +804,7 @@ __device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uin
     }
 }
 
-template <int R, int W, int D, bool kPacked, bool kOne>
+template <int R, int W, int D, bool kPacked>
 __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restrict__ x,
                                                          const uint16_t *__restrict__ codes,
                                                          const void *__restrict__ grid, float scale,
@@ -940,16 +924,9 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
     }
 
     // B operand addresses of this lane: column c16 = 4 m + term (column 0 for the idle ones)
-    // (kOne: columns 0 .. 7 = term c16 % 4 of the first or the second MFMA's 32 bytes, columns 8 and
-    // 9 = the means hi and lo, whose rows advance 64 bytes per step where a term row advances 256;
-    // the other columns repeat 2 .. 7)
     const int col = c16 < 4 * M ? c16 : 0;
     const int row8 = (c16 < 4 * M && (c16 & 3) < 2) ? 2 * (c16 >> 2) + (c16 & 3) : 0;   // hi or lo of x row c16 / 4
-    const bool mean_col = kOne && (c16 == 8 || c16 == 9);
-    const uint32_t xlane = !kOne      ? lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64)
-                           : mean_col ? lds_addr(x8t) + (uint32_t)((c16 - 8) * x8_pitch + q * 16)
-                                      : lds_addr(xt) + (uint32_t)((c16 & 3) * xt_pitch + q * 64 + ((c16 >> 2) & 1) * 32);
-    const uint32_t xstride = mean_col ? 64u : 256u;
+    const uint32_t xlane = lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64);
     const uint32_t x8lane = lds_addr(x8t) + (uint32_t)(row8 * x8_pitch + q * 16);
 
     f4_t acc[R][2];
@@ -965,42 +942,6 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
 
     auto finish_block = [&](int blk) {
         f4_t *rp = red + (blk & 1) * red_par;
-        if constexpr (kOne) {
-            // Batch 1: the wave only leaves 4 columns: term t of the first MFMAs (column t) plus
-            // term t of the second (column 4 + t); the shift term's columns 8 and 9 ride in slots
-            // 0 and 1, the second times 8 to meet the weight 1/8 it gets below ...
-            const float d_scale = c16 == 0 ? 1.f : c16 == 1 ? 8.f : 0.f;
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                f4_t v;
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    v[e] = dpp_shl_add<4>(acc[r][0][e], acc[r][1][e]) + dpp_shl_add<8>(0.f, accd[r][e]) * d_scale;
-                if (c16 < 4) rp[wave * (R * 16 + 1) + (r * 4 + q) * 4 + c16] = v;
-                acc[r][0] = acc[r][1] = accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
-            }
-            __syncthreads();
-            // ... and one wave per tile adds them up: lane (w, quarter) takes wave w's 4 columns with
-            // their weights 8^-c, then the 16 lanes of a row are added with DPP shifts
-            for (int r = wave; r < R; r += W) {
-                const f4_t *src = rp + c16 * (R * 16 + 1) + (r * 4 + q) * 4;
-                f4_t v = src[0];
-#pragma unroll
-                for (int c = 1; c < 4; c++) v += src[c] * __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)c * 3u << 23));
-#pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
-                const int tile = t0 + blk * R + r;
-                const int n = tile * 16 + 4 * q;
-                if (c16 == 15 && tile < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
-                    h4_t o;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
-                    *reinterpret_cast<h4_t *>(y + n) = o;
-                }
-            }
-            return;
-        }
-        (void)xstride;
 #pragma unroll
         for (int r = 0; r < R; r++) {
             // the four term columns of an x row are added first, each with the weight of its term:
@@ -1045,8 +986,7 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             if (i0 + d < n_items) {
                 const uint32_t step = (uint32_t)(wave + j * W);
                 const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
-                q8_step<R, kOne>(cw[d], kOne ? xlane + __umul24(step, xstride) : xlane + step * 256u, x8lane + step * 64u,
-                                 lane_base, acc, accd, nv);
+                q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 64u, lane_base, acc, accd, nv);
                 if (++j >= n_sw) {
                     j = 0;
                     finish_block(blk);
@@ -1055,6 +995,293 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
             }
             issue(cw[d]);
         }
+    }
+}
+
+// ------------------------------------------------------------------ batch 1 on 8-bit operands, x staged in chunks
+// gemv_q8_kernel's arithmetic (fp8 weights by two 8-byte gathers and two exclusive ors per code, x
+// as four bf8 terms, the shift term through the per-code means) for ONE row of x of any length: the
+// terms of x are staged 4096 values (16 k steps, one per wave) at a time into two LDS buffers taken
+// in turn, the chunk after the current one being split while the current one is multiplied, so
+//   * the launch starts multiplying after 512 pieces of x have been split, not after all of them,
+//     and the rest of the splitting runs beside the code stream;
+//   * the LDS holds 37 KB of x however long x is (K = 28672 needs 129 KB in one piece).
+// A workgroup walks its tiles in groups of up to T; within a group it goes chunk by chunk, and
+// in a chunk wave w does k step 16 c + w of every tile of the group with the same two registers
+// of B operands.  One barrier per chunk hands the x buffers over; the partial sums of the T tiles
+// meet once per group.  The code stream is one load per tile in flight per wave, refilled as soon
+// as the tile's step of the chunk is done.
+// LDS map: tables as in gemv_q8_kernel, partial sums [16 waves][T * 16 + 1] float4, two x buffers
+// (4 term rows of 4096 + 16 bytes, 2 rows of means of 1024 + 16 bytes), one flag word.
+constexpr int kQcChunkK = 4096;
+constexpr int kQcTermPitch = kQcChunkK + 16, kQcMeanPitch = kQcChunkK / 4 + 16;
+constexpr int kQcXBuf = 4 * kQcTermPitch + 2 * kQcMeanPitch;
+__host__ __device__ constexpr int qc_red_bytes(int T) { return 16 * (T * 16 + 1) * 16; }
+__host__ __device__ constexpr int qc_lds_bytes(int T) { return kSTablesBytes + qc_red_bytes(T) + 2 * kQcXBuf + 64; }
+
+// the four bf8 terms of a piece of x (8 halves) and the mean of the 8 as hi + lo halves; returns
+// whether all 8 are finite (their fp32 sum is finite exactly when they all are)
+__device__ __forceinline__ bool qc_split_piece(const u4_t &v, u2_t (&t)[4], uint32_t &mean_hi_lo)
+{
+    const h2_t ones = h2_t{(half_t)1.0f, (half_t)1.0f};
+    float r = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r = __builtin_amdgcn_fdot2(as_h2(v[i]), ones, r, false);
+    const bool finite = (__builtin_bit_cast(uint32_t, r) & 0x7F800000u) != 0x7F800000u;
+    r *= 0.125f;
+    const half_t hi = (half_t)r;
+    const half_t lo = (half_t)(r - (float)hi);
+    mean_hi_lo = as_u32(h2_t{hi, lo});
+    const h2_t eight = h2_t{(half_t)8.0f, (half_t)8.0f};
+    u4_t rem = v;
+#pragma unroll
+    for (int term = 0; term < 4; term++) {
+        t[term][0] = __builtin_amdgcn_perm(rem[1], rem[0], 0x07050301u);   // the high bytes of halves 0..3
+        t[term][1] = __builtin_amdgcn_perm(rem[3], rem[2], 0x07050301u);   // and of halves 4..7
+        if (term < 3) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) rem[i] = as_u32((as_h2(rem[i]) - as_h2(rem[i] & 0xFF00FF00u)) * eight);
+        }
+    }
+    return finite;
+}
+
+template <int T, int DC, bool kPacked>
+__global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restrict__ x,
+                                                        const uint16_t *__restrict__ codes,
+                                                        const void *__restrict__ grid, float scale,
+                                                        uint16_t *__restrict__ y, int N, int K, int tiles_q, int tiles_r)
+{
+    constexpr int W = 16;
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+    f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);
+    unsigned char *xbuf = smem_raw + kSTablesBytes + qc_red_bytes(T);
+    uint32_t *flags = reinterpret_cast<uint32_t *>(xbuf + 2 * kQcXBuf);   // [0 .. 15]: one vote per wave; [0] doubles as the running flag
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c16 = lane & 15;
+    const int q = lane >> 4;
+    const int n_steps = K >> 8;
+    const int n_chunks = (n_steps + W - 1) / W;
+    const int row_bytes = K >> 2;
+    const int n_pieces = K >> 3;
+    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;
+
+    // ---- prologue: grid rows to waves 8-11, sign rows to waves 12-15, the first chunk of x to waves 0-7
+    u4_t grow = u4_t{0u, 0u, 0u, 0u};
+    if (wave >= 8 && wave < 12) grow = reinterpret_cast<const u4_t *>(grid)[tid - 512];
+    u4_t xpiece = u4_t{0u, 0u, 0u, 0u};
+    if (wave < 8 && tid < n_pieces) xpiece = reinterpret_cast<const u4_t *>(x)[tid];
+
+    // this workgroup's tiles [t0, t1), walked in n_groups groups of up to T tiles whose sizes differ by
+    // at most one (7 tiles with T = 3: 3 + 2 + 2, not 3 + 3 + 1: a group of one leaves a wave a single
+    // load in flight)
+    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
+    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
+    const int n_groups = (t1 - t0 + T - 1) / T;
+    const int g_base = (t1 - t0) / n_groups, g_rem = (t1 - t0) % n_groups;
+    const int total = n_groups * n_chunks;   // chunks to go through, over all groups
+
+    const int n_tiles_all = (N + 15) >> 4;
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_tiles_all * 16 : N) * row_bytes), 0x00020000);
+    const int voff = kPacked ? lane * 16 : c16 * row_bytes + q * 16;
+    constexpr int kOut = (int)0x80000000;
+    // the code word of (group g, chunk c, tile t of the group) for this wave; out of range: zeros, no access
+    auto issue = [&](u4_t &cwd, int g, int c, int t) {
+        const int gt0 = t0 + g * g_base + (g < g_rem ? g : g_rem), gn = g_base + (g < g_rem ? 1 : 0);
+        const int tile = gt0 + t, step = c * W + wave;
+        const bool ok = g < n_groups && t < gn && step < n_steps;
+        const int soff = !ok ? kOut : kPacked ? (tile * n_steps + step) * 1024 : tile * 16 * row_bytes + step * 64;
+        cwd = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, soff, 0);
+    };
+    // the ring: DC chunks deep, one slot per tile of the group
+    u4_t cw[DC][T];
+    {
+        int g = 0, c = 0;
+#pragma unroll
+        for (int d = 0; d < DC; d++) {
+#pragma unroll
+            for (int t = 0; t < T; t++) issue(cw[d][t], g, c, t);
+            if (++c == n_chunks) { c = 0; g++; }
+        }
+    }
+
+    // one piece of x -> its terms and means in buffer `buf` (piece p of the chunk); returns finite
+    auto stage_piece = [&](const u4_t &v, int buf, int p) {
+        u2_t tm[4];
+        uint32_t mb;
+        const bool fin = qc_split_piece(v, tm, mb);
+        unsigned char *xb = xbuf + buf * kQcXBuf;
+#pragma unroll
+        for (int term = 0; term < 4; term++) *reinterpret_cast<u2_t *>(xb + term * kQcTermPitch + p * 8) = tm[term];
+        reinterpret_cast<uint16_t *>(xb + 4 * kQcTermPitch)[p] = (uint16_t)mb;
+        reinterpret_cast<uint16_t *>(xb + 4 * kQcTermPitch + kQcMeanPitch)[p] = (uint16_t)(mb >> 16);
+        return fin;
+    };
+
+    bool fits = true;   // stays true while x is finite and the grid fits fp8
+    if (wave >= 12) {
+        // sign rows: 128 rows of 16 slots (16 bytes = two copies each); thread t of these 256 writes
+        // 8 slots of row t / 2 (16 neighbouring lanes hit 16 different slot positions)
+        const int t = tid - 768, row = t >> 1;
+        const u2_t sb = sign_bytes((uint32_t)row);
+        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw) + row * 16 + (t & 1) * 8;
+#pragma unroll
+        for (int i = 0; i < 8; i++) sg[(i + row) & 7] = u4_t{sb[0], sb[1], sb[0], sb[1]};
+    } else if (wave >= 8) {
+        bool exact;
+        const u2_t g8 = grid_row_fp8(grow, exact);
+        fits = exact;
+        const int r = tid - 512;
+        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes) + r * 16;
+#pragma unroll
+        for (int i = 0; i < 16; i++) gg[(i + r) & 15] = u4_t{g8[0], g8[1], g8[0], g8[1]};
+    } else {
+        fits = stage_piece(xpiece, 0, tid);
+    }
+    // the vote: every wave publishes whether something of its own failed, in a word of its own (so
+    // nothing needs clearing first), and after the barrier every wave reads all of them
+    {
+        const bool wave_bad = __builtin_amdgcn_ballot_w64(!fits) != 0;
+        if (lane == 0) flags[wave] = wave_bad ? 1u : 0u;
+    }
+    __syncthreads();
+    // a grid value that does not fit 8 bits, or (here or in a later chunk) an x that is not finite: the
+    // 16-bit kernel does the whole call over, at the end of this function
+    bool hand_over = __builtin_amdgcn_ballot_w64(flags[lane & (W - 1)] != 0) != 0;
+
+    // B operands of this lane: columns 0 .. 7 = term c16 % 4 of the first or the second MFMA's 32 bytes
+    // of the wave's k step, columns 8 and 9 = the means (hi, lo); the other columns repeat 2 .. 7.
+    // Wave w always does step w of a chunk, so the address only depends on the buffer.
+    const bool mean_col = c16 == 8 || c16 == 9;
+    const uint32_t xlane = lds_addr(xbuf) + (mean_col ? (uint32_t)(4 * kQcTermPitch + (c16 - 8) * kQcMeanPitch + q * 16 + wave * 64)
+                                                      : (uint32_t)((c16 & 3) * kQcTermPitch + q * 64 + ((c16 >> 2) & 1) * 32 + wave * 256));
+
+    f4_t acc[T][2], accd[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) acc[t][0] = acc[t][1] = accd[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+    const float d_scale = c16 == 0 ? 1.f : c16 == 1 ? 8.f : 0.f;
+
+    // With one or two chunks all of x stays resident once staged (chunk c in buffer c); longer x goes
+    // through the two buffers in turn and is staged again for every group.
+    const bool resident = n_chunks <= 2;
+    int g = 0, c = 0;            // group and chunk of the chunk being multiplied
+    int pg = 0, pc = 0;          // ... of the chunk DC further on, whose code words refill the slots
+#pragma unroll
+    for (int d = 0; d < DC; d++)
+        if (++pc == n_chunks) { pc = 0; pg++; }
+    bool barrier_in_group = true;   // the prologue's
+
+    // one chunk; kSlot: its ring slot (static).  Every path issues exactly T code loads (tiles and
+    // steps that do not exist load nothing and get zeros), so the wait counters stay exact.
+    auto chunk = [&](auto slot_tag, int gc) {
+        constexpr int kSlot = decltype(slot_tag)::value;
+        const bool exists = gc < total;
+        const int gn = g_base + (g < g_rem ? 1 : 0);
+        const int ntg = exists ? gn : 0;                          // tiles of this group (uniform)
+        const bool last_c = c + 1 == n_chunks;
+        const int xb_cur = resident ? c : gc & 1;
+        // the chunk after this one: if its x is not in LDS yet, half of the waves split it while everybody
+        // multiplies, waves 0-7 and 8-15 taking turns
+        const int ng = last_c ? g + 1 : g, nc = last_c ? 0 : c + 1;
+        const bool stage_next = exists && gc + 1 < total && (!resident || gc + 1 < n_chunks);
+        const bool stager = stage_next && wave < 8;   // the waves the arbiter prefers: they are through their steps first
+        const int sp = tid & 511;
+        if (stager) {
+            const int p = nc * 512 + sp;
+            xpiece = p < n_pieces ? reinterpret_cast<const u4_t *>(x)[p] : u4_t{0u, 0u, 0u, 0u};
+        }
+        const bool step_ok = exists && c * W + wave < n_steps;
+        u4_t x0 = u4_t{0u, 0u, 0u, 0u}, x1 = x0;
+        if (step_ok) {
+            const uint32_t xa = xlane + (uint32_t)(xb_cur * kQcXBuf);
+            x0 = lds_read16(xa);
+            x1 = lds_read16(xa + 16);
+        }
+        const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            const bool live = step_ok && t < ntg;   // uniform
+            Q8Gather gt[4];
+            u4_t a8 = u4_t{0u, 0u, 0u, 0u};
+            if (live) {
+#pragma unroll
+                for (int t2 = 0; t2 < 4; t2++) q8_gather(gt[t2], cw[kSlot][t][t2], lane_base);
+                a8 = (cw[kSlot][t] & 0x80008000u) | 0x40004000u;   // +-2.0 per code: the shift term's A operand
+            }
+            if (live) {
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const Q8Gather &b0 = gt[2 * h], &b1 = gt[2 * h + 1];
+                    const i8_t a = i8_t{(int)(b0.g0[0] ^ b0.s0[0]), (int)(b0.g0[1] ^ b0.s0[1]), (int)(b0.g1[0] ^ b0.s1[0]),
+                                        (int)(b0.g1[1] ^ b0.s1[1]), (int)(b1.g0[0] ^ b1.s0[0]), (int)(b1.g0[1] ^ b1.s0[1]),
+                                        (int)(b1.g1[0] ^ b1.s1[0]), (int)(b1.g1[1] ^ b1.s1[1])};
+                    acc[t][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[t][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
+                }
+                accd[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8_t, a8), __builtin_bit_cast(h8_t, x0), accd[t], 0, 0, 0);
+            }
+            issue(cw[kSlot][t], pg, pc, t);                        // the slot's next code word
+        }
+        if (stager && !stage_piece(xpiece, resident ? nc : (gc + 1) & 1, sp)) flags[0] = 1u;
+        if (!exists) return;
+        const bool group_end = last_c;
+        if (group_end) {
+            // `red` still holds the sums of the group before while its reducers read them: a barrier has
+            // to lie between their read and this write
+            if (!barrier_in_group) __syncthreads();
+            // the group's partial sums: 4 columns per (wave, tile, quarter) - term t of the first MFMAs
+            // (column t) plus term t of the second (column 4 + t); the shift term's columns 8 and 9 ride
+            // in slots 0 and 1, the second times 8 to meet the weight 1/8 it gets from the reducer
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                if (t >= ntg) break;
+                f4_t v;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    v[e] = dpp_shl_add<4>(acc[t][0][e], acc[t][1][e]) + dpp_shl_add<8>(0.f, accd[t][e]) * d_scale;
+                if (c16 < 4) red[wave * (T * 16 + 1) + (t * 4 + q) * 4 + c16] = v;
+                acc[t][0] = acc[t][1] = accd[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+        barrier_in_group = !group_end && (barrier_in_group || stage_next);
+        if (stage_next || group_end) {
+            __syncthreads();   // hands the x buffers over and / or gathers the group's partial sums
+            if (stage_next && __builtin_amdgcn_ballot_w64(flags[0] != 0) != 0) hand_over = true;
+        }
+        if (group_end && !hand_over && wave < ntg) {
+            // wave t adds up tile t: lane (w, quarter) takes wave w's 4 columns with their weights 8^-c,
+            // then the 16 lanes of a row are added with DPP shifts
+            const f4_t *src = red + c16 * (T * 16 + 1) + (wave * 4 + q) * 4;
+            f4_t v = src[0];
+#pragma unroll
+            for (int cc = 1; cc < 4; cc++) v += src[cc] * __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)cc * 3u << 23));
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
+            const int gt0 = t0 + g * g_base + (g < g_rem ? g : g_rem);
+            const int n = (gt0 + wave) * 16 + 4 * q;
+            if (c16 == 15 && n < N) {   // N % 4 == 0, so the four rows are in range together
+                h4_t o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
+                *reinterpret_cast<h4_t *>(y + n) = o;
+            }
+        }
+        if (++c == n_chunks) { c = 0; g++; }
+        if (++pc == n_chunks) { pc = 0; pg++; }
+    };
+
+    for (int gc = 0; gc < total && !hand_over; gc += DC) {
+        chunk(std::integral_constant<int, 0>{}, gc);
+        if constexpr (DC > 1) {
+            if (!hand_over) chunk(std::integral_constant<int, 1>{}, gc + 1);
+        }
+    }
+    if (hand_over) {
+        __syncthreads();   // everybody has read the flags before the LDS is laid out anew
+        gemv_stream_body<1, W, 2, kPacked, 4>(x, codes, grid, scale, y, 1, N, K, tiles_q, tiles_r);
     }
 }
 
@@ -2330,6 +2557,33 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ 
     }
 }
 
+// ------------------------------------------------------------------ plain read of a code matrix
+// What the memory system gives a kernel that only reads: the batch-1 kernels' launch shape (one
+// workgroup of 16 waves per compute unit over contiguous ranges of 16-row tiles, a wave's load 16
+// rows x 64 bytes, the waves of a workgroup dealing out the 256-wide k steps) with two loads in flight
+// per wave and an exclusive or in place of the decode.  The yardstick the benchmark prints beside the
+// batch-1 kernels; `sink` is written only if the bytes happen to cancel (never for random codes),
+// which keeps the loads alive.
+__global__ __launch_bounds__(1024) void read_probe_kernel(const uint16_t *__restrict__ codes, uint32_t *__restrict__ sink,
+                                                          int N, int K, int tiles_q, int tiles_r)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, q = lane >> 4;
+    const int n_steps = K >> 8, row_bytes = K >> 2;
+    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
+    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
+    const __amdgpu_buffer_rsrc_t crsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
+    const int voff = c16 * row_bytes + q * 16;
+    u4_t acc = u4_t{0u, 0u, 0u, 0u};
+    for (int tile = t0; tile < t1; tile++)
+        for (int step = wave; step < n_steps; step += 32) {
+            const u4_t a = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, tile * 16 * row_bytes + step * 64, 0);
+            const u4_t b = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, step + 16 < n_steps ? tile * 16 * row_bytes + (step + 16) * 64 : (int)0x80000000, 0);
+            acc ^= a ^ b;
+        }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9E3779B9u && N < 0) sink[0] = acc[0];
+}
+
 // ------------------------------------------------------------------ scratch memory of the library
 // The one buffer the library owns: split-K partial sums for dmm_decode_matmul_noalloc_f16, whose
 // callers cannot allocate.  In host code the array's name is a stand-in, not a device address;
@@ -2391,9 +2645,7 @@ const std::vector<KernelInfo> &kernel_table()
 #define DMM_BOTH_LAYOUTS(X) X(false), X(true)
 #define DMM_K_STREAM(P) kinfo(gemv_stream_kernel<1, 16, 2, P, 4>, kLdsMax, true), kinfo(gemv_stream_kernel<1, 16, 2, P, 1>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_STREAM),
-#define DMM_K_Q8(P)                                                                                          \
-    kinfo(gemv_q8_kernel<1, 16, 2, P, true>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 2, P, false>, kLdsMax, true), \
-        kinfo(gemv_q8_kernel<1, 16, 3, P, true>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P, false>, kLdsMax, true)
+#define DMM_K_Q8(P) kinfo(gemv_q8_kernel<1, 16, 2, P>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P>, kLdsMax, true), kinfo(gemv_q8c_kernel<3, 1, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_Q8),
 #define DMM_K_REGX(P)                                                                                        \
     kinfo(gemv_regx_kernel<1, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 1, 2, P>, kLdsMax, true),     \
@@ -2540,13 +2792,32 @@ int launch_gemv_q8(const void *x, const void *codes, const void *grid, float sca
     const size_t shmem = (size_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    if (M == 1)   // the B operands of a step in two LDS reads
-        return launch(gemv_q8_kernel<R, W, D, kPacked, true>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
-                      (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N,
-                      (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
-    return launch(gemv_q8_kernel<R, W, D, kPacked, false>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+    return launch(gemv_q8_kernel<R, W, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+// the chunked 8-bit kernel: one row of x of any length the 16-bit kernel could take over (its x in LDS)
+bool gemv_q8c_ok(int64_t M, int64_t N, int64_t K)
+{
+    return M == 1 && (int64_t)kSTablesBytes + stream_red_bytes(1, 16, 1) + stream_x_bytes(1, K) <= kLdsMax &&
+           N * (K >> 2) < (1LL << 31);
+}
+
+// groups of up to three tiles, one code load per tile in flight per wave (four tiles per group spill
+// registers; two chunks in flight per wave were no faster)
+template <bool kPacked>
+int launch_gemv_q8c(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t N, int64_t K,
+                    hipStream_t stream)
+{
+    constexpr int T = 3;
+    size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(1, 16, 1) + (size_t)stream_x_bytes(1, K);   // the 16-bit hand-over
+    if (shmem < (size_t)qc_lds_bytes(T)) shmem = qc_lds_bytes(T);
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(gemv_q8c_kernel<T, 1, kPacked>, dim3((unsigned)wgs), dim3(1024), shmem, stream, (const uint16_t *)x,
+                  (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)N, (int)K, (int)(n_tiles / wgs),
+                  (int)(n_tiles % wgs));
 }
 
 template <int R, int W>
@@ -2584,29 +2855,36 @@ inline bool gemv_q8_enabled()
     return on == 1;
 }
 
-// The 8-bit kernel, one row tile at a time; the code stream three loads deep per wave when a
-// workgroup has more than two row tiles to walk through, two deep for shorter launches (where
-// a larger first burst only delays the first tile).
+// The 8-bit kernels.  One row of x: the chunked kernel.  Two to four rows: one row tile at a time, the
+// code stream three loads deep per wave when a workgroup has more than two row tiles to walk
+// through, two deep for shorter launches (where a larger first burst only delays the first tile).
 template <bool kPacked>
 int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                 int64_t N, int64_t K, hipStream_t stream)
 {
+    if (M == 1) return launch_gemv_q8c<kPacked>(x, codes, grid, scale, y, N, K, stream);
     const int64_t n_tiles = (N + 15) / 16;
     if (n_tiles > 2 * cu_count()) return launch_gemv_q8<1, 16, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
     return launch_gemv_q8<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
 }
 
-// The choice among the matrix-vector kernels.  Launches of more than three row tiles per
-// workgroup: the 8-bit kernel where it applies (its prologue is the dearer one, a grid that does
-// not fit fp8 costs it a second table build, and the 16-bit kernel's y is the correctly rounded
-// one).  Otherwise the 16-bit streaming kernel, one tile at a time; the register-x kernel when x
-// does not fit the LDS.
+// whether an 8-bit kernel can take the shape at all (grid and x permitting, which the kernel finds out)
+bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok(M, N, K) : gemv_q8_ok<1, 16>(M, N, K); }
+
+// The choice among the matrix-vector kernels.  The 8-bit kernels where they apply and pay: one row of x
+// from three row tiles per workgroup on (measured, 8-bit against 16-bit kernel, us: 8192 -> 10240 8.3 / 8.9,
+// 4096 -> 12288 5.4 / 5.9, 4096 -> 11008 5.5 / 6.2; with two tiles or fewer the 16-bit kernel wins, 8192 ->
+// 8192 7.2 / 6.5, its prologue being the cheaper one), two to four rows from more than three tiles on.  A
+// grid that does not fit fp8 costs them a second table build, and the 16-bit kernel's y is the
+// correctly rounded one.  Otherwise the 16-bit streaming kernel, one tile at a time; the register-x
+// kernel when x does not fit the LDS.
 enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
 
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
-    const bool long_launch = (N + 15) / 16 > 3 * (int64_t)cu_count();
-    if (long_launch && gemv_q8_enabled() && gemv_q8_ok<1, 16>(M, N, K)) return kGemvQ8;
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const bool long_launch = M == 1 ? n_tiles > 2 * cus : n_tiles > 3 * cus;
+    if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
     if (gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
     return kGemvRegx;
 }
@@ -2959,7 +3237,7 @@ const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K)
     if (M > 16) return "dmm::gemv_regx_kernel";
     switch (pick_gemv(M, N, K)) {
         case kGemvStream: return "dmm::gemv_stream_kernel";
-        case kGemvQ8: return "dmm::gemv_q8_kernel";
+        case kGemvQ8: return M == 1 ? "dmm::gemv_q8c_kernel" : "dmm::gemv_q8_kernel";
         default: return "dmm::gemv_regx_kernel";
     }
 }
@@ -2969,7 +3247,7 @@ int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float 
 {
     int st = check_common(x, codes, grid, y, M, N, K);
     if (st != DMM_OK || M == 0 || N == 0) return st;
-    if (!gemv_ok(x, codes, grid, y, M, N, K) || !gemv_q8_ok<1, 16>(M, N, K)) return DMM_ERR_UNSUPPORTED;
+    if (!gemv_ok(x, codes, grid, y, M, N, K) || !gemv_8bit_ok(M, N, K)) return DMM_ERR_UNSUPPORTED;
     if ((st = ensure_ready((hipStream_t)stream))) return st;
     return run_gemv_q8<false>(x, codes, grid, scale, y, M, N, K, (hipStream_t)stream);
 }
@@ -3098,6 +3376,18 @@ int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid,
     if (workspace && workspace_bytes > 0 && !aligned(workspace, 16)) return DMM_ERR_MISALIGNED;
     if ((st = ensure_ready((hipStream_t)stream))) return st;
     return dispatch_f16(x, codes, grid, scale, y, M, N, K, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int dmm_read_probe(const void *codes, void *sink, int64_t N, int64_t K, void *stream)
+{
+    if (N < 1 || K < 256 || (K & 255) || N * (K >> 2) >= (1LL << 31)) return DMM_ERR_UNSUPPORTED;
+    if (!codes || !sink) return DMM_ERR_NULL_POINTER;
+    if (!aligned(codes, 16) || !aligned(sink, 4)) return DMM_ERR_MISALIGNED;
+    if (int st = ensure_ready((hipStream_t)stream)) return st;
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(read_probe_kernel, dim3((unsigned)wgs), dim3(1024), 0, (hipStream_t)stream, (const uint16_t *)codes,
+                  (uint32_t *)sink, (int)N, (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
 
 int64_t dmm_noalloc_scratch_bytes(void) { return kScratchBytes; }

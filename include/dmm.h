@@ -225,6 +225,14 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K);
  * only timer (/root/reference/test_decode_matmul.py:8-22) brackets the whole call. */
 int dmm_set_kernel_events(void *start_event, void *stop_event);
 
+/* Yardstick for benchmarks: a kernel that only READS a row-major code matrix [N, K/8] with the
+ * batch-1 kernels' launch shape and access pattern (16 rows x 64 bytes per wave load) and does no
+ * decoding; timed with dmm_set_kernel_events like any other call, it shows what the memory system
+ * gives a launch of this size.  `sink`: 4 bytes of device memory that the kernel never writes in
+ * practice.  K % 256 == 0, 16-byte aligned codes, N * K / 4 below 2 GiB (DMM_ERR_UNSUPPORTED
+ * otherwise).  No counterpart in the reference. */
+int dmm_read_probe(const void *codes, void *sink, int64_t N, int64_t K, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

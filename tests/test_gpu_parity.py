@@ -129,6 +129,14 @@ def test_auto_dispatch_and_torch_operator(M, N, K):
 # ----------------------------------------------------------------- batch-1 kernel, 8-bit operands
 # M <= 4 with x small enough for the LDS runs on fp8 weights / bf8 terms of x when every grid
 # value fits fp8, and hands over to the 16-bit kernel inside the same launch when one does not.
+def _in_8bit_domain(M, K):
+    """LDS budget of the 8-bit kernels: one row of x is staged in chunks and only has to fit as halves (the
+    16-bit kernel may have to take the call over); two to four rows keep all their terms in LDS."""
+    if M == 1:
+        return 96 * 1024 + 2 * 16 * 4 * 16 + (2 * K + 16) + 128 <= 160 * 1024
+    return 96 * 1024 + 2 * 16 * 4 * M * 16 + 4 * M * (K + 16) + 2 * M * (K // 4 + 16) + 64 <= 160 * 1024
+
+
 def _gemv_vs_oracle(x, codes, grid, scale, packed=False, path="gemv8"):
     W = orc.decode_f16(codes, grid)
     ref = orc.matmul_f32(x, W, scale)
@@ -144,9 +152,7 @@ def _gemv_vs_oracle(x, codes, grid, scale, packed=False, path="gemv8"):
 @pytest.mark.parametrize("N,K", [(16, 256), (52, 1024), (4360, 2048), (1000, 4096), (12304, 8192)])
 @pytest.mark.parametrize("grid_kind", ["e8p", "fp8_all", "half_any", "one_off"])
 def test_gemv_8bit_operands_and_fallback(M, N, K, grid_kind):
-    red = 2 * 16 * 17 * 16 if M == 1 else 2 * 16 * 4 * M * 16
-    terms = 4 * M * (K + 16) + 2 * M * (K // 4 + 16) + 64
-    if 96 * 1024 + red + terms > 160 * 1024:
+    if not _in_8bit_domain(M, K):
         pytest.skip("the terms of x do not fit the LDS beside the tables: outside the kernel's domain")
     rng = np.random.default_rng(M * 7 + N + K)
     if grid_kind == "e8p":
@@ -178,6 +184,39 @@ def test_gemv_8bit_operands_and_fallback(M, N, K, grid_kind):
         assert torch.equal(y, ya)                # launches this long take the 8-bit kernel by themselves
 
 
+@pytest.mark.parametrize("N,K", [(48, 4352), (1000, 8192), (12304, 12288), (4112, 28672), (24592, 4096),
+                                 (16400, 9216), (28672, 8192)])
+@pytest.mark.parametrize("grid_kind", ["e8p", "half_any"])
+def test_gemv_8bit_one_row_of_x_in_chunks(N, K, grid_kind):
+    """The batch-1 form of the 8-bit kernel stages x 4096 values at a time: a last chunk that is not
+    full (K = 4352, 9216), x resident after one pass (K <= 8192) with one to three groups of tiles per
+    workgroup (N = 24592: 1538 tiles on 256 workgroups), x staged again for every group (K = 12288 with
+    two groups, K = 28672), and the hand-over to the 16-bit kernel for a grid no fp8 can hold."""
+    rng = np.random.default_rng(N + K)
+    grid = orc.grid_from_codebook(orc.build_codebook_abs())
+    if grid_kind == "half_any":
+        grid = (finite_random_grid(N).astype(np.float32).clip(-8, 8)).astype(np.float16)
+    x = rng.standard_normal((1, K)).astype(np.float16)
+    codes = rng.integers(0, 65536, size=(N, K // 8)).astype(np.uint16)
+    scale = float(np.float32(1.0 / (np.sqrt(K) * max(1.0, float(np.sqrt(np.mean(grid.astype(np.float64) ** 2)))))))
+    y, ref = _gemv_vs_oracle(x, codes, grid, scale)
+    assert_close_to_oracle(y, ref, "8-bit gemv in chunks %s N=%d K=%d" % (grid_kind, N, K))
+    y2, _ = _gemv_vs_oracle(x, codes, grid, scale)
+    assert torch.equal(y, y2)                    # same bits run after run
+    ya, _ = _gemv_vs_oracle(x, codes, grid, scale, path="auto")
+    yp, _ = _gemv_vs_oracle(x, codes, grid, scale, packed=True)
+    assert torch.equal(ya, yp)                   # packed codes: same kernel choice, same arithmetic, same order
+    if (N + 15) // 16 > 2 * 256:
+        assert torch.equal(y, ya)                # launches this long take the 8-bit kernel by themselves
+    if grid_kind == "half_any":                  # handed over: exactly the 16-bit kernel's result
+        was = capi.lib().dmm_set_gemv_8bit(0)
+        try:
+            y16 = c_matmul(dev(x), dev(codes), dev(grid), scale, "gemv")
+        finally:
+            capi.lib().dmm_set_gemv_8bit(was)
+        assert torch.equal(y, y16)
+
+
 def test_gemv_8bit_exact_for_extreme_x():
     """One non-zero x at a time, from all over the half range (largest, smallest normal,
     subnormals, all 11 significant bits set), against weights 0 and +-0.5: the four bf8 terms
@@ -206,8 +245,7 @@ def _random_8bit_cases(n, seed):
     while len(out) < n:
         M = int(rng.integers(1, 5))
         K = 256 * int(rng.integers(1, 50))
-        red = 2 * 16 * 17 * 16 if M == 1 else 2 * 16 * 4 * M * 16
-        if 96 * 1024 + red + 4 * M * (K + 16) + 2 * M * (K // 4 + 16) + 64 > 160 * 1024:
+        if not _in_8bit_domain(M, K):
             continue
         N = 4 * int(rng.integers(1, 1400)) if len(out) % 3 else 4 * int(rng.integers(1100, 2600))
         out.append((M, N, K))
@@ -243,9 +281,13 @@ def test_gemv_8bit_switch_and_kernel_name():
     ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
     was = lib.dmm_set_gemv_8bit(1)
     try:
-        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_q8_kernel"
-        assert lib.dmm_gemv_kernel_name(M, 12288, K) == b"dmm::gemv_stream_kernel"    # three tiles per CU
-        assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_stream_kernel"    # x terms do not fit
+        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_q8c_kernel"
+        assert lib.dmm_gemv_kernel_name(M, 12288, K) == b"dmm::gemv_q8c_kernel"       # three tiles per CU
+        assert lib.dmm_gemv_kernel_name(M, 8192, K) == b"dmm::gemv_stream_kernel"     # two
+        assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_q8c_kernel"       # x goes through in chunks
+        assert lib.dmm_gemv_kernel_name(3, N, K) == b"dmm::gemv_q8_kernel"            # two to four rows of x
+        assert lib.dmm_gemv_kernel_name(3, 12288, K) == b"dmm::gemv_stream_kernel"
+        assert lib.dmm_gemv_kernel_name(3, N, 28672) == b"dmm::gemv_regx_kernel"      # their terms do not fit
         assert lib.dmm_gemv_kernel_name(32, N, K) == b"dmm::gemv_regx_kernel"
         assert lib.dmm_gemv_kernel_name(M, N, 264) == b""
         y8 = c_matmul(dev(x), dev(codes), dev(grid), scale, "auto")
@@ -262,6 +304,23 @@ def test_gemv_8bit_switch_and_kernel_name():
         assert (y8.cpu().numpy() != want.astype(np.float16)).mean() < 0.05
     finally:
         lib.dmm_set_gemv_8bit(was)
+
+
+def test_gemv_8bit_non_finite_x_in_a_later_chunk():
+    """One row of x, staged in chunks: an infinity in the third chunk is found after two chunks have been
+    multiplied; the 16-bit kernel then does the whole call over."""
+    K, N = 12288, 16400
+    rng = np.random.default_rng(10)
+    grid = orc.grid_from_codebook(orc.build_codebook_abs())
+    x = rng.standard_normal((1, K)).astype(np.float16)
+    x[0, 8200] = -np.inf
+    codes = rng.integers(0, 65536, size=(N, K // 8)).astype(np.uint16)
+    y, ref = _gemv_vs_oracle(x, codes, grid, 0.01)
+    got = y.cpu().numpy().astype(np.float32)
+    assert np.isinf(got).any() and not np.isnan(ref).any()
+    assert np.array_equal(np.isinf(got), np.isinf(ref)) and np.array_equal(got[np.isinf(got)], ref[np.isinf(ref)])
+    fin = np.isfinite(ref)
+    assert np.all(np.abs(got[fin] - ref[fin]) <= 1e-2 + 1e-2 * np.abs(ref[fin]))
 
 
 def test_gemv_8bit_non_finite_x():

@@ -60,7 +60,8 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert lib.dmm_gemv_f16(p, p, p, 1.0, p, 1, 4, 16, None) == -5       # K % 256 != 0
     assert lib.dmm_gemv_f16(p, p, p, 1.0, p, 64, 4, 256, None) == -5     # M too large
     assert lib.dmm_gemv_8bit_f16(p, p, p, 1.0, p, 5, 4, 256, None) == -5    # M > 4
-    assert lib.dmm_gemv_8bit_f16(p, p, p, 1.0, p, 1, 4, 28672, None) == -5  # x terms do not fit the LDS
+    assert lib.dmm_gemv_8bit_f16(p, p, p, 1.0, p, 2, 4, 28672, None) == -5  # the terms of two rows of x do not fit the LDS
+    assert lib.dmm_gemv_8bit_f16(p, p, p, 1.0, p, 1, 4, 32768, None) == -5  # one row: the 16-bit hand-over does not fit
     assert lib.dmm_gemv_8bit_f16(None, p, p, 1.0, p, 1, 4, 256, None) == -1
     assert lib.dmm_gemm_f16(p, p, p, 1.0, p, 64, 4, 16, None) == -5      # K % 64 != 0
     # empty problems succeed without touching the device
