@@ -31,8 +31,14 @@ def _abs_rows():
 
 def build_codebook_abs(device="cpu"):
     """int64[256]; entry i packs byte d = (4 * row_i[d]) & 255.  Rows are ordered by squared
-    norm with ties kept in enumeration order (stable), which fixes the one thing the
-    reference's unstable argsort (test_decode_matmul.py:84) leaves open."""
+    norm with ties kept in enumeration order (stable).
+
+    The SET of rows is the reference's; the ORDER is not: the reference sorts with an unstable
+    argsort over keys that tie up to 126-fold (test_decode_matmul.py:84), and what that returns
+    depends on the torch build (under torch 2.10 on CPU 251 of the 256 rows sit at other indices than
+    here; tests/golden/reference_codebook_order.json holds that table).  Codes quantised against
+    another table must be decoded with THAT table: pass it to the operator, which takes the table
+    as an input and assumes no order."""
     rows = torch.tensor(_abs_rows(), dtype=torch.float64)
     order = torch.sort(rows.square().sum(1), stable=True).indices
     rows = rows[order]

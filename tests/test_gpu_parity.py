@@ -927,6 +927,29 @@ def test_reference_call_under_the_reference_name():
         decode_matmul(dev(xh), dev(ch), dev(gh))     # the half-precision form needs its scale
 
 
+@pytest.mark.parametrize("M", [1, 4])
+def test_projections_sharing_x_are_one_call_on_concatenated_rows(M):
+    """Several projections of the same activations (gate and up of a Llama-2-7B MLP, 4096 -> 2 x 11008)
+    need no grouped entry point: rows of W are independent, so one call on the concatenated code rows
+    gives, row for row, what the separate calls give - bit for bit when both run the same kernel
+    (they do here), and the oracle's product within the operator's tolerance."""
+    K, N1 = 4096, 11008
+    x, gate, grid, scale = workload.make_inputs(M, N1, K, seed=21)
+    _, up, _, _ = workload.make_inputs(M, N1, K, seed=22)
+    xd, gd = dev(x), dev(grid)
+    both = torch.cat([dev(gate), dev(up)], dim=0).contiguous()
+    y_cat = c_matmul(xd, both, gd, scale, "auto")
+    y_gate = c_matmul(xd, dev(gate), gd, scale, "auto")
+    y_up = c_matmul(xd, dev(up), gd, scale, "auto")
+    torch.cuda.synchronize()
+    lib = capi.lib()
+    assert lib.dmm_gemv_kernel_name(M, N1, K) == lib.dmm_gemv_kernel_name(M, 2 * N1, K)
+    assert torch.equal(y_cat[:, :N1], y_gate) and torch.equal(y_cat[:, N1:], y_up)
+    for codes, y in ((gate, y_gate), (up, y_up)):
+        ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
+        assert_close_to_oracle(y, ref, "projection sharing x, M=%d" % M)
+
+
 def test_kernel_event_hook_times_the_kernel():
     x, codes, grid, scale = workload.make_inputs(1, 8192, 8192, seed=2)
     xd, cd, gd = dev(x), dev(codes), dev(grid)
