@@ -74,7 +74,7 @@ def main():
     from decode_matmul_amd import capi, workload
 
     if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the operator has no CPU path", file=sys.stderr)
+        print("bench.py: no GPU visible; this benchmark measures the GPU kernels", file=sys.stderr)
         sys.exit(3)
     dev = "cuda:0"
     torch.cuda.set_device(0)

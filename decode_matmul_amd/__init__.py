@@ -10,10 +10,11 @@ in the half-precision form of the same code format:
     W = decode(codes, grid)                       # dense half [N,K], bit-exact decode
 
 The functions are the compiled PyTorch operator (`_C`, host C++) over the C ABI of
-`libdmm.so` (hand-written HIP).  There is no CPU implementation: without the built extension
-every operator raises ImportError (the import itself succeeds, so that
-`python -m decode_matmul_amd.build` can run on a fresh tree), and calling the operator with
-CPU tensors raises.
+`libdmm.so` (hand-written HIP).  GPU tensors run the HIP kernels; `decode_matmul` and `decode` also
+take tensors in host memory, which go to the library's own host route (plain C++ loops, the
+counterpart of the reference's CPU path, test_decode_matmul.py:29-71).  Nothing falls back: without
+the built extension every operator raises ImportError (the import itself succeeds, so that
+`python -m decode_matmul_amd.build` can run on a fresh tree).
 """
 import os as _os
 

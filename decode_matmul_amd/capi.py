@@ -34,6 +34,8 @@ SYMBOLS = {
     "dmm_decode_matmul_packed_f16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _I64, _I64, _I64, _P, _I64, _P]),
     "dmm_decode_matmul_i8": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, ctypes.c_int, _P]),
     "dmm_set_kernel_events": (ctypes.c_int, [_P, _P]),
+    "dmm_decode_host_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64]),
+    "dmm_decode_matmul_host_f16": (ctypes.c_int, [_P, _P, _P, _F, _P, _I64, _I64, _I64]),
     "dmm_read_probe": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
 }
 

@@ -14,6 +14,7 @@
 #include <hip/hip_runtime.h>
 #include <atomic>
 #include <mutex>
+#include <thread>
 #include <type_traits>
 #include <vector>
 #include <hip/hip_ext.h>
@@ -3124,6 +3125,44 @@ int dispatch_f16(const void *x, const void *codes, const void *grid, float scale
     return run_generic(x, codes, grid, scale, y, M, N, K, s);
 }
 
+// ------------------------------------------------------------------ the operator on host memory
+// The reference's own CPU path is a scalar decode and a triple loop (/root/reference/test_decode_matmul.py:29-71);
+// this is the same thing for the half-precision form, in plain C++ for tensors that live in host
+// memory: no GPU is involved and no GPU call is made.  Not a fallback: device pointers never come
+// here, the entry points below are separate ones.  One rounding per weight (the fp32 sum of a half
+// and +-1/4 is exact), fp32 sums over k in ascending order, rows of W spread over host threads.
+inline void host_decode_row(const uint16_t *codes, const half_t *grid, int64_t kc, half_t *w)
+{
+    for (int64_t j = 0; j < kc; j++) {
+        const uint32_t c = codes[j];
+        const uint32_t idx = c & 0xFFu, s7 = (c >> 8) & 0x7Fu;
+        const uint32_t s8 = s7 | ((uint32_t)(__builtin_popcount(s7) & 1) << 7);
+        const float shift = (c & 0x8000u) ? -0.25f : 0.25f;
+        for (int d = 0; d < 8; d++) {
+            const float g = (float)grid[idx * 8 + d];
+            w[j * 8 + d] = (half_t)(((s8 >> d) & 1u ? -g : g) + shift);
+        }
+    }
+}
+
+template <typename F>
+void host_parallel_rows(int64_t n_rows, int64_t work_per_row, F body)
+{
+    unsigned threads = std::thread::hardware_concurrency();
+    if (threads == 0) threads = 1;
+    if (threads > 16) threads = 16;
+    if (n_rows * work_per_row < (1 << 20) || n_rows < 2) threads = 1;
+    if ((int64_t)threads > n_rows) threads = (unsigned)n_rows;
+    if (threads == 1) {
+        body(0, n_rows);
+        return;
+    }
+    std::vector<std::thread> pool;
+    for (unsigned t = 0; t < threads; t++)
+        pool.emplace_back([=] { body(n_rows * t / threads, n_rows * (t + 1) / threads); });
+    for (auto &th : pool) th.join();
+}
+
 }  // namespace dmm
 
 using namespace dmm;
@@ -3376,6 +3415,42 @@ int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid,
     if (workspace && workspace_bytes > 0 && !aligned(workspace, 16)) return DMM_ERR_MISALIGNED;
     if ((st = ensure_ready((hipStream_t)stream))) return st;
     return dispatch_f16(x, codes, grid, scale, y, M, N, K, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int dmm_decode_host_f16(const void *codes, const void *grid, void *W, int64_t N, int64_t K)
+{
+    if (N < 0 || K < 0 || (K & 7)) return DMM_ERR_BAD_SHAPE;
+    if (N == 0 || K == 0) return DMM_OK;
+    if (!codes || !grid || !W) return DMM_ERR_NULL_POINTER;
+    if (!aligned(codes, 2) || !aligned(grid, 2) || !aligned(W, 2)) return DMM_ERR_MISALIGNED;
+    const int64_t kc = K >> 3;
+    host_parallel_rows(N, K, [=](int64_t n0, int64_t n1) {
+        for (int64_t n = n0; n < n1; n++)
+            host_decode_row((const uint16_t *)codes + n * kc, (const half_t *)grid, kc, (half_t *)W + n * K);
+    });
+    return DMM_OK;
+}
+
+int dmm_decode_matmul_host_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                               int64_t N, int64_t K)
+{
+    const int st = check_common(x, codes, grid, y, M, N, K);
+    if (st != DMM_OK || M == 0 || N == 0) return st;
+    const int64_t kc = K >> 3;
+    const half_t *xh = (const half_t *)x;
+    half_t *yh = (half_t *)y;
+    host_parallel_rows(N, K * (M + 1), [=](int64_t n0, int64_t n1) {
+        std::vector<half_t> w((size_t)K);
+        for (int64_t n = n0; n < n1; n++) {
+            host_decode_row((const uint16_t *)codes + n * kc, (const half_t *)grid, kc, w.data());
+            for (int64_t m = 0; m < M; m++) {
+                float acc = 0.f;
+                for (int64_t k = 0; k < K; k++) acc += (float)xh[m * K + k] * (float)w[(size_t)k];
+                yh[m * N + n] = (half_t)(acc * scale);
+            }
+        }
+    });
+    return DMM_OK;
 }
 
 int dmm_read_probe(const void *codes, void *sink, int64_t N, int64_t K, void *stream)

@@ -35,10 +35,17 @@ void check_status(int st, const char *what)
     TORCH_CHECK(st == DMM_OK, what, " failed: ", dmm_status_string(st), " (status ", st, ")");
 }
 
-void check_codes_grid(const torch::Tensor &codes, const torch::Tensor &grid)
+// allow_cpu: the operator and the decoder also take tensors in host memory (all of them there), which
+// go to the library's host route; every other operation is GPU-only
+void check_codes_grid(const torch::Tensor &codes, const torch::Tensor &grid, bool allow_cpu = false)
 {
-    DMM_CHECK_INPUT(codes);
-    DMM_CHECK_INPUT(grid);
+    if (allow_cpu && codes.is_cpu()) {
+        DMM_CHECK_CONTIGUOUS(codes);
+        DMM_CHECK_CONTIGUOUS(grid);
+    } else {
+        DMM_CHECK_INPUT(codes);
+        DMM_CHECK_INPUT(grid);
+    }
     TORCH_CHECK(is_code_dtype(codes), "codes must be int16 or uint16");
     TORCH_CHECK(grid.scalar_type() == torch::kHalf, "grid must be float16");
     TORCH_CHECK(codes.dim() == 2, "codes must be [N, K/8]");
@@ -51,8 +58,12 @@ enum class Path { kAuto, kGemv, kGemm, kGeneric };
 torch::Tensor run(const torch::Tensor &x, const torch::Tensor &codes, const torch::Tensor &grid,
                   double scale, Path path)
 {
-    DMM_CHECK_INPUT(x);
-    check_codes_grid(codes, grid);
+    if (x.is_cpu()) {
+        DMM_CHECK_CONTIGUOUS(x);
+    } else {
+        DMM_CHECK_INPUT(x);
+    }
+    check_codes_grid(codes, grid, true);
     TORCH_CHECK(x.scalar_type() == torch::kHalf, "x must be float16");
     TORCH_CHECK(x.dim() == 2, "x must be [M, K]");
     TORCH_CHECK(x.device() == codes.device(), "x and codes must be on the same device");
@@ -61,6 +72,21 @@ torch::Tensor run(const torch::Tensor &x, const torch::Tensor &codes, const torc
     const int64_t M = x.size(-2);
     const int64_t N = codes.size(-2);
     const int64_t K = x.size(-1);
+
+    if (x.is_cpu()) {
+        // tensors in host memory: the library's host route (the reference's CPU path,
+        // test_decode_matmul.py:58-71, in the half-precision form); no GPU call is made
+        TORCH_CHECK(path == Path::kAuto, "the named kernel paths are GPU paths; CPU tensors take path 'auto'");
+        torch::Tensor y = torch::empty({M, N}, x.options().requires_grad(false));
+        int st;
+        {
+            pybind11::gil_scoped_release nogil;
+            st = dmm_decode_matmul_host_f16(x.data_ptr(), codes.data_ptr(), grid.data_ptr(), static_cast<float>(scale),
+                                            y.data_ptr(), M, N, K);
+        }
+        check_status(st, "decode_matmul (host)");
+        return y;
+    }
 
     c10::DeviceGuard guard(x.device());
     torch::Tensor y = torch::empty({M, N}, x.options().requires_grad(false));
@@ -110,9 +136,19 @@ torch::Tensor decode_matmul_path(torch::Tensor x, torch::Tensor codes, torch::Te
 
 torch::Tensor decode(torch::Tensor codes, torch::Tensor grid)
 {
-    check_codes_grid(codes, grid);
+    check_codes_grid(codes, grid, true);
     const int64_t N = codes.size(0);
     const int64_t K = codes.size(1) * 8;
+    if (codes.is_cpu()) {   // host memory: the library's host decoder, no GPU call
+        torch::Tensor W = torch::empty({N, K}, grid.options().requires_grad(false));
+        int st;
+        {
+            pybind11::gil_scoped_release nogil;
+            st = dmm_decode_host_f16(codes.data_ptr(), grid.data_ptr(), W.data_ptr(), N, K);
+        }
+        check_status(st, "decode (host)");
+        return W;
+    }
     c10::DeviceGuard guard(codes.device());
     torch::Tensor W = torch::empty({N, K}, grid.options().requires_grad(false));
     hipStream_t stream = c10::hip::getCurrentHIPStream(codes.device().index()).stream();

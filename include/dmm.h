@@ -225,6 +225,17 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K);
  * only timer (/root/reference/test_decode_matmul.py:8-22) brackets the whole call. */
 int dmm_set_kernel_events(void *start_event, void *stop_event);
 
+/* The operator and the decoder on HOST memory (every pointer a host pointer): the counterpart of the
+ * reference's CPU path, its scalar `decode` and its triple-loop matmul
+ * (/root/reference/test_decode_matmul.py:29-71), in the half-precision form.  Plain C++ on the host's
+ * cores, no GPU call; for hosts without a GPU and for checking small cases.  These are separate
+ * entry points, not a fallback: the device entry points never come here, and a device pointer
+ * passed here is dereferenced as host memory.  Same code format, same one rounding per weight,
+ * fp32 sums over k in ascending order, y = half(scale * sum); blocking (returns when y is written). */
+int dmm_decode_host_f16(const void *codes, const void *grid, void *W, int64_t N, int64_t K);
+int dmm_decode_matmul_host_f16(const void *x, const void *codes, const void *grid, float scale,
+                               void *y, int64_t M, int64_t N, int64_t K);
+
 /* Yardstick for benchmarks: a kernel that only READS a row-major code matrix [N, K/8] with the
  * batch-1 kernels' launch shape and access pattern (16 rows x 64 bytes per wave load) and does no
  * decoding; timed with dmm_set_kernel_events like any other call, it shows what the memory system

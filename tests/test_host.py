@@ -116,11 +116,42 @@ def test_operator_rejects_bad_inputs_with_runtime_error():
     codes = torch.zeros(4, 8, dtype=torch.int16)
     grid = torch.zeros(256, 8, dtype=torch.float16)
     with pytest.raises(RuntimeError, match="GPU tensor"):
-        dmm.decode_matmul(x, codes, grid, 1.0)          # CPU tensors: there is no CPU path
+        dmm.pack_codes(torch.zeros(4, 32, dtype=torch.int16))        # the packed and the integer forms are GPU-only
     with pytest.raises(RuntimeError, match="GPU tensor"):
-        dmm.decode(codes, grid)
+        dmm.decode_matmul(torch.zeros(1, 64, dtype=torch.int8), codes, torch.zeros(256, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="CPU tensors take path"):
+        dmm.decode_matmul_path(x, codes, grid, 1.0, "gemv")          # the named kernel paths are GPU paths
     with pytest.raises(RuntimeError):
         dmm.decode_matmul_path(x, codes, grid, 1.0, "nonsense")
+    with pytest.raises(RuntimeError, match="float16"):
+        dmm.decode_matmul(x.float(), codes, grid, 1.0)
+    with pytest.raises(RuntimeError, match="8 \\* codes"):
+        dmm.decode_matmul(x[:, :56].contiguous(), codes, grid, 1.0)
+
+
+def test_config0_operator_on_host_tensors():
+    """configs[0], the CPU-runnable case, through the operator itself: tensors in host memory take the
+    library's host route (plain C++ loops, no GPU call).  W is bit-exact against the oracle, y within the
+    operator's tolerance of the fp32-accumulated product; a ragged shape too, and the C ABI directly."""
+    for M, N, K, seed in ((1, 4096, 4096, 0), (3, 37, 1000, 5), (2, 5, 8, 6)):
+        x, codes, grid, scale = workload.make_inputs(M, N, K, seed=seed)
+        W = dmm.decode(codes, grid)
+        want_W = orc.decode_f16(codes.numpy(), grid.numpy())
+        assert W.device.type == "cpu" and np.array_equal(W.numpy().view(np.uint16), want_W.view(np.uint16))
+        y = dmm.decode_matmul(x, codes, grid, scale)
+        assert y.dtype == torch.float16 and tuple(y.shape) == (M, N) and y.device.type == "cpu"
+        ref = orc.matmul_f32(x.numpy(), want_W, scale)
+        got = y.float().numpy()
+        assert np.all(np.abs(got - ref) <= 1e-2 + 1e-2 * np.abs(ref))
+    lib = capi.lib()
+    x, codes, grid, scale = workload.make_inputs(2, 16, 64, seed=7)
+    y = torch.full((2, 16), float("nan"), dtype=torch.float16)
+    assert lib.dmm_decode_matmul_host_f16(x.data_ptr(), codes.data_ptr(), grid.data_ptr(), scale, y.data_ptr(), 2, 16, 64) == 0
+    assert torch.equal(y, dmm.decode_matmul(x, codes, grid, scale))
+    assert lib.dmm_decode_matmul_host_f16(x.data_ptr(), codes.data_ptr(), grid.data_ptr(), scale, y.data_ptr(), 2, 16, 60) == -2
+    # empty sum and empty outputs
+    e = dmm.decode_matmul(torch.zeros(2, 0, dtype=torch.float16), torch.zeros(3, 0, dtype=torch.int16), grid, 1.0)
+    assert tuple(e.shape) == (2, 3) and torch.all(e == 0)
 
 
 def test_codebook_matches_oracle_and_reference_properties():
