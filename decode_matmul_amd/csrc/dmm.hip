@@ -1090,13 +1090,17 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
         const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_tiles_all * 16 : N) * row_bytes), 0x00020000);
     const int voff = kPacked ? lane * 16 : c16 * row_bytes + q * 16;
     constexpr int kOut = (int)0x80000000;
-    // the code word of (group g, chunk c, tile t of the group) for this wave; out of range: zeros, no access
-    auto issue = [&](u4_t &cwd, int g, int c, int t) {
-        const int gt0 = t0 + g * g_base + (g < g_rem ? g : g_rem), gn = g_base + (g < g_rem ? 1 : 0);
-        const int tile = gt0 + t, step = c * W + wave;
-        const bool ok = g < n_groups && t < gn && step < n_steps;
-        const int soff = !ok ? kOut : kPacked ? (tile * n_steps + step) * 1024 : tile * 16 * row_bytes + step * 64;
-        cwd = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, soff, 0);
+    // Scalar byte offset of the code word of (group g, chunk c, tile 0 of the group) for this wave, or the
+    // out-of-range offset when the group or the wave's step of the chunk does not exist; tile t of the
+    // group lies t * tile_stride further on.  Out of range: zeros, no memory access.
+    const int tile_stride = kPacked ? n_steps * 1024 : 16 * row_bytes;
+    auto chunk_offset = [&](int g, int c, int &gn) {
+        const int gt0 = t0 + g * g_base + (g < g_rem ? g : g_rem), step = c * W + wave;
+        gn = g < n_groups && step < n_steps ? g_base + (g < g_rem ? 1 : 0) : 0;
+        return kPacked ? (gt0 * n_steps + step) * 1024 : gt0 * tile_stride + step * 64;
+    };
+    auto issue = [&](u4_t &cwd, int base, int gn, int t) {
+        cwd = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, t < gn ? base + t * tile_stride : kOut, 0);
     };
     // the ring: DC chunks deep, one slot per tile of the group
     u4_t cw[DC][T];
@@ -1104,8 +1108,10 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
         int g = 0, c = 0;
 #pragma unroll
         for (int d = 0; d < DC; d++) {
+            int gn;
+            const int base = chunk_offset(g, c, gn);
 #pragma unroll
-            for (int t = 0; t < T; t++) issue(cw[d][t], g, c, t);
+            for (int t = 0; t < T; t++) issue(cw[d][t], base, gn, t);
             if (++c == n_chunks) { c = 0; g++; }
         }
     }
@@ -1180,7 +1186,7 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
     // steps that do not exist load nothing and get zeros), so the wait counters stay exact.
     auto chunk = [&](auto slot_tag, int gc) {
         constexpr int kSlot = decltype(slot_tag)::value;
-        const bool exists = gc < total;
+        const bool exists = DC == 1 || gc < total;   // only a second chunk of an unrolled pair may lie past the end
         const int gn = g_base + (g < g_rem ? 1 : 0);
         const int ntg = exists ? gn : 0;                          // tiles of this group (uniform)
         const bool last_c = c + 1 == n_chunks;
@@ -1196,6 +1202,8 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
             xpiece = p < n_pieces ? reinterpret_cast<const u4_t *>(x)[p] : u4_t{0u, 0u, 0u, 0u};
         }
         const bool step_ok = exists && c * W + wave < n_steps;
+        int p_gn;                                                 // the refills: chunk DC further on
+        const int p_base = chunk_offset(pg, pc, p_gn);
         u4_t x0 = u4_t{0u, 0u, 0u, 0u}, x1 = x0;
         if (step_ok) {
             const uint32_t xa = xlane + (uint32_t)(xb_cur * kQcXBuf);
@@ -1205,15 +1213,13 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
         const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
 #pragma unroll
         for (int t = 0; t < T; t++) {
-            const bool live = step_ok && t < ntg;   // uniform
-            Q8Gather gt[4];
-            u4_t a8 = u4_t{0u, 0u, 0u, 0u};
-            if (live) {
+            if (step_ok && t < ntg) {   // uniform
+                Q8Gather gt[4];
 #pragma unroll
                 for (int t2 = 0; t2 < 4; t2++) q8_gather(gt[t2], cw[kSlot][t][t2], lane_base);
-                a8 = (cw[kSlot][t] & 0x80008000u) | 0x40004000u;   // +-2.0 per code: the shift term's A operand
-            }
-            if (live) {
+                u4_t a8;   // +-2.0 per code, the shift term's A operand: the code words' shift bits over the bits of 2.0
+#pragma unroll
+                for (int i = 0; i < 4; i++) a8[i] = bfi(0x80008000u, cw[kSlot][t][i], 0x40004000u);
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     const Q8Gather &b0 = gt[2 * h], &b1 = gt[2 * h + 1];
@@ -1224,7 +1230,7 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
                 }
                 accd[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8_t, a8), __builtin_bit_cast(h8_t, x0), accd[t], 0, 0, 0);
             }
-            issue(cw[kSlot][t], pg, pc, t);                        // the slot's next code word
+            issue(cw[kSlot][t], p_base, p_gn, t);                  // the slot's next code word
         }
         if (stager && !stage_piece(xpiece, resident ? nc : (gc + 1) & 1, sp)) flags[0] = 1u;
         if (!exists) return;
