@@ -451,12 +451,17 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
     // LDS copy of x are built while the code loads fly ---------------------------------------
     const u4_t grow = tid < 256 ? reinterpret_cast<const u4_t *>(grid)[tid] : u4_t{0u, 0u, 0u, 0u};   // waves 0-3 stage the grid
     const int row_chunks = K >> 3;                     // 16-byte pieces per row of x
-    constexpr int kXPer = 4;                           // pieces of row 0 per thread fetched up front
+    const int n_pieces = M * row_chunks;               // x is [M][K] contiguous: piece p sits at x + 16 p
+    // pieces of x per thread fetched up front, before the code loads are queued: vector-memory results
+    // return in order, so a piece asked for later arrives behind the whole first burst of codes.  One
+    // row of x: up to four pieces (all of it for K <= 32768); more rows: up to six (all of x for M <= 4 at
+    // K = 11008).
+    constexpr int kXPer = 6, kXPer1 = 4;
     u4_t xv[kXPer];
 #pragma unroll
     for (int u = 0; u < kXPer; u++) {
-        const int c = u * 64 * W + tid;
-        xv[u] = c < row_chunks ? reinterpret_cast<const u4_t *>(x)[c] : u4_t{0u, 0u, 0u, 0u};
+        const int p = u * 64 * W + tid;
+        xv[u] = p < n_pieces && (u < kXPer1 || M > 1) ? reinterpret_cast<const u4_t *>(x)[p] : u4_t{0u, 0u, 0u, 0u};
     }
 
     const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;   // k steps of this wave per row block
@@ -500,17 +505,29 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x,
     stream_stage_signs<64 * W>(smem_raw, tid);
     __builtin_amdgcn_sched_barrier(0);   // keep the sign rows ahead of the waits for the loads
 
-    // x -> LDS (padded pitch): the pieces of row 0 fetched above, then whatever is left
+    // x -> LDS (row m at m * x_pitch): the pieces fetched above, then whatever is left
+    if (M == 1) {
 #pragma unroll
-    for (int u = 0; u < kXPer; u++) {
-        const int c = u * 64 * W + tid;
-        if (c < row_chunks) reinterpret_cast<u4_t *>(xs)[c] = xv[u];
+        for (int u = 0; u < kXPer1; u++) {
+            const int c = u * 64 * W + tid;
+            if (c < row_chunks) reinterpret_cast<u4_t *>(xs)[c] = xv[u];
+        }
+        for (int c = kXPer1 * 64 * W + tid; c < row_chunks; c += 64 * W)
+            reinterpret_cast<u4_t *>(xs)[c] = reinterpret_cast<const u4_t *>(x)[c];
+    } else {
+        int m = 0, c = tid;   // piece p = m * row_chunks + c
+#pragma unroll
+        for (int u = 0; u < kXPer; u++) {
+            while (c >= row_chunks) { c -= row_chunks; m++; }
+            if (m < M) reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = xv[u];
+            c += 64 * W;
+        }
+        for (int p = kXPer * 64 * W + tid; p < n_pieces; p += 64 * W) {
+            while (c >= row_chunks) { c -= row_chunks; m++; }
+            reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = reinterpret_cast<const u4_t *>(x)[p];
+            c += 64 * W;
+        }
     }
-    for (int c = kXPer * 64 * W + tid; c < row_chunks; c += 64 * W)
-        reinterpret_cast<u4_t *>(xs)[c] = reinterpret_cast<const u4_t *>(x)[c];
-    for (int m = 1; m < M; m++)
-        for (int c = tid; c < row_chunks; c += 64 * W)
-            reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = reinterpret_cast<const u4_t *>(x + (int64_t)m * K)[c];
     if (tid >= 64 * W - 8) reinterpret_cast<u4_t *>(xs + M * x_pitch)[tid - (64 * W - 8)] = u4_t{0u, 0u, 0u, 0u};
     stream_stage_grid<64 * W>(smem_raw, grow, tid);
     __syncthreads();
