@@ -46,6 +46,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--repeats", type=int, default=5,
                     help="how many times the region of exactly --steps steps is timed; the median region is reported")
+    ap.add_argument("--preheat-ms", type=float, default=200.0,
+                    help="untimed replays of the step for this long before the warmup steps: the device takes some "
+                         "15 ms of work to leave its idle clocks, more than a short --warmup covers")
     ap.add_argument("--quick", action="store_true", help="skip prefill / small-batch / CPU legs")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
     ap.add_argument("--graph-steps", type=int, default=12,
@@ -135,9 +138,9 @@ def main():
     # layers of these four projections at this size), not one of four: with a graph per step the
     # GPU sat idle for about 15 us between replays, a fifth of the step, and with four ctypes
     # calls per 56 us step the eager loop sits close to being bound by the host.
-    def timed_steps(tag):
-        """Wall time of exactly args.steps steps, `--repeats` times over (each region bracketed by
-        synchronisation; the median region is reported), with the kernel choice as it stands."""
+    def prepare_steps():
+        """A function that runs exactly n steps with the kernel choice as it stands now (the choice
+        is made when a launch is captured), and how it launches them."""
         def run_steps(n):
             for i in range(n):
                 step(i)
@@ -146,24 +149,18 @@ def main():
             try:
                 chunk = max(copies, args.graph_steps // copies * copies)   # whole turns of the buffer sets
                 graphs = {}
-
-                def graph_of(n):                 # n consecutive steps, starting on buffer set 0
-                    if n not in graphs:
-                        g = torch.cuda.CUDAGraph()
-                        with torch.cuda.graph(g):
-                            cap = torch.cuda.current_stream().cuda_stream
-                            for i in range(n):
-                                for p in probs:
-                                    st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][i % copies].data_ptr(),
-                                                                   p["grid"].data_ptr(), p["scale"], p["y"].data_ptr(),
-                                                                   1, p["N"], p["K"], cap)
-                                    if st != 0:
-                                        raise capi.DmmError("dmm_decode_matmul_f16", st)
-                        graphs[n] = g
-                    return graphs[n]
-
                 for n in {chunk, args.steps % chunk, args.warmup % chunk} - {0}:
-                    graph_of(n)
+                    g = torch.cuda.CUDAGraph()       # n consecutive steps, starting on buffer set 0
+                    with torch.cuda.graph(g):
+                        cap = torch.cuda.current_stream().cuda_stream
+                        for i in range(n):
+                            for p in probs:
+                                st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][i % copies].data_ptr(),
+                                                               p["grid"].data_ptr(), p["scale"], p["y"].data_ptr(),
+                                                               1, p["N"], p["K"], cap)
+                                if st != 0:
+                                    raise capi.DmmError("dmm_decode_matmul_f16", st)
+                    graphs[n] = g
 
                 def run_steps(n):                # exactly n steps: whole chunks, then the rest
                     for _ in range(n // chunk):
@@ -173,27 +170,51 @@ def main():
                 mode = "hip graph, %d steps (%d launches) per replay" % (chunk, chunk * len(probs))
             except Exception as e:   # capture unavailable: time the eager loop
                 print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
-        run_steps(args.warmup)
-        torch.cuda.synchronize()
-        regions = []
-        for _ in range(max(1, args.repeats)):
-            t0 = time.perf_counter()
-            run_steps(args.steps)
-            torch.cuda.synchronize()
-            regions.append(time.perf_counter() - t0)
-        return sorted(regions)[len(regions) // 2], regions, mode
+        return run_steps, mode
 
-    wall, regions, launch_mode = timed_steps("operator's choice")
-    ms_per_step = wall * 1e3 / args.steps
-    value = step_bytes * args.steps / wall / 1e9
-    # the same steps with the 8-bit kernels switched off: every launch in 16-bit arithmetic (half x half
-    # products, fp32 sums), the arithmetic the operator's definition states
+    def timed_region(run_steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps(args.steps)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    # the operator's own kernel choice, and the same steps with the 8-bit kernels switched off: every
+    # launch in 16-bit arithmetic (half x half products, fp32 sums), the arithmetic the operator's
+    # definition states.  Each is timed over exactly args.steps steps, `--repeats` times, the regions
+    # of the two taking turns so that a drift of the clocks meets both alike; the median region counts.
+    run_auto, launch_mode = prepare_steps()
     was = lib.dmm_set_gemv_8bit(0)
     try:
-        wall16, _, _ = timed_steps("16-bit kernels only")
+        run_f16, _ = prepare_steps()
         names16 = sorted({lib.dmm_gemv_kernel_name(1, N, K).decode() for K, N in shapes})
+        if args.no_graph:
+            run_f16 = None               # eager launches choose as they run: timed below, switched off
     finally:
         lib.dmm_set_gemv_8bit(was)
+    t_heat = time.perf_counter()
+    while (time.perf_counter() - t_heat) * 1e3 < args.preheat_ms:
+        run_auto(12)
+        torch.cuda.synchronize()
+    run_auto(args.warmup)
+    if run_f16:
+        run_f16(args.warmup)
+    regions, regions16 = [], []
+    for _ in range(max(1, args.repeats)):
+        regions.append(timed_region(run_auto))
+        if run_f16:
+            regions16.append(timed_region(run_f16))
+    if not run_f16:
+        was = lib.dmm_set_gemv_8bit(0)
+        try:
+            run_auto(args.warmup)
+            regions16 = [timed_region(run_auto) for _ in range(max(1, args.repeats))]
+        finally:
+            lib.dmm_set_gemv_8bit(was)
+    wall = sorted(regions)[len(regions) // 2]
+    wall16 = sorted(regions16)[len(regions16) // 2]
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes * args.steps / wall / 1e9
     value_f16_only = step_bytes * args.steps / wall16 / 1e9
 
     # same region again with the kernel's own begin/end events
@@ -256,10 +277,11 @@ def main():
         "ms_per_step_f16_only": round(wall16 * 1e3 / args.steps, 5),
         "kernels_f16_only": names16,
         "timed_regions_ms": [round(r * 1e3, 4) for r in regions],
+        "timed_regions_ms_f16_only": [round(r * 1e3, 4) for r in regions16],
         "data": "synthetic",
         "config": {"workload": "configs[2]: batch-1 decode-GEMV, 8192->10240, 8192->8192, 8192->28672, 28672->8192",
                    "M": 1, "code_buffers_rotated": copies, "distinct_code_MB": round(copies * step_bytes / 1e6, 1),
-                   "step": "4 GEMVs, one per shape", "launch": launch_mode},
+                   "step": "4 GEMVs, one per shape", "launch": launch_mode, "preheat_ms": args.preheat_ms},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
@@ -308,12 +330,17 @@ def timed_kernel(torch, lib, fn, reps):
 def hbm_read_probe(torch, lib, probs, copies, stream, steps):
     """What a kernel that only reads gets out of the memory system at the headline shapes: the
     library's read probe (same launch shape and access pattern as the batch-1 kernels, no decode)
-    over the same rotating code buffers, the four shapes taking turns, durations by events."""
-    sink = torch.zeros(16, dtype=torch.int32, device=probs[0]["x"].device)
+    over the same rotating code buffers, the four shapes taking turns.  Per shape the kernel's own
+    duration by events; `step_us` is the wall time per step of the four probes replayed as the
+    same kind of HIP graph the headline is timed with (so it holds the gaps between dependent
+    launches too), and `launch_us_empty` the wall time per launch of that graph when each probe has a
+    single row tile to read, i.e. what a launch costs before it moves any data."""
+    dev = probs[0]["x"].device
+    sink = torch.zeros(16, dtype=torch.int32, device=dev)
 
-    def fn(k, i):
+    def fn(k, i, s=stream):
         p = probs[k]
-        st = lib.dmm_read_probe(p["codes"][i % copies].data_ptr(), sink.data_ptr(), p["N"], p["K"], stream)
+        st = lib.dmm_read_probe(p["codes"][i % copies].data_ptr(), sink.data_ptr(), p["N"], p["K"], s)
         assert st == 0, st
     for i in range(3):
         for k in range(len(probs)):
@@ -338,7 +365,43 @@ def hbm_read_probe(torch, lib, probs, copies, stream, steps):
         b = p["N"] * p["K"] // 4
         rows.append({"K": p["K"], "N": p["N"], "code_bytes": b, "kernel_us": round(t * 1e6, 3),
                      "GBps": round(b / t / 1e9, 1), "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBS, 4)})
-    return {"kernel": "dmm::read_probe_kernel", "shapes": rows}
+    out = {"kernel": "dmm::read_probe_kernel", "shapes": rows}
+
+    graph_steps = max(copies, 12 // copies * copies)
+
+    def graph_us(empty):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            cap = torch.cuda.current_stream().cuda_stream
+            for i in range(graph_steps):
+                for k, p in enumerate(probs):
+                    if empty:
+                        st = lib.dmm_read_probe(p["codes"][i % copies].data_ptr(), sink.data_ptr(), 16, p["K"], cap)
+                        assert st == 0, st
+                    else:
+                        fn(k, i, cap)
+        for _ in range(10):
+            g.replay()
+        torch.cuda.synchronize()
+        t = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for _ in range(8):
+                g.replay()
+            torch.cuda.synchronize()
+            t.append((time.perf_counter() - t0) / (8 * graph_steps))
+        return sorted(t)[2] * 1e6
+    try:
+        step_us = graph_us(False)
+        step_bytes = sum(p["N"] * p["K"] // 4 for p in probs)
+        out["step_us"] = round(step_us, 3)
+        out["step_GBps"] = round(step_bytes / step_us / 1e3, 1)
+        out["step_frac_hbm"] = round(step_bytes / step_us / 1e3 / HBM_PEAK_GBS, 4)
+        out["launch_us_empty"] = round(graph_us(True) / len(probs), 3)
+        out["launch"] = "hip graph, %d steps (%d launches) per replay" % (graph_steps, graph_steps * len(probs))
+    except Exception as e:
+        print("bench.py: read-probe graph failed (%s)" % e, file=sys.stderr)
+    return out
 
 
 def gemv_7b_step(torch, lib, capi, workload, dev, rand_codes):
