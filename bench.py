@@ -5,11 +5,21 @@ Headline (the JSON line's `value`): batch-1 decode-GEMV at the Llama-2-70B proje
 shapes.  One step = the four GEMVs (8192->10240, 8192->8192, 8192->28672, 28672->8192), each
 on the next of several distinct code buffers so that the 256 MB Infinity Cache cannot serve
 the weights; `value` is code bytes (N*K/4 per GEMV) per second over the timed region, inputs
-resident in HBM.  `roofline` is the GEMV kernel that carries most of the step's bytes, alone:
-code bytes per launch over the kernel's own duration (HIP events placed around the kernel by
-the library's timing hook) against 8 TB/s; `all_gemv_launches` is the same figure over every
-launch of the step, per kernel.  `prefill` and `small_batch` carry the M=2048 and M=4..32 figures;
-`cpu_baseline` is the torch CPU path on the host cores on one 8192x8192 GEMV.
+resident in HBM.  The region of exactly --steps steps is timed --repeats times (HIP graph replays
+of 12 steps each, bracketed by synchronisation) and the median region counts; `value_f16_only` is
+the same with the 8-bit kernels switched off, its regions taking turns with the headline's.
+Before the --warmup steps the step is replayed for --preheat-ms (200 ms): the device needs some
+15 ms of work to leave its idle clocks.
+
+`roofline` is the GEMV kernel that carries most of the step's bytes, alone: code bytes per
+launch over the kernel's own duration (HIP events placed around the kernel by the library's
+timing hook, on the stream it is launched on) against 8 TB/s; `all_gemv_launches` is the same
+figure over every launch of the step, per kernel.  `hbm_read_probe` is what a kernel that only
+reads the same code buffers reaches (per shape, as a graph step, and per launch with nothing
+to read): the memory system's and the launch path's share of the step.  `gemv_7b_step` is a
+Llama-2-7B layer's four projections as one graph, gate and up as one call on concatenated code
+rows.  `prefill`, `small_batch` and `integer_operator` carry the M=2048, M=4..32 and int8
+figures; `cpu_baseline` is the torch CPU path on the host cores on one 8192x8192 GEMV.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
 """
@@ -26,17 +36,14 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8, published
-# HBM bytes one GEMV launch moves, per kernel, averaged over the shapes of the step that kernel
-# serves: rocprofv3 FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter
-# reads for a plain 256 MiB device copy (x2.000 and x1.000).
-# gemv_stream_kernel (three of the step's launches): 15,891.7 KiB fetched, 19.8 KiB written per
-# dispatch (32,156,331 code bytes); gemv_q8_kernel (8192 -> 28672): 28,829.0 KiB and 56.7 KiB
-# (58,720,256 code bytes).
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_stream_kernel": 32565000, "dmm::gemv_q8_kernel": 59095000}
-GEMV_TRAFFIC_SOURCE = {"dmm::gemv_stream_kernel": "profiles/gemv_stream_kernel_llama70b_batch1.md (rocprofv3 --pmc, an earlier run; "
-                                                  "not measured by this run)",
-                       "dmm::gemv_q8_kernel": "profiles/gemv_q8_kernel_llama70b_batch1.md (rocprofv3 --pmc, an earlier run; not "
-                                              "measured by this run)"}
+# HBM bytes one GEMV launch moves, per kernel, averaged over the four shapes of the step: rocprofv3
+# FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain
+# 256 MiB device copy (x2.000 and x1.000).  Both kernels move 39.2 MB per launch on average against
+# 38,855,680 algorithmic bytes (codes, x, grid, y): 1.009 of them.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8c_kernel": 39198889, "dmm::gemv_stream_kernel": 39188778}
+GEMV_TRAFFIC_SOURCE = {k: "constant from an earlier rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command, summarised in "
+                          "profiles/gemv_kernels_llama70b_batch1.md; not measured by this run (a counter run cannot share a "
+                          "process with the timed one)" for k in GEMV_TRAFFIC_BYTES_PER_LAUNCH}
 
 
 def parse():
@@ -269,7 +276,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
-        "dtype_note": "x, grid, y and the decoded weights are halves, sums fp32; launches of three or more row tiles "
+        "dtype_note": "x, grid, y and the decoded weights are halves, sums fp32; launches of two or more row tiles "
                       "per compute unit multiply fp8 weights (exact for this grid) by x split into four bf8 terms "
                       "(exact) on the 8-bit matrix unit; value_f16_only is the same step with every launch on "
                       "half x half products",

@@ -126,25 +126,27 @@ int dmm_decode_matmul_noalloc_f16(const void *x, const void *codes, const void *
  *                    DPP wave reduction.  The catch-all. */
 int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale,
                  void *y, int64_t M, int64_t N, int64_t K, void *stream);
-/*   dmm_gemv_8bit_f16  the matrix-vector kernel on 8-bit MFMA operands, which dmm_gemv_f16 and
- *                    the operator pick for M <= 4 on launches of more than three 16-row tiles
- *                    per compute unit (shorter ones gain nothing from it).  Weights as fp8
- *                    (e4m3) bytes - exact when every grid value has at most 4 significant bits
- *                    in fp8's range, as the E8P grid does - and x
- *                    as four bf8 (e5m2) terms that add up to it exactly; the +-1/4 shift of a
- *                    code is added through the per-code means of x (two halves, hi + lo, times
- *                    +-2 in a 16-bit MFMA of their own).  Nothing is lost in the operands;
- *                    the 8-bit MFMA aligns the products of a group to the largest of them, so y
- *                    is not always the 16-bit kernel's bit for bit: 98 % of the outputs
- *                    are the correctly rounded ones and the rest are one half ulp off (99th
- *                    percentile of the error 0.57 ulps; the tolerance of the operator is 1e-2,
- *                    thousands of ulps).  A grid that does not fit fp8, or an x
- *                    that is not finite, is detected inside the launch and served by the 16-bit
- *                    kernel: same call, same status.  dmm_set_gemv_8bit(0), or DMM_GEMV_8BIT=0
- *                    in the environment, keeps the operator off this kernel.  Domain: that of
- *                    dmm_gemv_f16 with M <= 4 and the terms of x and of its means fitting the
- *                    LDS beside the tables and the partial sums (4 M (K + 16) + 2 M (K / 4 + 16)
- *                    bytes: K <= 12544 at M = 1); DMM_ERR_UNSUPPORTED
+/*   dmm_gemv_8bit_f16  the matrix-vector kernels on 8-bit MFMA operands, which dmm_gemv_f16 and
+ *                    the operator pick for M = 1 on launches of two or more 16-row tiles per
+ *                    compute unit and for M = 2 .. 4 on launches of more than three (shorter
+ *                    ones gain nothing from them).  Weights as fp8 (e4m3) bytes - exact when
+ *                    every grid value has at most 4 significant bits in fp8's range, as the E8P
+ *                    grid does - and x as four bf8 (e5m2) terms that add up to it exactly; the
+ *                    +-1/4 shift of a code is added through the per-code means of x (two halves,
+ *                    hi + lo, times +-2 in a 16-bit MFMA of their own).  Nothing is lost in the
+ *                    operands; the 8-bit MFMA aligns the products of a group to the largest of
+ *                    them, so y is not always the 16-bit kernel's bit for bit: 98 % of the
+ *                    outputs are the correctly rounded ones and the rest are one half ulp off
+ *                    (99th percentile of the error 0.57 ulps; the tolerance of the operator is
+ *                    1e-2, thousands of ulps).  A grid that does not fit fp8, or an x that is not
+ *                    finite, is detected inside the launch and served by the 16-bit kernel: same
+ *                    call, same status.  dmm_set_gemv_8bit(0), or DMM_GEMV_8BIT=0 in the
+ *                    environment, keeps the operator off these kernels.  Domain: that of
+ *                    dmm_gemv_f16 with M <= 4; at M = 1 the terms of x go through the LDS 4096
+ *                    values at a time, so K is only limited by the 16-bit kernel the launch may
+ *                    hand over to (K <= 31488); at M = 2 .. 4 the terms of x and of its means have
+ *                    to fit the LDS beside the tables and the partial sums (4 M (K + 16) +
+ *                    2 M (K / 4 + 16) bytes: K <= 6656 / 4352 / 3072).  DMM_ERR_UNSUPPORTED
  *                    outside.  No counterpart in the reference (its kernel multiplies int8 by
  *                    int8). */
 int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float scale,
@@ -156,8 +158,9 @@ int dmm_gemv_8bit_f16(const void *x, const void *codes, const void *grid, float 
  * for calls made after it returns.  No counterpart in the reference. */
 int dmm_set_gemv_8bit(int enabled);
 /* Which matrix-vector kernel the operator runs for a shape with aligned pointers, as a profiler's
- * kernel trace names it without the template arguments ("dmm::gemv_q8_kernel",
- * "dmm::gemv_stream_kernel", "dmm::gemv_regx_kernel"; "" outside dmm_gemv_f16's domain).  For
+ * kernel trace names it without the template arguments ("dmm::gemv_q8c_kernel" - one row of x on
+ * 8-bit operands -, "dmm::gemv_q8_kernel", "dmm::gemv_stream_kernel", "dmm::gemv_regx_kernel"; ""
+ * outside dmm_gemv_f16's domain).  For
  * benchmarks that report per kernel.  Static storage.  No counterpart in the reference. */
 const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K);
 int dmm_gemm_f16(const void *x, const void *codes, const void *grid, float scale,
