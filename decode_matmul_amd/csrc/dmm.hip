@@ -1809,12 +1809,18 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_pad : N) * row_bytes), 0x00020000);
     const __amdgpu_buffer_rsrc_t xrsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, (int)((int64_t)M * K * 2), 0x00020000);
+    // Row-major codes travel four k tiles at a time: lane (row, half kq) loads the 32 bytes of its row that
+    // hold tiles 4 j + 2 kq and 4 j + 2 kq + 1 whole, so the two lanes of a row take 64 consecutive bytes
+    // (half a cache line per visit, not 16 bytes of it), and one v_permlane32_swap per word hands lanes
+    // l and l + 32 the halves they need of each other's tiles.  Tiles past the end of the block's share read
+    // whatever follows in the row (zeros past the end of the matrix); their x is zero, so they add nothing.
+    constexpr bool kWide = !kPacked;
     int cvoff[kGrTN];
 #pragma unroll
     for (int i = 0; i < kGrTN; i++) {
         const int n = n0 + wave * 64 + i * 32 + l32;
         if (kPacked) cvoff[i] = n < n_pad ? (n >> 4) * (K >> 8) * 1024 + (n & 15) * 16 + kq * 8 : kOut;
-        else cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
+        else cvoff[i] = n < N ? n * row_bytes + kq * 32 : kOut;
     }
     // rows r and r + 8 share a group of 16 lanes: with the 144-byte pitch their 16 pieces fall in
     // 16 different bank groups, so the LDS writes below are conflict-free like the fragment reads
@@ -1830,17 +1836,41 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
         u2_t cw[kGrTN];
         u4_t xv[TM];
     };
-    auto load_codes = [&](Stage &st, int kt) {   // kt counts this block's tiles
-        const int coff = kt < k_tiles ? (kt_lo + kt) * (kPacked ? 256 : 16) : kOut;
+    auto load_codes = [&](Stage &st, int kt) {   // kt counts this block's tiles (packed codes: one tile at a time)
+        const int coff = kt < k_tiles ? (kt_lo + kt) * 256 : kOut;
 #pragma unroll
         for (int i = 0; i < kGrTN; i++) st.cw[i] = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
+    };
+    // the codes of four tiles (row-major codes): w[row tile][h] holds, once swapped, tile h of the four in
+    // words 0 and 1 and tile h + 2 in words 2 and 3
+    struct CodeTrip {
+        u4_t w[kGrTN][2];
+    };
+    auto load_trip = [&](CodeTrip &ct, int kt) {   // kt: the first of the four tiles, counted within the block
+        const int coff = kt < k_tiles ? (kt_lo + kt) * 16 : kOut;
+#pragma unroll
+        for (int i = 0; i < kGrTN; i++)
+#pragma unroll
+            for (int h = 0; h < 2; h++) ct.w[i][h] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, cvoff[i] + 16 * h, coff, 0);
+    };
+    auto swap_trip = [&](CodeTrip &ct) {
+#pragma unroll
+        for (int i = 0; i < kGrTN; i++)
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int w = 0; w < 2; w++) {
+                    const u2_t r = __builtin_amdgcn_permlane32_swap(ct.w[i][h][w], ct.w[i][h][w + 2], false, false);
+                    ct.w[i][h][w] = r[0];
+                    ct.w[i][h][w + 2] = r[1];
+                }
     };
     auto load_x = [&](Stage &st, int kt, int p) {
         const int xoff = kt < k_tiles ? (kt_lo + kt) * 128 : kOut;
         st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
     };
     auto load_tile = [&](Stage &st, int kt) {
-        load_codes(st, kt);
+        if constexpr (!kWide) load_codes(st, kt);
 #pragma unroll
         for (int p = 0; p < TM; p++) load_x(st, kt, p);
     };
@@ -1849,6 +1879,8 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     const uint32_t xs_r = lds_addr(xs) + (uint32_t)(l32 * kGrLd + kq * 32) * 2u;             // this lane's B fragments
     constexpr uint32_t kXBuf = kBM * kGrLd * 2;
 
+    CodeTrip cur, nxt;   // row-major codes: the four tiles being decoded and the four after them
+    if constexpr (kWide) load_trip(nxt, 0);
     Stage ring[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) load_tile(ring[i], i);
@@ -1871,8 +1903,10 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     // rows of its unit and finishes (packed FMAs) the unit gathered one step earlier, so no
     // step waits for its own gathers.
     StreamGather g[2];
-    auto unit_gather = [&](StreamGather &o, const Stage &st, int u) {
-        stream_gather(o, st.cw[u & 1][u >> 1], lane_base, quarter_bits);
+    // unit u of tile kI of the four in `ct` (row-major codes) or of the tile in `st` (packed codes)
+    auto unit_gather = [&](StreamGather &o, const Stage &st, const CodeTrip &ct, int kI, int u) {
+        const uint32_t cwd = kWide ? ct.w[u & 1][kI & 1][2 * (kI >> 1) + (u >> 1)] : st.cw[u & 1][u >> 1];
+        stream_gather(o, cwd, lane_base, quarter_bits);
     };
     auto unit_finish = [&](const StreamGather &o, int abuf, int u) {
         afr[abuf][u & 1][2 * (u >> 1)] = __builtin_bit_cast(u4_t, gemm_finish<false>(o.g0, o.s0, o.dd));
@@ -1880,10 +1914,15 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     };
 
     __syncthreads();   // tables ready
+    if constexpr (kWide) swap_trip(nxt);
 #pragma unroll
     for (int u = 0; u < 4; u++) {
-        unit_gather(g[u & 1], ring[0], u);
+        unit_gather(g[u & 1], ring[0], nxt, 0, u);
         if (u < 3) unit_finish(g[u & 1], 0, u);   // unit 3 is finished by the first step of the loop
+    }
+    if constexpr (kWide) {
+        cur = nxt;
+        load_trip(nxt, 4);
     }
 #pragma unroll
     for (int p = 0; p < TM; p++) x_store(ring[0], 0, p);
@@ -1893,6 +1932,8 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
 #pragma unroll
         for (int j = 0; j < TM; j++) b[j] = lds_read16(xs_r + buf * kXBuf + (uint32_t)(j * 32 * kGrLd * 2 + s * 16));
     };
+    u4_t b[2][TM];   // the x fragments of the current and the next MFMA step
+    read_b(b[0], 0, 0);
     // MFMAs of tile kt (A = afr[buf], B from x buffer buf) while tile kt+1 (registers sn) is
     // decoded into afr[buf ^ 1] and its x written to buffer buf ^ 1, and tile kt+4 is fetched
     // into sf.  Past the last tile sn holds zeros (out-of-range loads): decoding and storing
@@ -1902,13 +1943,16 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     constexpr int kMfma = kGrTN * TM;                       // MFMAs per k step
     constexpr int kDsPer = (TM + 4 + kMfma - 1) / kMfma;    // LDS reads per MFMA group
     constexpr int kValuPer = (24 + kMfma - 1) / kMfma;      // VALU per MFMA group
-    auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf) {
-        u4_t b[2][TM];
-        read_b(b[0], buf, 0);
+    // kNext (row-major codes): which of its four tiles tile kt+1 is; 0 = the first of the four after
+    // the current ones, which then become the current ones while the loads of the four after them start
+    auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf, auto next_tag) {
+        constexpr int kNext = decltype(next_tag)::value;
+        if constexpr (kWide && kNext == 0) swap_trip(nxt);
+        const CodeTrip &ct = kNext == 0 ? nxt : cur;
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             // the global loads of tile kt+4 spread over the steps, woven between the MFMAs too
-            if (s == 0) load_codes(sf, kt + 4);
+            if (!kWide && s == 0) load_codes(sf, kt + 4);
             if (TM == 4 && (s == 1 || s == 2)) {
                 load_x(sf, kt + 4, 2 * s - 2);
                 load_x(sf, kt + 4, 2 * s - 1);
@@ -1916,26 +1960,46 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
             if (TM < 4 && s >= 1 && s <= TM) load_x(sf, kt + 4, s - 1);
             // unit 3 of the CURRENT tile was gathered in the last step of the previous tile
             unit_finish(g[(s + 1) & 1], s == 0 ? buf : buf ^ 1, (s + 3) & 3);
-            unit_gather(g[s & 1], sn, s);
+            unit_gather(g[s & 1], sn, ct, kNext, s);
             if (s < 3) read_b(b[(s + 1) & 1], buf, s + 1);
+            else read_b(b[0], buf ^ 1, 0);   // step 0 of tile kt + 1: its x is in place since the barrier
+            if (kWide && kNext == 0 && s == 3) {
+                cur = nxt;
+                load_trip(nxt, kt + 5);   // tile kt + 1 is the first of the new current four
+            }
 #pragma unroll
             for (int i = 0; i < kGrTN; i++)
 #pragma unroll
                 for (int j = 0; j < TM; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, afr[buf][i][s]),
                                                                        __builtin_bit_cast(h8_t, b[s & 1][j]), acc[i][j], 0, 0, 0);
-            if (s < TM) x_store(sn, buf ^ 1, s);
+            // the x of tile kt + 1 goes to the other buffer in steps 0 .. 2, ahead of the barrier
+            if (TM == 4) {
+                if (s == 0) x_store(sn, buf ^ 1, 0);
+                if (s == 1) {
+                    x_store(sn, buf ^ 1, 1);
+                    x_store(sn, buf ^ 1, 2);
+                }
+                if (s == 2) x_store(sn, buf ^ 1, 3);
+            } else if (s < TM) {
+                x_store(sn, buf ^ 1, s);
+            }
 #pragma unroll
             for (int r = 0; r < kMfma; r++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          // MFMA
                 __builtin_amdgcn_sched_group_barrier(0x100, kDsPer, 0);     // LDS reads
                 __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0);   // VALU
                 if (s < 3 && (r == 1 || r == kMfma / 2)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
+                if (kWide && kNext == 0 && s == 3 && r < 2 * kGrTN) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
-            if (s < TM) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS write
+            if (TM == 4 ? s < 3 : s < TM) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // LDS writes
+            if (TM == 4 && s == 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
             __builtin_amdgcn_sched_barrier(0);
+            // The tile's one barrier lies between steps 2 and 3, not at its end, so that no tile starts by
+            // waiting for an LDS read behind a barrier: buffer buf ^ 1 was last read in step 2 of the tile
+            // before (the fragments of its step 3), ahead of that tile's barrier, and is read again in step 3.
+            if (s == 2) __syncthreads();
         }
-        __syncthreads();
     };
 
     // Four tiles per trip with no way out in between: a path that left the loop body early
@@ -1943,15 +2007,19 @@ __global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restric
     // reuses, and the wait the compiler places there for that path (all loads done) would
     // be paid by every trip.  The up to three tiles left over run after the loop.
     int kt = 0;
+    typedef std::integral_constant<int, 0> N0;
+    typedef std::integral_constant<int, 1> N1;
+    typedef std::integral_constant<int, 2> N2;
+    typedef std::integral_constant<int, 3> N3;
     for (; kt + 4 <= k_tiles; kt += 4) {
-        tile(kt, 0, ring[1], ring[0]);
-        tile(kt + 1, 1, ring[2], ring[1]);
-        tile(kt + 2, 0, ring[3], ring[2]);
-        tile(kt + 3, 1, ring[0], ring[3]);
+        tile(kt, 0, ring[1], ring[0], N1{});
+        tile(kt + 1, 1, ring[2], ring[1], N2{});
+        tile(kt + 2, 0, ring[3], ring[2], N3{});
+        tile(kt + 3, 1, ring[0], ring[3], N0{});
     }
-    if (kt < k_tiles) tile(kt, 0, ring[1], ring[0]);
-    if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1]);
-    if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
+    if (kt < k_tiles) tile(kt, 0, ring[1], ring[0], N1{});
+    if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1], N2{});
+    if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2], N3{});
 
     // D layout of 32x32: element e of lane: row (n) = 8*(e/4) + 4*(lane/32) + e%4, column (m) = lane%32
     const bool n_vec = (N & 3) == 0 && (kSplit || y_vec != 0);   // 8-byte stores need an 8-byte aligned y
@@ -2358,23 +2426,30 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 
 
 // ------------------------------------------------------------------ the integer operator, many rows of x
-// Block tile 256 (n) x 128 (m) x 64 (k), eight waves (two per SIMD, to hide the table gathers),
-// each 32 rows of W x all 128 rows of x = 4 accumulators of v_mfma_i32_32x32x32_i8.  Like the half-precision gemm_reg_kernel, every wave
-// decodes its own rows straight into A operands - here that is two 8-byte gathers and two
-// exclusive ors per code (int8x_kernel's tables), four codes per lane and k tile - and only x goes
-// through the LDS (rows 80 bytes apart: the 16 lanes the LDS serves per clock, 16 consecutive
-// rows, hit 16 different bank groups).  Lane (row, half h = lane / 32) takes codes 4 h .. 4 h + 3
-// of its row's 8 in the k tile (8 consecutive bytes; in the reference's tile order, the 16 bytes
-// of the pair of rows, of which one v_perm per two codes keeps ours) and pairs them with bytes
-// 32 h .. 32 h + 31 of the x rows.  Global loads run four k tiles ahead in a ring of registers;
-// one barrier per k tile.  A table with a byte that is not 2 mod 4: the workgroup does its tile
-// with the scalar decode.
+// Block tile 256 (n) x 128 (m) x 64 (k), four waves (one per SIMD), each 64 rows of W (two 32-row
+// tiles) x all 128 rows of x = 8 accumulators of v_mfma_i32_32x32x32_i8.  Like the half-precision
+// gemm_reg_kernel, every wave decodes its own rows straight into A operands - here that is two
+// 8-byte gathers and two exclusive ors per code (int8x_kernel's tables), eight codes per lane and
+// k tile - and only x goes through the LDS (rows 80 bytes apart: the 16 lanes the LDS serves per
+// clock, 16 consecutive rows, hit 16 different bank groups).  With 64 rows per wave a fragment of x
+// read from the LDS feeds two MFMAs: per k tile the workgroup moves 32 KB of x fragments and 32 KB of
+// table rows through the LDS for 64 MFMAs (eight waves of 32 rows each moved 64 + 32 KB, more
+// LDS time than the matrix units needed for the tile).  Lane (row, half h = lane / 32) takes codes
+// 4 h .. 4 h + 3 of its row's 8 in the k tile (8 consecutive bytes; in the reference's tile order, the
+// 16 bytes of the pair of rows, of which one v_perm per two codes keeps ours) and pairs them with
+// bytes 32 h .. 32 h + 31 of the x rows.
+// The decode runs one k tile ahead of the MFMAs as a stream of units (the two codes of one row tile
+// and MFMA step): a step gathers the table rows of two units and finishes (exclusive ors) the two
+// gathered a step earlier, and scheduling hints weave that between the step's eight MFMAs - with
+// one wave per SIMD nothing else hides it.  Global loads run four k tiles ahead in a ring of
+// registers; one barrier per k tile.  A table with a byte that is not 2 mod 4: the workgroup does its
+// tile with the scalar decode.
 typedef int i16_t __attribute__((ext_vector_type(16)));
 constexpr int kI8gBN = 256, kI8gBM = 128, kI8gBK = 64, kI8gLd = 80;
 constexpr int kI8gSmem = 2 * kI8TableBytes + 2 * kI8gBM * kI8gLd;
 
 template <bool kTiled>
-__global__ __launch_bounds__(512) void int8g_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+__global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
                                                     const int64_t *__restrict__ codebook_abs,
                                                     int32_t *__restrict__ out, int M, int N, int K)
 {
@@ -2392,24 +2467,78 @@ __global__ __launch_bounds__(512) void int8g_kernel(const int8_t *__restrict__ x
     const int k_tiles = K / kI8gBK;
     constexpr int kOut = (int)0x80000000;
 
-    // tables: threads 0 .. 255 write the 32 copies of table entry tid, threads 256 .. 511 those of
-    // the mask of high byte tid - 256 (the mask table follows the grid table: row tid either way)
-    const uint64_t entry = tid < 256 ? (uint64_t)codebook_abs[tid] : 0x0202020202020202ull;
-    {
-        uint64_t v = entry;
-        if (tid >= 256) {
-            const uint32_t t = (uint32_t)tid - 256u;
-            uint32_t s8 = t & 0x7Fu;
-            s8 |= (__builtin_popcount(s8) & 1u) << 7;
-            v = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
+    // global sources, as raw buffer loads (rows past N / M and tiles past the end: zeros, no access)
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kTiled ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(x), 0, (int)((int64_t)M * K), 0x00020000);
+    // codes of row tile i (32 rows): row-major 8 bytes at row * K / 4 + kt * 16 + 8 h; tiled: tile
+    // (row / 16, 2 kt + h) of 128 bytes, 16 bytes at (row % 8) * 16
+    int cvoff[2];
 #pragma unroll
-            for (int d = 0; d < 8; d++)
-                if ((s8 >> d) & 1u) v ^= 0xFCull << (8 * d);
+    for (int i = 0; i < 2; i++) {
+        const int n = n0 + wave * 64 + i * 32 + l32;
+        if (kTiled) cvoff[i] = n < N ? (n >> 4) * 16 * row_bytes + kq * 128 + (n & 7) * 16 : kOut;
+        else cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
+    }
+    const uint32_t half_sel = (l32 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
+    // x: thread tid loads piece tid % 4 (16 bytes) of rows tid / 4 and tid / 4 + 64 of the tile
+    int xvoff[2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const int m = m0 + (tid >> 2) + 64 * p;
+        xvoff[p] = m < M ? m * K + (tid & 3) * 16 : kOut;
+    }
+    unsigned char *xw_ptr = xs + (tid >> 2) * kI8gLd + (tid & 3) * 16;
+    const uint32_t xr_addr = lds_addr(xs) + (uint32_t)(l32 * kI8gLd + kq * 32);
+
+    struct Stage {
+        u4_t cw[2];   // row-major: only the low 8 bytes are loaded
+        u4_t xv[2];
+    };
+    auto load = [&](Stage &st, int kt) {
+        const int ok = kt < k_tiles;
+        const int coff = ok ? (kTiled ? kt * 256 : kt * 16) : kOut;
+        const int xoff = ok ? kt * kI8gBK : kOut;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (kTiled) {
+                st.cw[i] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, cvoff[i], coff, 0);
+            } else {
+                const u2_t v = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
+                st.cw[i] = u4_t{v[0], v[1], 0u, 0u};
+            }
         }
-        u4_t *rowp = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;
-        const u4_t vv = u4_t{(uint32_t)v, (uint32_t)(v >> 32), (uint32_t)v, (uint32_t)(v >> 32)};
 #pragma unroll
-        for (int i = 0; i < 16; i++) rowp[(i + tid) & 15] = vv;   // 16 lanes, 16 bank groups
+        for (int p = 0; p < 2; p++) st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
+    };
+    auto stage_x = [&](const Stage &st, int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++)
+            *reinterpret_cast<u4_t *>(xw_ptr + buf * kI8gBM * kI8gLd + p * 64 * kI8gLd) = st.xv[p];
+    };
+    Stage ring[4];
+#pragma unroll
+    for (int d = 0; d < 4; d++) load(ring[d], d);
+
+    // tables: thread tid writes the 32 copies of table entry tid and those of the mask of high byte
+    // tid (the mask table follows the grid table)
+    const uint64_t entry = (uint64_t)codebook_abs[tid];
+    {
+        const uint32_t t = (uint32_t)tid;
+        uint32_t s8 = t & 0x7Fu;
+        s8 |= (__builtin_popcount(s8) & 1u) << 7;
+        uint64_t mk = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
+#pragma unroll
+        for (int d = 0; d < 8; d++)
+            if ((s8 >> d) & 1u) mk ^= 0xFCull << (8 * d);
+        u4_t *rowp = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;
+        const u4_t ve = u4_t{(uint32_t)entry, (uint32_t)(entry >> 32), (uint32_t)entry, (uint32_t)(entry >> 32)};
+        const u4_t vm = u4_t{(uint32_t)mk, (uint32_t)(mk >> 32), (uint32_t)mk, (uint32_t)(mk >> 32)};
+#pragma unroll
+        for (int i = 0; i < 16; i++) rowp[(i + tid) & 15] = ve;   // 16 lanes, 16 bank groups
+#pragma unroll
+        for (int i = 0; i < 16; i++) rowp[256 * 16 + ((i + tid) & 15)] = vm;
     }
     // the vote on the table (one word per wave in the x area, read by everybody after the barrier)
     {
@@ -2418,144 +2547,147 @@ __global__ __launch_bounds__(512) void int8g_kernel(const int8_t *__restrict__ x
         const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
         if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
         __syncthreads();
-        const bool any_bad = (votes[0] | votes[1] | votes[2] | votes[3]) != 0;   // the table is in waves 0 - 3
+        const bool any_bad = (votes[0] | votes[1] | votes[2] | votes[3]) != 0;
         __syncthreads();   // the votes are read before x overwrites them
         if (any_bad) {
             uint64_t *table = reinterpret_cast<uint64_t *>(xs);
-            if (tid < 256) table[tid] = entry;
+            table[tid] = entry;
             __syncthreads();
             const int64_t n_end = (int64_t)n0 + kI8gBN < N ? (int64_t)n0 + kI8gBN : N;
             const int64_t mc = M - m0 < kI8gBM ? M - m0 : kI8gBM;
             int8_rows<false>(x + (int64_t)m0 * K, codes, table, table, out + (int64_t)m0 * N, mc, N, K, kTiled ? 1 : 0,
-                             false, (int64_t)n0 + wave, 8, n_end);
+                             false, (int64_t)n0 + wave, 4, n_end);
             return;
         }
     }
 
-    // global sources, as raw buffer loads (rows past N / M and tiles past the end: zeros, no access)
-    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kTiled ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
-    const __amdgpu_buffer_rsrc_t xrsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(x), 0, (int)((int64_t)M * K), 0x00020000);
-    // codes of row group i (32 rows): row-major 8 bytes at row * K / 4 + kt * 16 + 8 h; tiled: tile
-    // (row / 16, 2 kt + h) of 128 bytes, 16 bytes at (row % 8) * 16
-    int cvoff;
-    {
-        const int n = n0 + wave * 32 + l32;
-        if (kTiled) cvoff = n < N ? (n >> 4) * 16 * row_bytes + kq * 128 + (n & 7) * 16 : kOut;
-        else cvoff = n < N ? n * row_bytes + kq * 8 : kOut;
-    }
-    const uint32_t half_sel = (l32 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
-    // x: thread tid loads piece tid % 4 (16 bytes) of row tid / 4 of the tile
-    int xvoff;
-    {
-        const int m = m0 + (tid >> 2);
-        xvoff = m < M ? m * K + (tid & 3) * 16 : kOut;
-    }
-    unsigned char *xw_ptr = xs + (tid >> 2) * kI8gLd + (tid & 3) * 16;
-    const uint32_t xr_addr = lds_addr(xs) + (uint32_t)(l32 * kI8gLd + kq * 32);
-
-    struct Stage {
-        u4_t cw;   // row-major: only the low 8 bytes are loaded
-        u4_t xv;
-    };
-    auto load = [&](Stage &st, int kt) {
-        const int ok = kt < k_tiles;
-        const int coff = ok ? (kTiled ? kt * 256 : kt * 16) : kOut;
-        const int xoff = ok ? kt * kI8gBK : kOut;
-        if (kTiled) {
-            st.cw = __builtin_amdgcn_raw_buffer_load_b128(crsrc, cvoff, coff, 0);
-        } else {
-            const u2_t v = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff, coff, 0);
-            st.cw = u4_t{v[0], v[1], 0u, 0u};
-        }
-        st.xv = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff, xoff, 0);
-    };
-    auto stage_x = [&](const Stage &st, int buf) {
-        *reinterpret_cast<u4_t *>(xw_ptr + buf * kI8gBM * kI8gLd) = st.xv;
-    };
-
-    i16_t acc[4];
+    i16_t acc[2][4];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) acc[j][e] = 0;
-
-    // k tile kt out of LDS buffer kt % 2 with the codes of ring slot `cur`; then the x of tile
-    // kt + 1 (slot `nxt`, loaded three tiles ago) goes to the other buffer, slot `cur` is refilled
-    // with tile kt + 4, and the barrier hands the buffers over
-    auto tile = [&](int kt, Stage &cur, const Stage &nxt) {
-        const uint32_t xb_addr = xr_addr + (uint32_t)((kt & 1) * kI8gBM * kI8gLd);
-        u4_t b[4][2];
+    for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++)
 #pragma unroll
-            for (int s2 = 0; s2 < 2; s2++) b[j][s2] = lds_read16(xb_addr + (uint32_t)(j * 32 * kI8gLd + s2 * 16));
-        uint32_t cwi[2];   // [MFMA step]: two codes each
-        if (kTiled) {
-            cwi[0] = __builtin_amdgcn_perm(cur.cw[1], cur.cw[0], half_sel);
-            cwi[1] = __builtin_amdgcn_perm(cur.cw[3], cur.cw[2], half_sel);
-        } else {
-            cwi[0] = cur.cw[0];
-            cwi[1] = cur.cw[1];
-        }
-        u2_t g[4], k[4];   // all 8 gathers of the tile go out before the first MFMA
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
+
+    // unit u of a tile: the two codes (8 weights each) of row tile u % 2 and MFMA step u / 2
+    struct Unit {
+        u2_t g[2], k[2];
+    };
+    i4_t afr[2][2][2];   // A operands: [buffer][row tile][MFMA step]
+    auto unit_gather = [&](Unit &o, const Stage &st, int u) {
+        const int i = u & 1, s2 = u >> 1;
+        const uint32_t w = kTiled ? __builtin_amdgcn_perm(st.cw[i][2 * s2 + 1], st.cw[i][2 * s2], half_sel) : st.cw[i][s2];
+        o.g[0] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
+        o.k[0] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
+        o.g[1] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
+        o.k[1] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
+    };
+    auto unit_finish = [&](const Unit &o, int abuf, int u) {
+        afr[abuf][u & 1][u >> 1] = i4_t{(int)(o.g[0][0] ^ o.k[0][0]), (int)(o.g[0][1] ^ o.k[0][1]),
+                                        (int)(o.g[1][0] ^ o.k[1][0]), (int)(o.g[1][1] ^ o.k[1][1])};
+    };
+    Unit ga[2], gb[2];   // units 0, 1 (MFMA step 0) and 2, 3 (step 1) in flight
+
+    auto read_b = [&](u4_t (&b)[4], int buf, int s2) {
 #pragma unroll
-        for (int s2 = 0; s2 < 2; s2++) {
-            const uint32_t w = cwi[s2];
-            g[2 * s2] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
-            k[2 * s2] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
-            g[2 * s2 + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
-            k[2 * s2 + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
-        }
+        for (int j = 0; j < 4; j++)
+            b[j] = lds_read16(xr_addr + (uint32_t)(buf * kI8gBM * kI8gLd + j * 32 * kI8gLd + s2 * 16));
+    };
+    u4_t b0[4], b1[4];   // the x fragments of MFMA step 0 and 1
+
+    stage_x(ring[0], 0);
+    unit_gather(ga[0], ring[0], 0);
+    unit_gather(ga[1], ring[0], 1);
+    unit_finish(ga[0], 0, 0);
+    unit_finish(ga[1], 0, 1);
+    unit_gather(gb[0], ring[0], 2);
+    unit_gather(gb[1], ring[0], 3);
+    __syncthreads();   // x tile 0 staged
+    read_b(b0, 0, 0);
+
+    // MFMAs of tile kt (A = afr[buf], B from x buffer buf).  Step 0 finishes the tile's own second
+    // pair of units (gathered in the last step of the tile before), gathers the first pair of tile
+    // kt + 1 (registers sn), reads its own second set of x fragments, writes the x of tile kt + 1
+    // to buffer buf ^ 1 and fetches tile kt + 4 into sf; step 1 finishes that pair into afr[buf ^ 1],
+    // gathers the second and reads the first x fragments of tile kt + 1.  The tile's one barrier lies
+    // between the two steps, so that no step starts by waiting for an LDS read behind a barrier: buffer
+    // buf ^ 1 is last read before the barrier of the tile before (its fragments of step 1) and first
+    // read after this one.
+    auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf) {
+        unit_finish(gb[0], buf, 2);
+        unit_finish(gb[1], buf, 3);
+        unit_gather(ga[0], sn, 0);
+        unit_gather(ga[1], sn, 1);
+        read_b(b1, buf, 1);
+        stage_x(sn, buf ^ 1);
+        load(sf, kt + 4);
 #pragma unroll
-        for (int s2 = 0; s2 < 2; s2++) {
-            const i4_t a = i4_t{(int)(g[2 * s2][0] ^ k[2 * s2][0]), (int)(g[2 * s2][1] ^ k[2 * s2][1]),
-                                (int)(g[2 * s2 + 1][0] ^ k[2 * s2 + 1][0]), (int)(g[2 * s2 + 1][1] ^ k[2 * s2 + 1][1])};
+        for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, __builtin_bit_cast(i4_t, b[j][s2]), acc[j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[buf][i][0], __builtin_bit_cast(i4_t, b0[j]), acc[i][j], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // MFMA
+            if (r < 4) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);     // LDS reads, early: done by the barrier
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                // VALU
+            if (r == 4) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);    // LDS writes
+            if (r >= 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // global loads
         }
-        stage_x(nxt, (kt + 1) & 1);
-        load(cur, kt + 4);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        unit_finish(ga[0], buf ^ 1, 0);
+        unit_finish(ga[1], buf ^ 1, 1);
+        unit_gather(gb[0], sn, 2);
+        unit_gather(gb[1], sn, 3);
+        read_b(b0, buf ^ 1, 0);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[buf][i][1], __builtin_bit_cast(i4_t, b1[j]), acc[i][j], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // MFMA
+            if (r < 4) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);     // LDS reads
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                // VALU
+        }
+        __builtin_amdgcn_sched_barrier(0);
     };
 
-    Stage ring[4];
-#pragma unroll
-    for (int d = 0; d < 4; d++) load(ring[d], d);
-    stage_x(ring[0], 0);
-    __syncthreads();
     int kt = 0;
     for (; kt + 4 <= k_tiles; kt += 4) {
-        tile(kt, ring[0], ring[1]);
-        tile(kt + 1, ring[1], ring[2]);
-        tile(kt + 2, ring[2], ring[3]);
-        tile(kt + 3, ring[3], ring[0]);
+        tile(kt, 0, ring[1], ring[0]);
+        tile(kt + 1, 1, ring[2], ring[1]);
+        tile(kt + 2, 0, ring[3], ring[2]);
+        tile(kt + 3, 1, ring[0], ring[3]);
     }
-    if (kt < k_tiles) tile(kt, ring[0], ring[1]);
-    if (kt + 1 < k_tiles) tile(kt + 1, ring[1], ring[2]);
-    if (kt + 2 < k_tiles) tile(kt + 2, ring[2], ring[3]);
+    if (kt < k_tiles) tile(kt, 0, ring[1], ring[0]);
+    if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1]);
+    if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
 
     // D layout of 32x32: element e of lane: row (n) = 8 * (e / 4) + 4 * (lane / 32) + e % 4, column (m) = lane % 32
     const bool n_vec = (N & 3) == 0;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int m = m0 + j * 32 + l32;
-        if (m >= M) continue;
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int e4 = 0; e4 < 4; e4++) {
-            const int n = n0 + wave * 32 + 8 * e4 + 4 * kq;
-            int32_t *dst = out + (int64_t)m * N + n;
-            if (n_vec && n + 3 < N) {
-                *reinterpret_cast<i4_t *>(dst) = i4_t{acc[j][4 * e4], acc[j][4 * e4 + 1], acc[j][4 * e4 + 2], acc[j][4 * e4 + 3]};
-            } else {
+        for (int j = 0; j < 4; j++) {
+            const int m = m0 + j * 32 + l32;
+            if (m >= M) continue;
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (n + e < N) dst[e] = acc[j][4 * e4 + e];
+            for (int e4 = 0; e4 < 4; e4++) {
+                const int n = n0 + wave * 64 + i * 32 + 8 * e4 + 4 * kq;
+                int32_t *dst = out + (int64_t)m * N + n;
+                if (n_vec && n + 3 < N) {
+                    *reinterpret_cast<i4_t *>(dst) =
+                        i4_t{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < N) dst[e] = acc[i][j][4 * e4 + e];
+                }
             }
         }
-    }
 }
 
 __global__ void zero_i32_kernel(int32_t *y, int64_t n)
@@ -3101,7 +3233,7 @@ int launch_int8g(const void *x, const void *codes, const void *cb, void *out, in
                  hipStream_t stream)
 {
     dim3 g((unsigned)((M + kI8gBM - 1) / kI8gBM), (unsigned)((N + kI8gBN - 1) / kI8gBN));
-    return launch(int8g_kernel<kTiled>, g, dim3(512), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
+    return launch(int8g_kernel<kTiled>, g, dim3(256), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
                   (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
 }
 
