@@ -2426,38 +2426,45 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 
 
 // ------------------------------------------------------------------ the integer operator, many rows of x
-// Block tile 256 (n) x 128 (m) x 64 (k), four waves (one per SIMD), each 64 rows of W (two 32-row
-// tiles) x all 128 rows of x = 8 accumulators of v_mfma_i32_32x32x32_i8.  Like the half-precision
-// gemm_reg_kernel, every wave decodes its own rows straight into A operands - here that is two
-// 8-byte gathers and two exclusive ors per code (int8x_kernel's tables), eight codes per lane and
-// k tile - and only x goes through the LDS (rows 80 bytes apart: the 16 lanes the LDS serves per
-// clock, 16 consecutive rows, hit 16 different bank groups).  With 64 rows per wave a fragment of x
-// read from the LDS feeds two MFMAs: per k tile the workgroup moves 32 KB of x fragments and 32 KB of
-// table rows through the LDS for 64 MFMAs (eight waves of 32 rows each moved 64 + 32 KB, more
-// LDS time than the matrix units needed for the tile).  Lane (row, half h = lane / 32) takes codes
-// 4 h .. 4 h + 3 of its row's 8 in the k tile (8 consecutive bytes; in the reference's tile order, the
-// 16 bytes of the pair of rows, of which one v_perm per two codes keeps ours) and pairs them with
-// bytes 32 h .. 32 h + 31 of the x rows.
+// Block tile 256 (n) x 128 (m), eight waves in two groups of four.  A group is a complete
+// 256 x 128 x 64 pipeline - one wave per SIMD, each 64 rows of W (two 32-row tiles) x all 128 rows
+// of x = 8 accumulators of v_mfma_i32_32x32x32_i8 - and the two groups take the even and the odd k
+// tiles of the same output tile, so that every SIMD holds two waves working on different k tiles:
+// while one waits for its table gathers or its x fragments the other's MFMAs run.  At the end each
+// group hands the other the partial sums of one of its two row tiles through the LDS (the tables'
+// space, by then free) and stores the other one.
+// Like the half-precision gemm_reg_kernel, every wave decodes its own rows straight into A
+// operands - here that is two 8-byte gathers and two exclusive ors per code (int8x_kernel's
+// tables), eight codes per lane and k tile - and only x goes through the LDS: four buffers (two
+// per group) of 128 rows x 64 bytes, the 16-byte pieces of a row exchanged by (row / 4) % 4 so
+// that the 16 lanes the LDS serves per clock hit 16 different bank groups without padding (the
+// tables take 128 KB of the 160).  Lane (row, half h = lane / 32) takes codes 4 h .. 4 h + 3 of its
+// row's 8 in the k tile (8 consecutive bytes; in the reference's tile order, the 16 bytes of the
+// pair of rows, of which one v_perm per two codes keeps ours) and pairs them with bytes 32 h ..
+// 32 h + 31 of the x rows.
 // The decode runs one k tile ahead of the MFMAs as a stream of units (the two codes of one row tile
 // and MFMA step): a step gathers the table rows of two units and finishes (exclusive ors) the two
-// gathered a step earlier, and scheduling hints weave that between the step's eight MFMAs - with
-// one wave per SIMD nothing else hides it.  Global loads run four k tiles ahead in a ring of
-// registers; one barrier per k tile.  A table with a byte that is not 2 mod 4: the workgroup does its
-// tile with the scalar decode.
+// gathered a step earlier, and scheduling hints weave that between the step's eight MFMAs.  Global
+// loads run three of the group's k tiles ahead in a ring of registers; one barrier per pair of k
+// tiles (one of either group).
+// A table with a byte that is not 2 mod 4: the workgroup does its tile with the scalar decode.
 typedef int i16_t __attribute__((ext_vector_type(16)));
-constexpr int kI8gBN = 256, kI8gBM = 128, kI8gBK = 64, kI8gLd = 80;
-constexpr int kI8gSmem = 2 * kI8TableBytes + 2 * kI8gBM * kI8gLd;
+constexpr int kI8gBN = 256, kI8gBM = 128, kI8gBK = 64;
+constexpr int kI8gXBuf = kI8gBM * kI8gBK;                       // one x tile, unpadded
+constexpr int kI8gSmem = 2 * kI8TableBytes + 4 * kI8gXBuf;      // 160 KB
 
 template <bool kTiled>
-__global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+__global__ __launch_bounds__(512) void int8g_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
                                                     const int64_t *__restrict__ codebook_abs,
                                                     int32_t *__restrict__ out, int M, int N, int K)
 {
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    unsigned char *xs = smem_raw + 2 * kI8TableBytes;   // two x tiles of 128 rows x 80 bytes
+    unsigned char *xs = smem_raw + 2 * kI8TableBytes;   // x tiles: [group][buffer]
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave >> 2, w4 = wave & 3;            // group (k tile parity) and place along n
+    const int gtid = tid & 255;
     const int l32 = lane & 31, kq = lane >> 5;
     const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;   // grid rows: [0, 64K)
     const uint32_t lane_base2 = lane_base | 0x10000u;        // mask rows: [64K, 128K)
@@ -2465,6 +2472,7 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
     const int n0 = blockIdx.y * kI8gBN;
     const int row_bytes = K >> 2;
     const int k_tiles = K / kI8gBK;
+    const int g_tiles = (k_tiles + 1) >> 1;              // tiles per group (the odd group's last may not exist)
     constexpr int kOut = (int)0x80000000;
 
     // global sources, as raw buffer loads (rows past N / M and tiles past the end: zeros, no access)
@@ -2477,26 +2485,31 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
     int cvoff[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        const int n = n0 + wave * 64 + i * 32 + l32;
+        const int n = n0 + w4 * 64 + i * 32 + l32;
         if (kTiled) cvoff[i] = n < N ? (n >> 4) * 16 * row_bytes + kq * 128 + (n & 7) * 16 : kOut;
         else cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
     }
     const uint32_t half_sel = (l32 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
-    // x: thread tid loads piece tid % 4 (16 bytes) of rows tid / 4 and tid / 4 + 64 of the tile
+    // x: thread gtid of a group loads piece gtid % 4 (16 bytes) of rows gtid / 4 and gtid / 4 + 64 of the
+    // group's tile; in the LDS piece p of row r sits at r * 64 + (p ^ (r / 4) % 4) * 16
     int xvoff[2];
 #pragma unroll
     for (int p = 0; p < 2; p++) {
-        const int m = m0 + (tid >> 2) + 64 * p;
-        xvoff[p] = m < M ? m * K + (tid & 3) * 16 : kOut;
+        const int m = m0 + (gtid >> 2) + 64 * p;
+        xvoff[p] = m < M ? m * K + (gtid & 3) * 16 : kOut;
     }
-    unsigned char *xw_ptr = xs + (tid >> 2) * kI8gLd + (tid & 3) * 16;
-    const uint32_t xr_addr = lds_addr(xs) + (uint32_t)(l32 * kI8gLd + kq * 32);
+    unsigned char *xg = xs + grp * 2 * kI8gXBuf;   // this group's two buffers
+    unsigned char *xw_ptr = xg + (gtid >> 2) * 64 + (((gtid & 3) ^ ((gtid >> 4) & 3)) << 4);
+    const uint32_t swz = (uint32_t)(l32 >> 2) & 3u;
+    const uint32_t xr_addr = lds_addr(xg) + (uint32_t)(l32 * 64);
+    const uint32_t xr_off[2] = {(((uint32_t)kq * 2u) ^ swz) << 4, (((uint32_t)kq * 2u + 1u) ^ swz) << 4};
 
     struct Stage {
         u4_t cw[2];   // row-major: only the low 8 bytes are loaded
         u4_t xv[2];
     };
-    auto load = [&](Stage &st, int kt) {
+    auto load = [&](Stage &st, int t) {   // t: the group's tile, k tile 2 t + grp
+        const int kt = 2 * t + grp;
         const int ok = kt < k_tiles;
         const int coff = ok ? (kTiled ? kt * 256 : kt * 16) : kOut;
         const int xoff = ok ? kt * kI8gBK : kOut;
@@ -2514,31 +2527,30 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
     };
     auto stage_x = [&](const Stage &st, int buf) {
 #pragma unroll
-        for (int p = 0; p < 2; p++)
-            *reinterpret_cast<u4_t *>(xw_ptr + buf * kI8gBM * kI8gLd + p * 64 * kI8gLd) = st.xv[p];
+        for (int p = 0; p < 2; p++) *reinterpret_cast<u4_t *>(xw_ptr + buf * kI8gXBuf + p * 64 * 64) = st.xv[p];
     };
-    Stage ring[4];
+    Stage ring[3];
 #pragma unroll
-    for (int d = 0; d < 4; d++) load(ring[d], d);
+    for (int d = 0; d < 3; d++) load(ring[d], d);
 
-    // tables: thread tid writes the 32 copies of table entry tid and those of the mask of high byte
-    // tid (the mask table follows the grid table)
-    const uint64_t entry = (uint64_t)codebook_abs[tid];
+    // tables: threads 0 .. 255 write the 32 copies of table entry tid, threads 256 .. 511 those of
+    // the mask of high byte tid - 256 (the mask table follows the grid table: row tid either way)
+    const uint64_t entry = tid < 256 ? (uint64_t)codebook_abs[tid] : 0x0202020202020202ull;
     {
-        const uint32_t t = (uint32_t)tid;
-        uint32_t s8 = t & 0x7Fu;
-        s8 |= (__builtin_popcount(s8) & 1u) << 7;
-        uint64_t mk = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
+        uint64_t v = entry;
+        if (tid >= 256) {
+            const uint32_t t = (uint32_t)tid - 256u;
+            uint32_t s8 = t & 0x7Fu;
+            s8 |= (__builtin_popcount(s8) & 1u) << 7;
+            v = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
 #pragma unroll
-        for (int d = 0; d < 8; d++)
-            if ((s8 >> d) & 1u) mk ^= 0xFCull << (8 * d);
+            for (int d = 0; d < 8; d++)
+                if ((s8 >> d) & 1u) v ^= 0xFCull << (8 * d);
+        }
         u4_t *rowp = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;
-        const u4_t ve = u4_t{(uint32_t)entry, (uint32_t)(entry >> 32), (uint32_t)entry, (uint32_t)(entry >> 32)};
-        const u4_t vm = u4_t{(uint32_t)mk, (uint32_t)(mk >> 32), (uint32_t)mk, (uint32_t)(mk >> 32)};
+        const u4_t vv = u4_t{(uint32_t)v, (uint32_t)(v >> 32), (uint32_t)v, (uint32_t)(v >> 32)};
 #pragma unroll
-        for (int i = 0; i < 16; i++) rowp[(i + tid) & 15] = ve;   // 16 lanes, 16 bank groups
-#pragma unroll
-        for (int i = 0; i < 16; i++) rowp[256 * 16 + ((i + tid) & 15)] = vm;
+        for (int i = 0; i < 16; i++) rowp[(i + tid) & 15] = vv;   // 16 lanes, 16 bank groups
     }
     // the vote on the table (one word per wave in the x area, read by everybody after the barrier)
     {
@@ -2547,16 +2559,16 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
         const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
         if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
         __syncthreads();
-        const bool any_bad = (votes[0] | votes[1] | votes[2] | votes[3]) != 0;
+        const bool any_bad = (votes[0] | votes[1] | votes[2] | votes[3]) != 0;   // the table is in waves 0 - 3
         __syncthreads();   // the votes are read before x overwrites them
         if (any_bad) {
             uint64_t *table = reinterpret_cast<uint64_t *>(xs);
-            table[tid] = entry;
+            if (tid < 256) table[tid] = entry;
             __syncthreads();
             const int64_t n_end = (int64_t)n0 + kI8gBN < N ? (int64_t)n0 + kI8gBN : N;
             const int64_t mc = M - m0 < kI8gBM ? M - m0 : kI8gBM;
             int8_rows<false>(x + (int64_t)m0 * K, codes, table, table, out + (int64_t)m0 * N, mc, N, K, kTiled ? 1 : 0,
-                             false, (int64_t)n0 + wave, 4, n_end);
+                             false, (int64_t)n0 + wave, 8, n_end);
             return;
         }
     }
@@ -2590,11 +2602,8 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
 
     auto read_b = [&](u4_t (&b)[4], int buf, int s2) {
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-            b[j] = lds_read16(xr_addr + (uint32_t)(buf * kI8gBM * kI8gLd + j * 32 * kI8gLd + s2 * 16));
+        for (int j = 0; j < 4; j++) b[j] = lds_read16(xr_addr + (uint32_t)(buf * kI8gXBuf + j * 32 * 64) + xr_off[s2]);
     };
-    u4_t b0[4], b1[4];   // the x fragments of MFMA step 0 and 1
-
     stage_x(ring[0], 0);
     unit_gather(ga[0], ring[0], 0);
     unit_gather(ga[1], ring[0], 1);
@@ -2602,92 +2611,116 @@ __global__ __launch_bounds__(256) void int8g_kernel(const int8_t *__restrict__ x
     unit_finish(ga[1], 0, 1);
     unit_gather(gb[0], ring[0], 2);
     unit_gather(gb[1], ring[0], 3);
-    __syncthreads();   // x tile 0 staged
-    read_b(b0, 0, 0);
+    __syncthreads();   // x tile 0 of either group staged
 
-    // MFMAs of tile kt (A = afr[buf], B from x buffer buf).  Step 0 finishes the tile's own second
-    // pair of units (gathered in the last step of the tile before), gathers the first pair of tile
-    // kt + 1 (registers sn), reads its own second set of x fragments, writes the x of tile kt + 1
-    // to buffer buf ^ 1 and fetches tile kt + 4 into sf; step 1 finishes that pair into afr[buf ^ 1],
-    // gathers the second and reads the first x fragments of tile kt + 1.  The tile's one barrier lies
-    // between the two steps, so that no step starts by waiting for an LDS read behind a barrier: buffer
-    // buf ^ 1 is last read before the barrier of the tile before (its fragments of step 1) and first
-    // read after this one.
-    auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf) {
+    // MFMAs of the group's tile t (A = afr[buf], B from the group's x buffer buf).  Step 0 finishes the
+    // tile's own second pair of units (gathered in the last step of the tile before), gathers the first
+    // pair of tile t + 1 (registers sn), writes the x of tile t + 1 to buffer buf ^ 1 and fetches tile
+    // t + 3 into sf; step 1 finishes that pair into afr[buf ^ 1] and gathers the second.  Each step
+    // reads its own x fragments as it starts: the SIMD's other wave covers the wait.
+    auto tile = [&](int t, int buf, const Stage &sn, Stage &sf) {
+        u4_t b[4];
+        read_b(b, buf, 0);
         unit_finish(gb[0], buf, 2);
         unit_finish(gb[1], buf, 3);
         unit_gather(ga[0], sn, 0);
         unit_gather(ga[1], sn, 1);
-        read_b(b1, buf, 1);
         stage_x(sn, buf ^ 1);
-        load(sf, kt + 4);
+        load(sf, t + 3);
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[buf][i][0], __builtin_bit_cast(i4_t, b0[j]), acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[buf][i][0], __builtin_bit_cast(i4_t, b[j]), acc[i][j], 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < 8; r++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // MFMA
-            if (r < 4) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);     // LDS reads, early: done by the barrier
+            if (r < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // LDS reads
             __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                // VALU
             if (r == 4) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);    // LDS writes
             if (r >= 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // global loads
         }
         __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
+        read_b(b, buf, 1);
         unit_finish(ga[0], buf ^ 1, 0);
         unit_finish(ga[1], buf ^ 1, 1);
         unit_gather(gb[0], sn, 2);
         unit_gather(gb[1], sn, 3);
-        read_b(b0, buf ^ 1, 0);
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[buf][i][1], __builtin_bit_cast(i4_t, b1[j]), acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[buf][i][1], __builtin_bit_cast(i4_t, b[j]), acc[i][j], 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < 8; r++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // MFMA
-            if (r < 4) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);     // LDS reads
+            if (r < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // LDS reads
             __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                // VALU
         }
         __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
     };
 
-    int kt = 0;
-    for (; kt + 4 <= k_tiles; kt += 4) {
-        tile(kt, 0, ring[1], ring[0]);
-        tile(kt + 1, 1, ring[2], ring[1]);
-        tile(kt + 2, 0, ring[3], ring[2]);
-        tile(kt + 3, 1, ring[0], ring[3]);
+    // both groups make the same number of trips (the barriers are the workgroup's); six tiles per trip
+    // so that ring slot and x buffer are compile-time constants
+    int t = 0;
+    for (; t + 6 <= g_tiles; t += 6) {
+        tile(t, 0, ring[1], ring[0]);
+        tile(t + 1, 1, ring[2], ring[1]);
+        tile(t + 2, 0, ring[0], ring[2]);
+        tile(t + 3, 1, ring[1], ring[0]);
+        tile(t + 4, 0, ring[2], ring[1]);
+        tile(t + 5, 1, ring[0], ring[2]);
     }
-    if (kt < k_tiles) tile(kt, 0, ring[1], ring[0]);
-    if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1]);
-    if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
+    if (t < g_tiles) tile(t, 0, ring[1], ring[0]);
+    if (t + 1 < g_tiles) tile(t + 1, 1, ring[2], ring[1]);
+    if (t + 2 < g_tiles) tile(t + 2, 0, ring[0], ring[2]);
+    if (t + 3 < g_tiles) tile(t + 3, 1, ring[1], ring[0]);
+    if (t + 4 < g_tiles) tile(t + 4, 0, ring[2], ring[1]);
+
+    // The two groups hold partial sums of the same 256 x 128 outputs.  Group g keeps row tile g of
+    // each of its waves' two and gets the other group's sums for it through the LDS: wave (g, w4)
+    // leaves row tile 1 - g in slot (g, w4), 16 KB of the tables' space, and adds slot (1 - g, w4).
+    {
+        int *slot_w = reinterpret_cast<int *>(smem_raw) + (grp * 4 + w4) * 4096 + lane;
+        const int *slot_r = reinterpret_cast<const int *>(smem_raw) + ((1 - grp) * 4 + w4) * 4096 + lane;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) slot_w[(j * 16 + e) * 64] = grp == 0 ? acc[1][j][e] : acc[0][j][e];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int v = slot_r[(j * 16 + e) * 64];
+                if (grp == 0) acc[0][j][e] += v;
+                else acc[1][j][e] += v;
+            }
+    }
 
     // D layout of 32x32: element e of lane: row (n) = 8 * (e / 4) + 4 * (lane / 32) + e % 4, column (m) = lane % 32
     const bool n_vec = (N & 3) == 0;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int j = 0; j < 4; j++) {
+        const int m = m0 + j * 32 + l32;
+        if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int m = m0 + j * 32 + l32;
-            if (m >= M) continue;
+        for (int e4 = 0; e4 < 4; e4++) {
+            const int n = n0 + w4 * 64 + grp * 32 + 8 * e4 + 4 * kq;
+            int32_t *dst = out + (int64_t)m * N + n;
+            i4_t v;
 #pragma unroll
-            for (int e4 = 0; e4 < 4; e4++) {
-                const int n = n0 + wave * 64 + i * 32 + 8 * e4 + 4 * kq;
-                int32_t *dst = out + (int64_t)m * N + n;
-                if (n_vec && n + 3 < N) {
-                    *reinterpret_cast<i4_t *>(dst) =
-                        i4_t{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
-                } else {
+            for (int e = 0; e < 4; e++) v[e] = grp == 0 ? acc[0][j][4 * e4 + e] : acc[1][j][4 * e4 + e];
+            if (n_vec && n + 3 < N) {
+                *reinterpret_cast<i4_t *>(dst) = v;
+            } else {
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (n + e < N) dst[e] = acc[i][j][4 * e4 + e];
-                }
+                for (int e = 0; e < 4; e++)
+                    if (n + e < N) dst[e] = v[e];
             }
         }
+    }
 }
 
 __global__ void zero_i32_kernel(int32_t *y, int64_t n)
@@ -3233,7 +3266,7 @@ int launch_int8g(const void *x, const void *codes, const void *cb, void *out, in
                  hipStream_t stream)
 {
     dim3 g((unsigned)((M + kI8gBM - 1) / kI8gBM), (unsigned)((N + kI8gBN - 1) / kI8gBN));
-    return launch(int8g_kernel<kTiled>, g, dim3(256), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
+    return launch(int8g_kernel<kTiled>, g, dim3(512), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
                   (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
 }
 
