@@ -482,9 +482,11 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
 @pytest.mark.parametrize("M,N,K,tiled,table", [
     (128, 32768, 256, True, "e8p"), (300, 16 * 1030, 512, False, "mod4"), (64, 40000, 256, False, "any"),
     (2048, 4096, 512, True, "e8p"), (200, 16 * 1030, 1280, True, "mod4"), (129, 16 * 1030, 256, True, "any"),
-    (256, 4096, 4096, True, "e8p"), (512, 2048, 8192, False, "mod4")])
+    (256, 4096, 4096, True, "e8p"), (512, 2048, 8192, False, "mod4"),
+    (512, 2048, 768, False, "e8p"), (384, 4096, 2304, True, "mod4"), (640, 8192, 1536, True, "e8p")])
 def test_integer_operator_matrix_matrix(M, N, K, tiled, table):
-    """Many rows of x run on the int8 matrix-matrix kernel: partial tiles in M and N, both code layouts, 4 to 20 k tiles, and a
+    """Many rows of x run on the int8 matrix-matrix kernel: partial tiles in M and N, both code layouts, 4 to 128 k tiles
+    (2 to 64 per half of the workgroup: every count of leftover tiles after its trips of six, and none), and a
     table with bytes that are not 2 mod 4 (scalar decode per workgroup, with x rows and output
     rows offset by the workgroup's m block).  Exact against the oracle's decode times x in
     float64 (every sum is far below 2^53, so that product is the integer one)."""
