@@ -5,16 +5,17 @@ Headline (the JSON line's `value`): batch-1 decode-GEMV at the Llama-2-70B proje
 shapes.  One step = the four GEMVs (8192->10240, 8192->8192, 8192->28672, 28672->8192), each
 on the next of several distinct code buffers so that the 256 MB Infinity Cache cannot serve
 the weights; `value` is code bytes (N*K/4 per GEMV) per second over the timed region, inputs
-resident in HBM.  The region of exactly --steps steps is timed --repeats times (HIP graph replays
-of 12 steps each, bracketed by synchronisation) and the median region counts; `value_f16_only` is
-the same with the 8-bit kernels switched off, its regions taking turns with the headline's.
+resident in HBM.  The region of exactly --steps steps is timed --repeats times (one HIP graph
+replay of up to 60 steps, bracketed by synchronisation) and the median region counts;
+`value_f16_only` is the same with the 8-bit kernels switched off, timed after the headline.
 Before the --warmup steps the step is replayed for --preheat-ms (200 ms): the device needs some
 15 ms of work to leave its idle clocks.
 
 `roofline` is the GEMV kernel that carries most of the step's bytes, alone: code bytes per
-launch over the kernel's own duration (HIP events placed around the kernel by the library's
-timing hook, on the stream it is launched on) against 8 TB/s; `all_gemv_launches` is the same
-figure over every launch of the step, per kernel.  `hbm_read_probe` is what a kernel that only
+launch over the kernel's launch duration - HIP events on the stream around replays of a graph of
+that kernel's launches of the step, region / launches - against 8 TB/s; `gemv_shapes` and
+`all_gemv_launches` hold every launch of the step, per shape and per kernel, from HIP events
+placed around each eager launch by the library's timing hook.  `hbm_read_probe` is what a kernel that only
 reads the same code buffers reaches (per shape, as a graph step, and per launch with nothing
 to read): the memory system's and the launch path's share of the step.  `gemv_7b_step` is a
 Llama-2-7B layer's four projections as one graph, gate and up as one call on concatenated code
@@ -36,11 +37,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8, published
-# HBM bytes one GEMV launch moves, per kernel, averaged over the four shapes of the step: rocprofv3
-# FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain
-# 256 MiB device copy (x2.000 and x1.000).  Both kernels move 39.2 MB per launch on average against
-# 38,855,680 algorithmic bytes (codes, x, grid, y): 1.009 of them.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8c_kernel": 39198889, "dmm::gemv_stream_kernel": 39188778}
+# HBM bytes one GEMV launch moves, per kernel, averaged over the shapes it serves in a run of this
+# file (the 8-bit kernel: the three shapes the operator gives it; the 16-bit kernel: all four, from
+# the 16-bit-only leg): rocprofv3 FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the
+# same counter reads for a plain 256 MiB device copy (x2.000 and x1.000).  46.57 MB per launch against
+# 46,202,880 algorithmic bytes (codes, x, grid, y) and 39.19 MB against 38,855,680: 1.008 and 1.009.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8c_kernel": 46570133, "dmm::gemv_stream_kernel": 39188881}
 GEMV_TRAFFIC_SOURCE = {k: "constant from an earlier rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command, summarised in "
                           "profiles/gemv_kernels_llama70b_batch1.md; not measured by this run (a counter run cannot share a "
                           "process with the timed one)" for k in GEMV_TRAFFIC_BYTES_PER_LAUNCH}
@@ -58,7 +60,7 @@ def parse():
                          "15 ms of work to leave its idle clocks, more than a short --warmup covers")
     ap.add_argument("--quick", action="store_true", help="skip prefill / small-batch / CPU legs")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
-    ap.add_argument("--graph-steps", type=int, default=12,
+    ap.add_argument("--graph-steps", type=int, default=60,
                     help="steps per HIP graph replay (rounded down to whole turns of the code-buffer sets)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the M = 2048 leg and print its object (for profiling the matrix-matrix kernel)")
@@ -180,10 +182,57 @@ def main():
                         graph_of(chunk).replay()
                     if n % chunk:
                         graph_of(n % chunk).replay()
-                mode = "hip graph, %d steps (%d launches) per replay" % (chunk, chunk * len(probs))
+                per = min(chunk, args.steps)
+                mode = "hip graph, %d steps (%d launches) per replay" % (per, per * len(probs))
             except Exception as e:   # capture unavailable: time the eager loop
                 print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
         return run_steps, mode
+
+    def dominant_kernel_timing():
+        """The kernel that carries most of the step's bytes (by the operator's choice per shape), and its
+        launch duration in the regime the headline runs in: its launches of the step alone (its shapes
+        taking turns over the rotating buffers) as a HIP graph, HIP events on the stream around each
+        replay, duration = region / launches.  That is how a kernel trace of graph launches reads too (one
+        dispatch begins as the one before ends).  Eager, event-bracketed launches start cold after an idle
+        gap and read 0.5 - 1 us longer; they are in `gemv_shapes` and `all_gemv_launches`."""
+        per_kernel = {}
+        for p in probs:
+            n = lib.dmm_gemv_kernel_name(1, p["N"], p["K"]).decode()
+            per_kernel[n] = per_kernel.get(n, 0) + workload.code_bytes(p["N"], p["K"])
+        dom = max(per_kernel, key=per_kernel.get)
+        dom_probs = [p for p in probs if lib.dmm_gemv_kernel_name(1, p["N"], p["K"]).decode() == dom]
+        if args.no_graph:
+            return dom, dom_probs, None, "eager launches, HIP events around each kernel"
+        try:
+            gsteps = max(copies, args.graph_steps // copies * copies)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                cap = torch.cuda.current_stream().cuda_stream
+                for i in range(gsteps):
+                    for p in dom_probs:
+                        st = lib.dmm_decode_matmul_f16(p["x"].data_ptr(), p["codes"][i % copies].data_ptr(), p["grid"].data_ptr(),
+                                                       p["scale"], p["y"].data_ptr(), 1, p["N"], p["K"], cap)
+                        if st != 0:
+                            raise capi.DmmError("dmm_decode_matmul_f16", st)
+            replays = max(1, -(-args.steps // gsteps))
+            for _ in range(3):
+                g.replay()
+            torch.cuda.synchronize()
+            regs = []
+            for _ in range(max(1, args.repeats)):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(replays):
+                    g.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                regs.append(e0.elapsed_time(e1) * 1e-3 / (replays * gsteps * len(dom_probs)))
+            mode = ("HIP events around replays of a graph of this kernel's launches of the step (%d launches per replay, "
+                    "%d replays per region, median of %d regions)" % (gsteps * len(dom_probs), replays, len(regs)))
+            return dom, dom_probs, sorted(regs)[len(regs) // 2], mode
+        except Exception as e:
+            print("bench.py: roofline graph failed (%s); using the eager event timing" % e, file=sys.stderr)
+            return dom, dom_probs, None, "eager launches, HIP events around each kernel"
 
     def timed_region(run_steps):
         torch.cuda.synchronize()
@@ -194,8 +243,8 @@ def main():
 
     # the operator's own kernel choice, and the same steps with the 8-bit kernels switched off: every
     # launch in 16-bit arithmetic (half x half products, fp32 sums), the arithmetic the operator's
-    # definition states.  Each is timed over exactly args.steps steps, `--repeats` times, the regions
-    # of the two taking turns so that a drift of the clocks meets both alike; the median region counts.
+    # definition states.  Each is timed over exactly args.steps steps, `--repeats` times; the median
+    # region counts.
     run_auto, launch_mode = prepare_steps()
     was = lib.dmm_set_gemv_8bit(0)
     try:
@@ -210,14 +259,17 @@ def main():
         run_auto(12)
         torch.cuda.synchronize()
     run_auto(args.warmup)
+    regions = [timed_region(run_auto) for _ in range(max(1, args.repeats))]
+    dom, dom_probs, dom_launch_s, dom_mode = dominant_kernel_timing()
+    # The 16-bit-only variant afterwards, not in turns with the headline: regions of the two taking turns
+    # read 1.5 - 3 % slower than regions of one alone (measured), and a region right after a change of
+    # kernels slower still, hence the untimed regions first.
     if run_f16:
         run_f16(args.warmup)
-    regions, regions16 = [], []
-    for _ in range(max(1, args.repeats)):
-        regions.append(timed_region(run_auto))
-        if run_f16:
-            regions16.append(timed_region(run_f16))
-    if not run_f16:
+        for _ in range(5):
+            timed_region(run_f16)
+        regions16 = [timed_region(run_f16) for _ in range(max(1, args.repeats))]
+    else:
         was = lib.dmm_set_gemv_8bit(0)
         try:
             run_auto(args.warmup)
@@ -265,10 +317,13 @@ def main():
         k["bytes"] += workload.code_bytes(N, K) * len(v)
     # the roofline object covers the kernel that carries most of the step's bytes; all launches
     # together are in `all_gemv_launches`
-    dom = max(kernels, key=lambda n: kernels[n]["bytes"])
     kd = kernels[dom]
-    achieved = kd["bytes"] / kd["seconds"] / 1e9
+    eager_launch_us = kd["seconds"] / kd["launches"] * 1e6
     all_gbs = step_bytes * args.steps / kern_s / 1e9
+    dom_bytes_per_launch = kd["bytes"] / kd["launches"]
+    if dom_launch_s is None:
+        dom_launch_s = kd["seconds"] / kd["launches"]
+    achieved = dom_bytes_per_launch / dom_launch_s / 1e9
 
     out = {
         "metric": "batch-1 effective weight GB/s (code bytes N*K/4 per second, Llama-2-70B projection shapes)",
@@ -282,7 +337,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
-        "dtype_note": "x, grid, y and the decoded weights are halves, sums fp32; launches of two or more row tiles "
+        "dtype_note": "x, grid, y and the decoded weights are halves, sums fp32; launches of more than two row tiles "
                       "per compute unit multiply fp8 weights (exact for this grid) by x split into four bf8 terms "
                       "(exact) on the 8-bit matrix unit; value_f16_only is the same step with every launch on "
                       "half x half products",
@@ -300,8 +355,10 @@ def main():
                      "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
                      "traffic_source": GEMV_TRAFFIC_SOURCE.get(dom),
                      "kernel": dom, "launches": kd["launches"],
-                     "avg_launch_us": round(kd["seconds"] / kd["launches"] * 1e6, 3),
-                     "algorithmic_bytes_per_launch": kd["bytes"] / kd["launches"]},
+                     "avg_launch_us": round(dom_launch_s * 1e6, 3),
+                     "timing": dom_mode,
+                     "avg_launch_us_eager_events": round(eager_launch_us, 3),
+                     "algorithmic_bytes_per_launch": dom_bytes_per_launch},
         "all_gemv_launches": {"launches": n_launch, "avg_launch_us": round(kern_s / n_launch * 1e6, 3),
                               "GBps": round(all_gbs, 2), "frac_hbm": round(all_gbs / HBM_PEAK_GBS, 4),
                               "kernels": {n: {"launches": k["launches"],

@@ -3061,11 +3061,13 @@ int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale,
 bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok(M, N, K) : gemv_q8_ok<1, 16>(M, N, K); }
 
 // The choice among the matrix-vector kernels.  The 8-bit kernels where they apply and pay: one row of x
-// from two row tiles per workgroup on (measured as launches of one HIP graph on rotating code buffers,
-// 8-bit against 16-bit kernel, us per launch: 8192 -> 10240 8.0 / 8.8, 8192 -> 28672 15.5 / 17.1,
-// 28672 -> 8192 15.8 / 16.3, 4096 -> 22016 8.7 / 10.9, 8192 -> 8192 6.9 / 7.0; below two tiles the 16-bit
-// kernel wins, 5120 -> 5120 6.2 / 5.6, 11008 -> 4096 6.9 / 5.5, its prologue being the cheaper one), two to
-// four rows from more than three tiles on.  A grid that does not fit fp8 costs them a second table
+// from more than two row tiles per workgroup on, and at exactly two for long x (measured as launches of
+// one HIP graph on rotating code buffers, the two kernels taking turns, 8-bit against 16-bit kernel, us
+// per launch: 8192 -> 10240 7.9 / 8.7, 8192 -> 9216 7.9 / 8.7, 8192 -> 28672 15.3 / 16.6, 4096 -> 22016
+// 8.7 / 10.9; two tiles: 28672 -> 8192 15.5 / 16.2, 16384 -> 8192 10.4 / 10.6, 12288 -> 8192 8.5 / 8.6,
+// 8192 -> 8192 7.0 / 7.0, 4096 -> 8192 5.3 / 5.3, 5120 -> 8192 6.2 / 5.7; below two tiles the 16-bit
+// kernel wins, 5120 -> 5120 6.2 / 5.6, 11008 -> 4096 6.9 / 5.5, its prologue being the cheaper one), two
+// to four rows from more than three tiles on.  A grid that does not fit fp8 costs them a second table
 // build, and the 16-bit kernel's y is the correctly rounded one.  Otherwise the 16-bit streaming
 // kernel, one tile at a time; the register-x kernel when x does not fit the LDS.
 enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
@@ -3073,7 +3075,7 @@ enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const bool long_launch = M == 1 ? n_tiles >= 2 * cus : n_tiles > 3 * cus;
+    const bool long_launch = M == 1 ? n_tiles > 2 * cus || (n_tiles == 2 * cus && K >= 12288) : n_tiles > 3 * cus;
     if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
     if (gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
     return kGemvRegx;

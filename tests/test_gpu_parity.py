@@ -282,8 +282,9 @@ def test_gemv_8bit_switch_and_kernel_name():
     was = lib.dmm_set_gemv_8bit(1)
     try:
         assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_q8c_kernel"
-        assert lib.dmm_gemv_kernel_name(M, 8192, K) == b"dmm::gemv_q8c_kernel"        # two tiles per CU
-        assert lib.dmm_gemv_kernel_name(M, 8176, K) == b"dmm::gemv_stream_kernel"     # one short of that
+        assert lib.dmm_gemv_kernel_name(M, 8208, K) == b"dmm::gemv_q8c_kernel"        # more than two tiles per CU
+        assert lib.dmm_gemv_kernel_name(M, 8192, K) == b"dmm::gemv_stream_kernel"     # two, short x
+        assert lib.dmm_gemv_kernel_name(M, 8192, 12288) == b"dmm::gemv_q8c_kernel"    # two, long x
         assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_q8c_kernel"       # x goes through in chunks
         assert lib.dmm_gemv_kernel_name(3, N, K) == b"dmm::gemv_q8_kernel"            # two to four rows of x
         assert lib.dmm_gemv_kernel_name(3, 12288, K) == b"dmm::gemv_stream_kernel"
