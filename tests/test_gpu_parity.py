@@ -272,6 +272,21 @@ def test_gemv_8bit_random_shapes(M, N, K):
     assert torch.all(buf[:guard] == 777.0) and torch.all(buf[guard + M * N:] == 777.0)
 
 
+def test_read_probe_reads_and_leaves_its_sink_alone():
+    """The benchmark's yardstick kernel: runs on the caller's stream for short and long launches (fewer
+    tiles than compute units, several per unit, N no multiple of 16), returns DMM_OK and never writes
+    its sink for codes whose bytes do not cancel."""
+    lib = capi.lib()
+    sink = torch.full((4,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+    for N, K in ((16, 256), (1000, 512), (8192, 8192), (28672, 2048)):
+        _, codes, _, _ = workload.make_inputs(1, N, K, seed=N % 7)
+        cd = dev(codes)
+        st = lib.dmm_read_probe(cd.data_ptr(), sink.data_ptr(), N, K, torch.cuda.current_stream().cuda_stream)
+        assert st == 0, capi.status_string(st)
+    torch.cuda.synchronize()
+    assert torch.all(sink == 0x5A5A5A5A)
+
+
 def test_gemv_8bit_switch_and_kernel_name():
     """The operator's choice follows dmm_set_gemv_8bit; with the 8-bit kernel off the result is the
     16-bit kernel's, i.e. what the explicit 16-bit configuration of the same launch gives."""

@@ -64,6 +64,13 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert lib.dmm_gemv_8bit_f16(p, p, p, 1.0, p, 1, 4, 32768, None) == -5  # one row: the 16-bit hand-over does not fit
     assert lib.dmm_gemv_8bit_f16(None, p, p, 1.0, p, 1, 4, 256, None) == -1
     assert lib.dmm_gemm_f16(p, p, p, 1.0, p, 64, 4, 16, None) == -5      # K % 64 != 0
+    # the benchmark's read probe: same rules as the batch-1 kernels it stands beside
+    assert lib.dmm_read_probe(p, p, 16, 128, None) == -5                 # K % 256 != 0
+    assert lib.dmm_read_probe(p, p, 0, 256, None) == -5
+    assert lib.dmm_read_probe(p, p, 1 << 20, 1 << 14, None) == -5        # 2^32 code bytes
+    assert lib.dmm_read_probe(None, p, 16, 256, None) == -1
+    assert lib.dmm_read_probe(p, None, 16, 256, None) == -1
+    assert lib.dmm_read_probe(odd, p, 16, 256, None) == -3
     # empty problems succeed without touching the device
     assert lib.dmm_decode_f16(None, None, None, 0, 64, None) == 0
     assert lib.dmm_decode_matmul_f16(None, None, None, 1.0, None, 0, 4, 16, None) == 0
