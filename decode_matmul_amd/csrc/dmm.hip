@@ -232,6 +232,12 @@ __device__ __forceinline__ u4_t lds_read16(uint32_t byte_addr)
     return *reinterpret_cast<lds_u4_t *>(byte_addr);
 }
 
+typedef __attribute__((address_space(3))) u4_t lds_u4_rw_t;
+__device__ __forceinline__ void lds_write16(uint32_t byte_addr, const u4_t &v)
+{
+    *reinterpret_cast<lds_u4_rw_t *>(byte_addr) = v;
+}
+
 // w = g * s + d with d taken from the low (kHi = false) or high half of dd for both lanes
 template <bool kHi>
 __device__ __forceinline__ uint32_t pk_fma_bcast(uint32_t g, uint32_t s, uint32_t dd)
@@ -284,18 +290,19 @@ __device__ __forceinline__ void stream_stage_signs(unsigned char *smem, int tid)
     if (tid < 256 || tid >= 512) return;
     const int t = tid - 256, row = t >> 1;
     const u4_t sv = sign_row((uint32_t)row);
-    u4_t *sg = reinterpret_cast<u4_t *>(smem) + row * 16 + (t & 1) * 8;
+    // slot i ^ (row % 8) of the thread's eight: one exclusive or per address
+    const uint32_t sg = lds_addr(smem) + (uint32_t)((row * 16 + (t & 1) * 8 + (row & 7)) * 16);
 #pragma unroll
-    for (int i = 0; i < 8; i++) sg[(i + row) & 7] = sv;
+    for (int i = 0; i < 8; i++) lds_write16(sg ^ (uint32_t)(i * 16), sv);
 }
 
 template <int kNThreads>
 __device__ __forceinline__ void stream_stage_grid(unsigned char *smem, const u4_t &grow, int tid)
 {
     if (tid >= 256) return;
-    u4_t *gg = reinterpret_cast<u4_t *>(smem + kSSignBytes) + tid * 16;
+    const uint32_t gg = lds_addr(smem) + (uint32_t)(kSSignBytes + (tid * 16 + (tid & 15)) * 16);   // slot i ^ (tid % 16)
 #pragma unroll
-    for (int i = 0; i < 16; i++) gg[(i + tid) & 15] = grow;
+    for (int i = 0; i < 16; i++) lds_write16(gg ^ (uint32_t)(i * 16), grow);
 }
 
 // Sum over each row of 16 lanes, result in lane 15 of the row (all 64 lanes must be active).
@@ -715,8 +722,9 @@ __device__ __forceinline__ u2_t grid_row_fp8(const u4_t &row, bool &exact)
         int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * i], f[4 * i + 1], 0, false);
         p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * i + 2], f[4 * i + 3], p, true);
         r[i] = (uint32_t)p;
-        exact = exact && __builtin_amdgcn_cvt_f32_fp8(p, 0) == f[4 * i] && __builtin_amdgcn_cvt_f32_fp8(p, 1) == f[4 * i + 1] &&
-                __builtin_amdgcn_cvt_f32_fp8(p, 2) == f[4 * i + 2] && __builtin_amdgcn_cvt_f32_fp8(p, 3) == f[4 * i + 3];
+        // (no short circuit: eight compares in a row beat eight branches)
+        exact = exact & (__builtin_amdgcn_cvt_f32_fp8(p, 0) == f[4 * i]) & (__builtin_amdgcn_cvt_f32_fp8(p, 1) == f[4 * i + 1]) &
+                (__builtin_amdgcn_cvt_f32_fp8(p, 2) == f[4 * i + 2]) & (__builtin_amdgcn_cvt_f32_fp8(p, 3) == f[4 * i + 3]);
     }
     return r;
 }
@@ -895,9 +903,9 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
         // 8 slots of row t / 2 (16 neighbouring lanes hit 16 different slot positions)
         const int t = tid - 256, row = t >> 1;
         const u2_t sb = sign_bytes((uint32_t)row);
-        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw) + row * 16 + (t & 1) * 8;
+        const uint32_t sg = lds_addr(smem_raw) + (uint32_t)((row * 16 + (t & 1) * 8 + (row & 7)) * 16);   // slot i ^ (row % 8)
 #pragma unroll
-        for (int i = 0; i < 8; i++) sg[(i + row) & 7] = u4_t{sb[0], sb[1], sb[0], sb[1]};
+        for (int i = 0; i < 8; i++) lds_write16(sg ^ (uint32_t)(i * 16), u4_t{sb[0], sb[1], sb[0], sb[1]});
     }
     __builtin_amdgcn_sched_barrier(0);   // keep the sign rows ahead of the waits for the loads
 
@@ -924,9 +932,9 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restr
         bool exact;
         const u2_t g8 = grid_row_fp8(grow, exact);
         fits = fits && exact;
-        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes) + tid * 16;
+        const uint32_t gg = lds_addr(smem_raw) + (uint32_t)(kSSignBytes + (tid * 16 + (tid & 15)) * 16);   // slot i ^ (tid % 16)
 #pragma unroll
-        for (int i = 0; i < 16; i++) gg[(i + tid) & 15] = u4_t{g8[0], g8[1], g8[0], g8[1]};
+        for (int i = 0; i < 16; i++) lds_write16(gg ^ (uint32_t)(i * 16), u4_t{g8[0], g8[1], g8[0], g8[1]});
     }
     // the vote: every wave publishes whether one of its rows or pieces failed, in a word of its own (so
     // nothing needs clearing first), and after the barrier every wave reads all of them
@@ -1099,7 +1107,11 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
     const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
     const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
     const int n_groups = (t1 - t0 + T - 1) / T;
-    const int g_base = (t1 - t0) / n_groups, g_rem = (t1 - t0) % n_groups;
+    // (t1 - t0) / n_groups without a division, which would stand between the kernel's start and its first loads:
+    // with T = 3 the groups of two or more are of 2 or 3 tiles, of 3 only if all are
+    static_assert(T == 3, "the group sizes below are those of T = 3");
+    const int g_base = n_groups <= 1 ? t1 - t0 : (t1 - t0 == 3 * n_groups ? 3 : 2);
+    const int g_rem = n_groups <= 1 ? 0 : t1 - t0 - g_base * n_groups;
     const int total = n_groups * n_chunks;   // chunks to go through, over all groups
 
     const int n_tiles_all = (N + 15) >> 4;
@@ -1152,17 +1164,18 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
         // 8 slots of row t / 2 (16 neighbouring lanes hit 16 different slot positions)
         const int t = tid - 768, row = t >> 1;
         const u2_t sb = sign_bytes((uint32_t)row);
-        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw) + row * 16 + (t & 1) * 8;
+        // slot i ^ (row % 8) of the thread's eight: one exclusive or per address
+        const uint32_t sg = lds_addr(smem_raw) + (uint32_t)((row * 16 + (t & 1) * 8 + (row & 7)) * 16);
 #pragma unroll
-        for (int i = 0; i < 8; i++) sg[(i + row) & 7] = u4_t{sb[0], sb[1], sb[0], sb[1]};
+        for (int i = 0; i < 8; i++) lds_write16(sg ^ (uint32_t)(i * 16), u4_t{sb[0], sb[1], sb[0], sb[1]});
     } else if (wave >= 8) {
         bool exact;
         const u2_t g8 = grid_row_fp8(grow, exact);
         fits = exact;
         const int r = tid - 512;
-        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes) + r * 16;
+        const uint32_t gg = lds_addr(smem_raw) + (uint32_t)(kSSignBytes + (r * 16 + (r & 15)) * 16);   // slot i ^ (r % 16)
 #pragma unroll
-        for (int i = 0; i < 16; i++) gg[(i + r) & 15] = u4_t{g8[0], g8[1], g8[0], g8[1]};
+        for (int i = 0; i < 16; i++) lds_write16(gg ^ (uint32_t)(i * 16), u4_t{g8[0], g8[1], g8[0], g8[1]});
     } else {
         fits = stage_piece(xpiece, 0, tid);
     }
@@ -2329,9 +2342,10 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
                 if ((s8 >> d) & 1u) v ^= 0xFCull << (8 * d);
         }
         const uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
-        u4_t *rowp = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;   // tid >= 256 lands in the mask table
+        // tid >= 256 lands in the mask table; slot i ^ (tid % 16): 16 lanes, 16 bank groups, one exclusive or per address
+        const uint32_t rowp = lds_addr(smem_raw) + (uint32_t)((tid * 16 + (tid & 15)) * 16);
 #pragma unroll
-        for (int i = 0; i < 16; i++) rowp[(i + tid) & 15] = u4_t{lo, hi, lo, hi};   // 16 lanes, 16 bank groups
+        for (int i = 0; i < 16; i++) lds_write16(rowp ^ (uint32_t)(i * 16), u4_t{lo, hi, lo, hi});
     }
     // the vote on the table: one word per wave in the partial-sum area, read by everybody after the barrier
     uint32_t *votes = reinterpret_cast<uint32_t *>(smem_raw + 2 * kI8TableBytes);
