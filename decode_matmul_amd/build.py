@@ -49,7 +49,8 @@ def hipcc_path():
 
 
 def build_lib(verbose=False):
-    """hipcc: csrc/dmm.hip -> libdmm.so (gfx950 code object + the extern "C" entry points)."""
+    """hipcc: csrc/dmm.hip (which includes the dmm_*.h kernel files beside it) -> libdmm.so
+    (gfx950 code object + the extern "C" entry points)."""
     cmd = [hipcc_path()] + HIPCC_FLAGS + ["-Rpass-analysis=kernel-resource-usage",
                                           "-I" + INCLUDE, "-o", LIB_PATH, os.path.join(CSRC, "dmm.hip")]
     out = _run(cmd)
@@ -66,15 +67,19 @@ def build_lib(verbose=False):
     if spilled:
         os.remove(LIB_PATH)
         raise RuntimeError("kernels spill registers to scratch memory: %s" % ", ".join(spilled))
-    rest, skip = [], 0
-    for line in out.splitlines():   # drop the remarks and the two source-context lines after each
+    rest, held, skip = [], [], 0
+    for line in out.splitlines():   # drop the remarks, the include trail ahead of each and the
+        if line.startswith("In file included from "):   # two source-context lines after it
+            held.append(line)
+            continue
         if "-Rpass-analysis=kernel-resource-usage" in line:
-            skip = 2
+            held, skip = [], 2
         elif skip and re.match(r"^\s*\d*\s*\|", line):
             skip -= 1
         else:
             skip = 0
-            rest.append(line)
+            rest += held + [line]
+            held = []
     rest = "\n".join(rest)
     if verbose and rest.strip():
         print(rest)

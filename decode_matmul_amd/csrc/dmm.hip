@@ -11,6 +11,18 @@
 // whose result registers are, unchanged, the 8-halves-per-lane operand of the
 // 16x16x32 / 32x32x16 half MFMA.  Nothing decoded ever goes back through memory on the
 // matrix-vector path.
+//
+// This file is the one translation unit of the library: shared types, then the kernel files
+// beside it (each included once, inside namespace dmm, in dependency order), then the
+// extern "C" entry points.
+//   dmm_tables.h      decode tables, decode of one code, standalone decoder, catch-all operator
+//   dmm_gemv_f16.h    matrix-vector helpers and the streaming kernel on 16-bit operands
+//   dmm_gemv_q8.h     matrix-vector kernels on 8-bit operands (fp8 weights, bf8 terms of x)
+//   dmm_gemv_small.h  small-batch kernel with x in registers
+//   dmm_gemm.h        matrix-matrix kernels and the split-K reduction
+//   dmm_int8.h        the reference's integer operator
+//   dmm_aux.h         offline repack, read probe
+//   dmm_host.h        library scratch memory, launch plumbing, set-up, checks and dispatch
 #include <hip/hip_runtime.h>
 #include <atomic>
 #include <mutex>
@@ -38,3335 +50,14 @@ typedef int i8_t __attribute__((ext_vector_type(8)));
 
 constexpr int kWave = 64;
 
-
-// ------------------------------------------------------------------ decode tables in LDS
-struct DecodeTables {
-    u4_t grid[256];   // row i: 8 halves of grid[i][0..7]
-    u4_t sign[128];   // row s: 8 halves, +-1.0, dim d negative iff bit d of (s | parity(s) << 7)
-};
-
-__device__ __forceinline__ u4_t sign_row(uint32_t s7)
-{
-    const uint32_t s8 = s7 | ((__builtin_popcount(s7) & 1u) << 7);
-    u4_t r;
-#pragma unroll
-    for (int i = 0; i < 4; i++)   // +-1.0 = 0x3C00 with the sign bit of dim 2i (low half) / 2i+1 (high half)
-        r[i] = 0x3C003C00u | (((s8 >> (2 * i)) & 1u) << 15) | (((s8 >> (2 * i + 1)) & 1u) << 31);
-    return r;
-}
-
-// Fill the tables with `nthreads` threads (tid in [0, nthreads)).  grid16 tells whether the
-// global grid pointer may be read 16 bytes at a time.
-template <bool kAligned>
-__device__ __forceinline__ void stage_tables(DecodeTables &t, const void *grid, int tid, int nthreads)
-{
-    for (int i = tid; i < 256; i += nthreads) {
-        if (kAligned) {
-            t.grid[i] = reinterpret_cast<const u4_t *>(grid)[i];
-        } else {
-            const uint16_t *g = reinterpret_cast<const uint16_t *>(grid) + i * 8;
-            u4_t r;
-#pragma unroll
-            for (int j = 0; j < 4; j++) r[j] = (uint32_t)g[2 * j] | ((uint32_t)g[2 * j + 1] << 16);
-            t.grid[i] = r;
-        }
-    }
-    for (int i = tid; i < 128; i += nthreads) t.sign[i] = sign_row((uint32_t)i);
-}
-
-__device__ __forceinline__ h2_t as_h2(uint32_t v) { return __builtin_bit_cast(h2_t, v); }
-__device__ __forceinline__ uint32_t as_u32(h2_t v) { return __builtin_bit_cast(uint32_t, v); }
-
-// Decode one code (low 16 bits of c) into 8 halves = 4 packed registers.
-__device__ __forceinline__ u4_t decode8(uint32_t c, const DecodeTables &t)
-{
-    u4_t g = t.grid[c & 0xFFu];
-    u4_t s = t.sign[(c >> 8) & 0x7Fu];
-    uint32_t db = ((c & 0x8000u) * 0x10001u) | 0x34003400u;   // packed (+-0.25, +-0.25)
-    h2_t d = as_h2(db);
-    u4_t w;
-#pragma unroll
-    for (int i = 0; i < 4; i++) w[i] = as_u32(__builtin_elementwise_fma(as_h2(g[i]), as_h2(s[i]), d));
-    return w;
-}
-
-// Two codes packed in one 32-bit word (low half = first code).
-__device__ __forceinline__ void decode8x2(uint32_t w, const DecodeTables &t, u4_t &w0, u4_t &w1)
-{
-    u4_t g0 = t.grid[w & 0xFFu];
-    u4_t s0 = t.sign[(w >> 8) & 0x7Fu];
-    u4_t g1 = t.grid[(w >> 16) & 0xFFu];
-    u4_t s1 = t.sign[(w >> 24) & 0x7Fu];
-    uint32_t db = (w & 0x80008000u) | 0x34003400u;            // delta of code 0 | delta of code 1 << 16
-    h2_t d0 = as_h2((db & 0xFFFFu) * 0x10001u);
-    h2_t d1 = as_h2((db >> 16) * 0x10001u);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        w0[i] = as_u32(__builtin_elementwise_fma(as_h2(g0[i]), as_h2(s0[i]), d0));
-        w1[i] = as_u32(__builtin_elementwise_fma(as_h2(g1[i]), as_h2(s1[i]), d1));
-    }
-}
-
-// ------------------------------------------------------------------ standalone decoder
-// Flat: code i -> halves [8i, 8i+8).  kAligned: each thread takes 8 codes with one
-// 16-byte load and issues eight 16-byte stores; otherwise one code per thread.
-template <bool kAligned>
-__global__ __launch_bounds__(256) void decode_kernel(const uint16_t *__restrict__ codes,
-                                                     const void *__restrict__ grid,
-                                                     uint16_t *__restrict__ W, int64_t n_codes)
-{
-    __shared__ DecodeTables tab;
-    stage_tables<kAligned>(tab, grid, threadIdx.x, 256);
-    __syncthreads();
-    if (kAligned) {
-        // a wave covers 64 consecutive 32-bit words per step: loads are 256 B per wave,
-        // stores 2 KiB per wave, both contiguous.
-        const int64_t n_words = n_codes >> 1;
-        const uint32_t *cw = reinterpret_cast<const uint32_t *>(codes);
-        u4_t *out = reinterpret_cast<u4_t *>(W);
-        for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_words; i += (int64_t)gridDim.x * 256) {
-            u4_t w0, w1;
-            decode8x2(cw[i], tab, w0, w1);
-            out[2 * i] = w0;
-            out[2 * i + 1] = w1;
-        }
-        if ((n_codes & 1) && blockIdx.x == 0 && threadIdx.x == 0)
-            out[n_codes - 1] = decode8(codes[n_codes - 1], tab);
-    } else {
-        for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_codes; i += (int64_t)gridDim.x * 256) {
-            u4_t w = decode8(codes[i], tab);
-            uint16_t *o = W + i * 8;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                o[2 * j] = (uint16_t)(w[j] & 0xFFFFu);
-                o[2 * j + 1] = (uint16_t)(w[j] >> 16);
-            }
-        }
-    }
-}
-
-// ------------------------------------------------------------------ generic operator path
-// One wave per output row n, lanes stride over the row's codes, dot products on the
-// vector ALU with fp32 accumulation, DPP/shuffle reduction across the wave.  Handles any
-// M, N, K % 8 == 0 and 2-byte alignment; M is processed in chunks of kMC rows of x.
-constexpr int kGenericMC = 4;
-
-__device__ __forceinline__ float wave_sum(float v)
-{
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-
-__global__ __launch_bounds__(256) void generic_kernel(const uint16_t *__restrict__ x,
-                                                      const uint16_t *__restrict__ codes,
-                                                      const void *__restrict__ grid, float scale,
-                                                      uint16_t *__restrict__ y, int64_t M, int64_t N,
-                                                      int64_t K)
-{
-    __shared__ DecodeTables tab;
-    stage_tables<false>(tab, grid, threadIdx.x, 256);
-    __syncthreads();
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int64_t kc = K >> 3;
-    for (int64_t n = (int64_t)blockIdx.x * 4 + wave; n < N; n += (int64_t)gridDim.x * 4) {
-        const uint16_t *crow = codes + n * kc;
-        for (int64_t m0 = 0; m0 < M; m0 += kGenericMC) {
-            float acc[kGenericMC] = {};
-            for (int64_t j = lane; j < kc; j += kWave) {
-                u4_t w = decode8(crow[j], tab);
-                float wf[8];
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    h2_t p = as_h2(w[i]);
-                    wf[2 * i] = (float)p[0];
-                    wf[2 * i + 1] = (float)p[1];
-                }
-#pragma unroll
-                for (int mm = 0; mm < kGenericMC; mm++) {
-                    if (m0 + mm < M) {
-                        const uint16_t *xr = x + (m0 + mm) * K + j * 8;
-#pragma unroll
-                        for (int d = 0; d < 8; d++) {
-                            half_t xv = __builtin_bit_cast(half_t, xr[d]);
-                            acc[mm] = __builtin_fmaf((float)xv, wf[d], acc[mm]);
-                        }
-                    }
-                }
-            }
-#pragma unroll
-            for (int mm = 0; mm < kGenericMC; mm++) {
-                float s = wave_sum(acc[mm]);
-                if (lane == 0 && m0 + mm < M) {
-                    half_t h = (half_t)(s * scale);
-                    y[(m0 + mm) * N + n] = __builtin_bit_cast(uint16_t, h);
-                }
-            }
-        }
-    }
-}
-
-// ------------------------------------------------------------------ matrix-vector paths (M <= 32)
-// A workgroup owns 16*R consecutive rows of W for the whole of K; its W waves split K in
-// interleaved 256-wide steps.  In one step a lane (row r = lane%16 of each 16-row tile,
-// quarter q = lane/16) loads 8 consecutive codes (16 bytes) of its row, decodes them one at a
-// time and feeds each as the A operand (16 rows x 32 k: this lane supplies the 8 k of its
-// quarter) of v_mfma_f32_16x16x32_f16.  The B operand is x: column c = lane%16 is row m = c of
-// x, same 8 k.  Any k order works as long as A and B agree, so the 32 k of MFMA number t in a
-// step are {64*q + 8*t .. +8 : q = 0..3} rather than 32 consecutive k; that is what lets the
-// code load be one 16-byte load per lane.  For M = 1 only column 0 carries data, the other 15
-// columns cost nothing extra: the matrix unit has the headroom.
-// Accumulator layout: lane holds rows 4*q + i (i = 0..3) of column c, i.e.
-// y[m = c][n = n0 + 4*q + i] - four consecutive halves of a row of y.
-typedef __attribute__((address_space(3))) const u4_t lds_u4_t;
-
-// 32-bit LDS byte address of a pointer into shared memory
-__device__ __forceinline__ uint32_t lds_addr(const void *p)
-{
-    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
-}
-
-__device__ __forceinline__ u4_t lds_read16(uint32_t byte_addr)
-{
-    return *reinterpret_cast<lds_u4_t *>(byte_addr);
-}
-
-typedef __attribute__((address_space(3))) u4_t lds_u4_rw_t;
-__device__ __forceinline__ void lds_write16(uint32_t byte_addr, const u4_t &v)
-{
-    *reinterpret_cast<lds_u4_rw_t *>(byte_addr) = v;
-}
-
-// w = g * s + d with d taken from the low (kHi = false) or high half of dd for both lanes
-template <bool kHi>
-__device__ __forceinline__ uint32_t pk_fma_bcast(uint32_t g, uint32_t s, uint32_t dd)
-{
-    uint32_t r;
-    if (kHi)
-        asm("v_pk_fma_f16 %0, %1, %2, %3 op_sel:[0,0,1] op_sel_hi:[1,1,1]" : "=v"(r) : "v"(g), "v"(s), "v"(dd));
-    else
-        asm("v_pk_fma_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,1,0]" : "=v"(r) : "v"(g), "v"(s), "v"(dd));
-    return r;
-}
-
-// ------------------------------------------------------------------ streaming matrix-vector path
-// The batch-1 path proper (small M, x small enough to live in LDS).  Two facts shape it: HBM
-// answers in a few microseconds under load, so a CU must keep tens of KB of code bytes
-// outstanding at all times, and vector-memory results return in order, so any x load queued
-// behind the code prefetch would stall until the whole prefetch had landed.  Hence:
-//   * x is copied once per workgroup into LDS (row pitch 2K + 16 bytes, so the rows read
-//     together fall in different bank groups) and B operands are read from there;
-//   * the code stream is a ring of D register buffers per wave, refilled with raw buffer
-//     loads: the per-lane part of the address never changes, everything that moves (row
-//     block, k step) is in the scalar offset, and past the end that offset is out of range,
-//     which the hardware answers with zeros - no branch around any vector-memory
-//     instruction, so the wait counters stay exact and D * R loads per wave stay in flight;
-//   * workgroups are persistent (one per CU) and walk over row blocks, so the tables and x
-//     are staged once and the prefetch runs across row-block boundaries;
-//   * the LDS serves 16 lanes of a 16-byte gather per clock, so the decode tables hold 16
-//     copies of every row (row pitch 256 bytes, lane reads copy lane % 16): conflict-free for
-//     any codes.  A table address is one v_perm_b32: a byte of the code word placed above
-//     the lane's copy offset.
-// LDS map: [0, 32K) sign rows (128 x 256 B), [32K, 96K) grid rows (256 x 256 B),
-//          then 2 x (W x R x 4 x M) float4 partial sums (double-buffered per row block), then x.
-
-constexpr int kSSignBytes = 128 * 256;
-constexpr int kSGridBytes = 256 * 256;
-constexpr int kSTablesBytes = kSSignBytes + kSGridBytes;
-
-__host__ __device__ constexpr int stream_red_bytes(int R, int W, int M) { return 2 * W * R * 4 * M * 16; }
-
-// Table staging.  Every instruction of the prologue is paid once per wave that runs it, so the
-// two tables go to different waves instead of a share of each to every thread: the first 256
-// threads (waves 0-3) fetch one grid row each and write its 16 copies, the next 256 (waves 4-7)
-// compute the sign rows (thread t: row t / 2, 8 of its 16 copies; needs no load, so it runs
-// while the loads are in flight).  16 neighbouring lanes always write 16 different copy
-// positions, i.e. 16 bank groups.
-template <int kNThreads>
-__device__ __forceinline__ void stream_stage_signs(unsigned char *smem, int tid)
-{
-    static_assert(kNThreads >= 512, "staging assumes at least 8 waves");
-    if (tid < 256 || tid >= 512) return;
-    const int t = tid - 256, row = t >> 1;
-    const u4_t sv = sign_row((uint32_t)row);
-    // slot i ^ (row % 8) of the thread's eight: one exclusive or per address
-    const uint32_t sg = lds_addr(smem) + (uint32_t)((row * 16 + (t & 1) * 8 + (row & 7)) * 16);
-#pragma unroll
-    for (int i = 0; i < 8; i++) lds_write16(sg ^ (uint32_t)(i * 16), sv);
-}
-
-template <int kNThreads>
-__device__ __forceinline__ void stream_stage_grid(unsigned char *smem, const u4_t &grow, int tid)
-{
-    if (tid >= 256) return;
-    const uint32_t gg = lds_addr(smem) + (uint32_t)(kSSignBytes + (tid * 16 + (tid & 15)) * 16);   // slot i ^ (tid % 16)
-#pragma unroll
-    for (int i = 0; i < 16; i++) lds_write16(gg ^ (uint32_t)(i * 16), grow);
-}
-
-// Sum over each row of 16 lanes, result in lane 15 of the row (all 64 lanes must be active).
-template <int kCtrl>
-__device__ __forceinline__ float dpp_shr_add(float v)
-{
-    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xF, 0xF, true));
-}
-__device__ __forceinline__ float row_sum16(float v)
-{
-    v = dpp_shr_add<0x118>(v);   // row_shr:8, lanes shifted in from outside the row read 0
-    v = dpp_shr_add<0x114>(v);   // row_shr:4
-    v = dpp_shr_add<0x112>(v);   // row_shr:2
-    return dpp_shr_add<0x111>(v);   // row_shr:1
-}
-
-// (a & m) | (b & ~m) in one instruction
-__device__ __forceinline__ uint32_t bfi(uint32_t m, uint32_t a, uint32_t b)
-{
-    uint32_t r;
-    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(r) : "s"(m), "v"(a), "v"(b));
-    return r;
-}
-
-struct StreamGather {
-    u4_t g0, s0, g1, s1;
-    uint32_t dd;
-};
-
-// lane_base = (lane % 16) * 16; the tables start at LDS address 0
-__device__ __forceinline__ void stream_gather(StreamGather &o, uint32_t w, uint32_t lane_base, uint32_t quarter_bits)
-{
-    const uint32_t w7 = w & 0x7FFF7FFFu;                 // sign-row index must not see the shift bit
-    o.g0 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u) + kSSignBytes);
-    o.s0 = lds_read16(__builtin_amdgcn_perm(w7, lane_base, 0x0C0C0500u));
-    o.g1 = lds_read16(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u) + kSSignBytes);
-    o.s1 = lds_read16(__builtin_amdgcn_perm(w7, lane_base, 0x0C0C0700u));
-    o.dd = bfi(0x7FFF7FFFu, quarter_bits, w);            // (+-0.25, +-0.25): signs from the shift bits
-}
-
-template <bool kHi>
-__device__ __forceinline__ h8_t stream_finish(const u4_t &g, const u4_t &sg, uint32_t dd)
-{
-    u4_t r;
-#pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = pk_fma_bcast<kHi>(g[i], sg[i], dd);
-    return __builtin_bit_cast(h8_t, r);
-}
-
-// One 256-wide k step for the first nv (uniform, 1 <= nv <= R) of R row tiles.  Items (word
-// t2 of row tile r) run t2-major; the gathers of item i+1 are issued before the math of item i.
-// Tiles past nv are skipped by uniform branches around their gathers and their math.
-//
-// The B operand.  A lane's 8 codes of the step feed 8 MFMAs (i = 0 .. 7), and MFMA i needs the
-// 16-byte piece i of the lane quarter's 128 bytes of x in the lanes of ONE column per x row.
-// JP = 1: column m holds row m (M <= 16) and every MFMA reads its piece, 8 wave-wide LDS reads
-// per step, a third of the kernel's LDS traffic for one useful lane in 16.  JP = 4 (M <= 4):
-// column 4 m + j holds piece 4 s + j of row m in register set s, so TWO reads fetch the whole
-// step; MFMA i multiplies by set i / 4, and since its other columns hold the pieces of other
-// MFMAs, MFMA i adds into accumulator i % 4, of which only the columns 4 m + i % 4 are ever
-// looked at (finish_block adds column 4 m + j of accumulator j over j).  Lanes of columns past
-// 4 M read zeros.
-template <int JP>
-struct StreamB {
-    static constexpr int kAcc = JP == 1 ? 2 : JP;   // accumulators per row tile
-};
-
-template <int R, int JP>
-__device__ __forceinline__ void stream_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t lane_base,
-                                            uint32_t quarter_bits, f4_t (&acc)[R][StreamB<JP>::kAcc], int nv)
-{
-    constexpr int kItems = 4 * R;
-    StreamGather buf[2];
-    constexpr int kSets = JP == 1 ? 4 : 8 / JP;
-    u4_t xb[kSets];
-    if constexpr (JP == 1) {
-        xb[0] = lds_read16(xaddr);
-        xb[1] = lds_read16(xaddr + 16);
-    } else {
-#pragma unroll
-        for (int s = 0; s < kSets; s++) xb[s] = lds_read16(xaddr + s * JP * 16);
-    }
-    stream_gather(buf[0], cw[0][0], lane_base, quarter_bits);
-#pragma unroll
-    for (int i = 0; i < kItems; i++) {
-        const int t2 = i / R, r = i % R;
-        if (i + 1 < kItems) {
-            const int nt2 = (i + 1) / R, nr = (i + 1) % R;
-            if (nr == 0) {
-                if constexpr (JP == 1) {
-                    xb[(nt2 & 1) * 2] = lds_read16(xaddr + nt2 * 32);
-                    xb[(nt2 & 1) * 2 + 1] = lds_read16(xaddr + nt2 * 32 + 16);
-                }
-                stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
-            } else if (nr < nv) {
-                stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
-            }
-        }
-        if (r == 0 || r < nv) {
-            // 4 packed FMAs, MFMA, 4 packed FMAs, MFMA: the second group and the next item's
-            // address math run in the shadow of the matrix unit
-            const StreamGather &b = buf[i & 1];
-            constexpr int kA = StreamB<JP>::kAcc;
-            const int i0 = 2 * t2, i1 = 2 * t2 + 1;
-            const u4_t &b0 = JP == 1 ? xb[(t2 & 1) * 2] : xb[i0 / JP];
-            const u4_t &b1 = JP == 1 ? xb[(t2 & 1) * 2 + 1] : xb[i1 / JP];
-            const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
-            acc[r][i0 % kA] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, b0), acc[r][i0 % kA], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
-            acc[r][i1 % kA] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, b1), acc[r][i1 % kA], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-}
-
-// v + (the value of the lane kShl places up the row of 16)
-template <int kShl>
-__device__ __forceinline__ float dpp_shl_add(float v, float w)
-{
-    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, w), 0x100 + kShl, 0xF, 0xF, true));
-}
-
-// bytes of the LDS copy of x: M padded rows and 128 bytes of zeros behind them (the B operand
-// of the columns that hold no x)
-__host__ __device__ constexpr int64_t stream_x_bytes(int64_t M, int64_t K) { return M * (2 * K + 16) + 128; }
-
-template <int R, int W, int D, bool kPacked, int JP>
-__device__ __forceinline__ void gemv_stream_body(const uint16_t *__restrict__ x, const uint16_t *__restrict__ codes,
-                                                 const void *__restrict__ grid, float scale,
-                                                 uint16_t *__restrict__ y, int M, int N, int K, int tiles_q,
-                                                 int tiles_r)
-{
-    static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
-    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // [2][W][R][4 * M]
-    const int red_par = W * R * 4 * M;                                 // float4 per parity
-    unsigned char *xs = smem_raw + kSTablesBytes + stream_red_bytes(R, W, M);
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: offsets derived from it live in SGPRs
-    const int c16 = lane & 15;
-    const int q = lane >> 4;
-    const int n_steps = K >> 8;
-    const int row_bytes = K >> 2;
-    const int x_pitch = 2 * K + 16;
-    const uint32_t lane_base = (uint32_t)c16 * 16u;
-    const uint32_t quarter_bits = 0x34003400u;
-
-    // ---- prologue: this thread's grid row and its share of x first (short latency, nothing
-    // queued in front of them), then the first D items of the code stream; the tables and the
-    // LDS copy of x are built while the code loads fly ---------------------------------------
-    const u4_t grow = tid < 256 ? reinterpret_cast<const u4_t *>(grid)[tid] : u4_t{0u, 0u, 0u, 0u};   // waves 0-3 stage the grid
-    const int row_chunks = K >> 3;                     // 16-byte pieces per row of x
-    const int n_pieces = M * row_chunks;               // x is [M][K] contiguous: piece p sits at x + 16 p
-    // pieces of x per thread fetched up front, before the code loads are queued: vector-memory results
-    // return in order, so a piece asked for later arrives behind the whole first burst of codes.  One
-    // row of x: up to four pieces (all of it for K <= 32768); more rows: up to six (all of x for M <= 4 at
-    // K = 11008).
-    constexpr int kXPer = 6, kXPer1 = 4;
-    u4_t xv[kXPer];
-#pragma unroll
-    for (int u = 0; u < kXPer; u++) {
-        const int p = u * 64 * W + tid;
-        xv[u] = p < n_pieces && (u < kXPer1 || M > 1) ? reinterpret_cast<const u4_t *>(x)[p] : u4_t{0u, 0u, 0u, 0u};
-    }
-
-    const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;   // k steps of this wave per row block
-    // this workgroup's share of the 16-row tiles: a contiguous range, tiles_q tiles plus one
-    // more for the first tiles_r workgroups (quotient and remainder of tiles / workgroups, from
-    // the host), walked R tiles (one row block) at a time; the last block may be partial
-    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
-    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
-    const int nb_wg = (t1 - t0 + R - 1) / R;
-
-    // Row-major codes [N][K/8]: a lane's 16 bytes are 8 codes of its row, a wave's load touches
-    // 16 rows x 64 bytes.  Packed codes (pack_kernel): the same 16 bytes sit at
-    // ((tile * n_steps + step) * 64 + lane) * 16, so a wave's load is 1 KB of consecutive bytes.
-    const int n_tiles_all = (N + 15) >> 4;
-    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_tiles_all * 16 : N) * row_bytes), 0x00020000);
-    // per-lane byte offset inside a row block (never changes) ...
-    int voff[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) voff[r] = kPacked ? lane * 16 + r * n_steps * 1024 : (16 * r + c16) * row_bytes + q * 16;
-    // ... and the scalar part: first tile and k step of the next item to prefetch.  Rows past N
-    // land past the end of the buffer by themselves (row-major) or are zero padding (packed);
-    // items past the end get an offset no buffer reaches.
-    constexpr int kOut = (int)0x80000000;
-    int pf_blk = 0, pf_j = 0;
-    auto issue = [&](u4_t (&cwd)[R]) {
-        const bool ok = pf_blk < nb_wg && n_sw > 0;
-        const int tb = t0 + pf_blk * R;
-        const int soff = !ok ? kOut
-                         : kPacked ? (tb * n_steps + wave + pf_j * W) * 1024
-                                   : tb * 16 * row_bytes + (wave + pf_j * W) * 64;
-#pragma unroll
-        for (int r = 0; r < R; r++)   // tiles of a partial block that belong to the next workgroup: no access
-            cwd[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], (r == 0 || tb + r < t1) ? soff : kOut, 0);
-        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
-    };
-
-    u4_t cw[D][R];
-#pragma unroll
-    for (int d = 0; d < D; d++) issue(cw[d]);
-    stream_stage_signs<64 * W>(smem_raw, tid);
-    __builtin_amdgcn_sched_barrier(0);   // keep the sign rows ahead of the waits for the loads
-
-    // x -> LDS (row m at m * x_pitch): the pieces fetched above, then whatever is left
-    if (M == 1) {
-#pragma unroll
-        for (int u = 0; u < kXPer1; u++) {
-            const int c = u * 64 * W + tid;
-            if (c < row_chunks) reinterpret_cast<u4_t *>(xs)[c] = xv[u];
-        }
-        for (int c = kXPer1 * 64 * W + tid; c < row_chunks; c += 64 * W)
-            reinterpret_cast<u4_t *>(xs)[c] = reinterpret_cast<const u4_t *>(x)[c];
-    } else {
-        int m = 0, c = tid;   // piece p = m * row_chunks + c
-#pragma unroll
-        for (int u = 0; u < kXPer; u++) {
-            while (c >= row_chunks) { c -= row_chunks; m++; }
-            if (m < M) reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = xv[u];
-            c += 64 * W;
-        }
-        for (int p = kXPer * 64 * W + tid; p < n_pieces; p += 64 * W) {
-            while (c >= row_chunks) { c -= row_chunks; m++; }
-            reinterpret_cast<u4_t *>(xs + m * x_pitch)[c] = reinterpret_cast<const u4_t *>(x)[p];
-            c += 64 * W;
-        }
-    }
-    if (tid >= 64 * W - 8) reinterpret_cast<u4_t *>(xs + M * x_pitch)[tid - (64 * W - 8)] = u4_t{0u, 0u, 0u, 0u};
-    stream_stage_grid<64 * W>(smem_raw, grow, tid);
-    __syncthreads();
-
-    // B operand address of this lane.  JP = 1: row m = c16 (row 0 for columns past M), quarter
-    // q.  JP = 4: column c16 = 4 m + j reads piece j (and 4 + j) of row m's quarter; columns past
-    // 4 M read the zeros behind x, at every step (their step stride is 0).
-    constexpr int kAcc = StreamB<JP>::kAcc;
-    const bool col_live = JP == 1 || c16 / JP < M;
-    const uint32_t xlane = JP == 1    ? lds_addr(xs) + (uint32_t)((c16 < M ? c16 : 0) * x_pitch + q * 128)
-                           : col_live ? lds_addr(xs) + (uint32_t)((c16 / JP) * x_pitch + q * 128 + (c16 % JP) * 16)
-                                      : lds_addr(xs) + (uint32_t)(M * x_pitch);
-    const uint32_t xstride = col_live ? 512u : 0u;
-
-    f4_t acc[R][kAcc];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int a = 0; a < kAcc; a++) acc[r][a] = f4_t{0.f, 0.f, 0.f, 0.f};
-
-    // publish this wave's partial sums of a finished row block, meet the other waves, add up
-    // and store
-    auto finish_block = [&](int blk) {
-        f4_t *rp = red + (blk & 1) * red_par;
-        if constexpr (JP == 1) {
-            if (c16 < M) {
-#pragma unroll
-                for (int r = 0; r < R; r++) rp[(wave * R + r) * 4 * M + q * M + c16] = acc[r][0] + acc[r][1];
-            }
-        } else {
-            // column 4 m + j of accumulator j, added over j into the lane of column 4 m
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                f4_t v = acc[r][0];
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    v[e] = dpp_shl_add<1>(v[e], acc[r][1][e]);
-                    v[e] = dpp_shl_add<2>(v[e], acc[r][2][e]);
-                    v[e] = dpp_shl_add<3>(v[e], acc[r][3][e]);
-                }
-                if (c16 % JP == 0 && c16 / JP < M) rp[(wave * R + r) * 4 * M + q * M + c16 / JP] = v;
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < R; r++)
-#pragma unroll
-            for (int a = 0; a < kAcc; a++) acc[r][a] = f4_t{0.f, 0.f, 0.f, 0.f};
-        __syncthreads();
-        // (row tile r, x row m) pairs go round the waves; lane (w = lane % 16, quarter lane / 16)
-        // fetches ONE partial sum, wave w's, and the 16 of a row of lanes are added with DPP
-        // shifts: a single LDS round trip instead of a chain of W dependent ones
-        for (int p = wave; p < R * M; p += W) {
-            const int r = M == 1 ? p : p / M, m = p - r * M;
-            f4_t v = f4_t{0.f, 0.f, 0.f, 0.f};
-            if (c16 < W) v = rp[(c16 * R + r) * 4 * M + q * M + m];
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
-            const int tile = t0 + blk * R + r;
-            const int n = tile * 16 + 4 * q;
-            if (c16 == 15 && tile < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
-                h4_t o;
-#pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
-                *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
-            }
-        }
-    };
-
-    if (n_sw == 0) {
-        // no k step for this wave (K shorter than the workgroup is wide): it still meets the
-        // others at every row block's barrier, contributing zeros
-        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
-        return;
-    }
-
-    const int n_items = nb_wg * n_sw;
-    int blk = 0, j = 0;
-    for (int i0 = 0; i0 < n_items; i0 += D) {
-#pragma unroll
-        for (int d = 0; d < D; d++) {
-            if (i0 + d < n_items) {
-                const uint32_t xa = xlane + __umul24((uint32_t)(wave + j * W), xstride);
-                const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
-                stream_step<R, JP>(cw[d], xa, lane_base, quarter_bits, acc, nv);
-                if (++j >= n_sw) {
-                    j = 0;
-                    finish_block(blk);
-                    blk++;
-                }
-            }
-            issue(cw[d]);
-        }
-    }
-}
-
-template <int R, int W, int D, bool kPacked, int JP>
-__global__ __launch_bounds__(64 * W) void gemv_stream_kernel(const uint16_t *__restrict__ x,
-                                                             const uint16_t *__restrict__ codes,
-                                                             const void *__restrict__ grid, float scale,
-                                                             uint16_t *__restrict__ y, int M, int N, int K,
-                                                             int tiles_q, int tiles_r)
-{
-    gemv_stream_body<R, W, D, kPacked, JP>(x, codes, grid, scale, y, M, N, K, tiles_q, tiles_r);
-}
-
-// ------------------------------------------------------------------ streaming matrix-vector path, 8-bit operands
-// The streaming kernel above is bound by the LDS: two 16-byte table gathers per code.  When
-// every grid value is exactly representable in 8 bits (fp8 e4m3: 4 significant bits - the E8P
-// grid of half-odd values is), the same product can be formed with 8-byte gathers, which the
-// LDS serves at twice the rate, by running the matrix unit on 8-bit operands:
-//   * weights.  w = s g + d, s = +-1 per dim, d = +-1/4 per code.  The grid table holds rows of
-//     8 fp8 bytes, the sign table rows of 8 flag bytes (0x80 = flipped); one exclusive or per
-//     4 weights applies the signs, and the 8 bytes of a code are a quarter of the A operand of
-//     v_mfma_f32_16x16x128_f8f6f4 (four codes = 32 consecutive k per lane; twice the time of the
-//     16x16x32 form for four times the work) as they are.  d is left out of the decode and added by the
-//     matrix unit instead: sum_k d x[k] = sum over codes of (8 d) * (mean of the code's 8 x
-//     values), one more MFMA (the 16-bit 16x16x32 form) per 16 rows x 256 k, into an
-//     accumulator of its own, whose A operand is +-2.0 per code, made from the code words
-//     themselves (the shift bit is the sign bit of a half), and whose B operand is the means as
-//     two halves, hi + lo (22 bits of the fp32 sum of the 8 values), in two columns;
-//   * x.  A half with a zero low byte IS a bf8 (e5m2) number in its high byte.  Cutting x after
-//     its top byte, subtracting, scaling what is left by 8 and repeating gives
-//     x = t0 + t1 / 8 + t2 / 64 + t3 / 512 exactly for every normal x (3 significant bits per
-//     term, 11 in a half); the four terms sit in four B columns - at batch 1 the other 15
-//     columns of the 16-wide tile are idle anyway - and the four result columns are added, with
-//     those weights, at the end.
-// s g + d is exact in half for every fp8 g and the terms of x add up to x (subnormal x may lose
-// bits below 2^-24 * 4), so nothing is lost in the operands, and the products are exact in the
-// fp32 accumulators.  Two things remain: the means (hi + lo drops what lies 22 bits below the
-// leading one of a mean) and the matrix unit's adder, which aligns the products of a group to
-// the largest of them.  Measured against the fp64 reference on the benchmark's inputs: 98 %
-// of the outputs are the correctly rounded ones and the 99th percentile of the error is 0.57
-// half ulps (the 16-bit kernel: 0.5, the output rounding alone); with 100-fold outliers in x
-// 2.6 ulps; x with few significant bits: every output correctly rounded.  All of it a
-// hundredth of the operator's tolerance of 1e-2 or less.  A grid with a value fp8 cannot hold is found while the table is built
-// (convert, convert back, compare), an x that is not finite while it is split; every workgroup
-// then runs the 16-bit kernel above instead: same launch, same result as that kernel gives.
-// LDS map: [0, 32K) sign rows (128 x 32 copies x 8 B), [32K, 96K) grid rows (256 x 32 copies x
-// 8 B; a lane reads copy lane % 32, conflict-free for any codes), partial sums, then the terms
-// of x (column m * 4 + t, pitch K + 16 bytes) and the means (rows 2 m: hi, 2 m + 1: lo; K / 8
-// halves each, pitch K / 4 + 16 bytes).
-typedef __attribute__((address_space(3))) const u2_t lds_u2_t;
-__device__ __forceinline__ u2_t lds_read8(uint32_t byte_addr)
-{
-    return *reinterpret_cast<lds_u2_t *>(byte_addr);
-}
-
-// Partial sums of a row block, two parities: one float4 per (wave, tile, quarter, x row), the term
-// columns already added by the wave.
-__host__ __device__ constexpr int q8_red_bytes(int R, int W, int M) { return 2 * W * R * 4 * M * 16; }
-// terms of x (4 rows of K bytes per x row), the per-code means of x as two halves each (hi + lo:
-// 2 rows of K / 8 halves per x row), and one word per wave for the vote on the grid
-__host__ __device__ constexpr int64_t q8_x_bytes(int64_t M, int64_t K)
-{
-    return 4 * M * (K + 16) + 2 * M * (K / 4 + 16) + 64;
-}
-
-// the 8 sign flags of a sign-row index as bytes: dims 0-3 in [0], 4-7 in [1]
-__device__ __forceinline__ u2_t sign_bytes(uint32_t s7)
-{
-    const uint32_t s8 = s7 | ((__builtin_popcount(s7) & 1u) << 7);
-    u2_t r;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const uint32_t n = (s8 >> (4 * i)) & 0xFu;
-        r[i] = ((n & 1u) << 7) | ((n & 2u) << 14) | ((n & 4u) << 21) | ((n & 8u) << 28);
-    }
-    return r;
-}
-
-// a grid row as 8 fp8 bytes; exact: every value survives the round trip
-__device__ __forceinline__ u2_t grid_row_fp8(const u4_t &row, bool &exact)
-{
-    float f[8];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const h2_t h = as_h2(row[i]);
-        f[2 * i] = (float)h[0];
-        f[2 * i + 1] = (float)h[1];
-    }
-    u2_t r;
-    exact = true;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * i], f[4 * i + 1], 0, false);
-        p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * i + 2], f[4 * i + 3], p, true);
-        r[i] = (uint32_t)p;
-        // (no short circuit: eight compares in a row beat eight branches)
-        exact = exact & (__builtin_amdgcn_cvt_f32_fp8(p, 0) == f[4 * i]) & (__builtin_amdgcn_cvt_f32_fp8(p, 1) == f[4 * i + 1]) &
-                (__builtin_amdgcn_cvt_f32_fp8(p, 2) == f[4 * i + 2]) & (__builtin_amdgcn_cvt_f32_fp8(p, 3) == f[4 * i + 3]);
-    }
-    return r;
-}
-
-// A half as four bf8 terms, h = t0 + t1 / 8 + t2 / 64 + t3 / 512: a term is the top byte of what
-// is left, and what is left after it is scaled by 8 (exact, and it keeps the remainder as far
-// above the subnormal range as h itself was), so every normal h is split without loss.
-// 8 halves (one 16-byte piece of x) at a time: term t of the 8 as 8 bytes in t[t].  Returns
-// whether all 8 are finite (if not, the caller hands the launch to the 16-bit kernel: an
-// infinity must meet the whole weight, not its two parts one after the other).
-__device__ __forceinline__ bool split_piece_bf8(const u4_t &v, u2_t (&t)[4])
-{
-    bool finite = true;
-#pragma unroll
-    for (int i = 0; i < 4; i++) finite = finite && (v[i] & 0x7C00u) != 0x7C00u && (v[i] & 0x7C000000u) != 0x7C000000u;
-    const h2_t eight = h2_t{(half_t)8.0f, (half_t)8.0f};
-    u4_t r = v;
-#pragma unroll
-    for (int term = 0; term < 4; term++) {
-        const u4_t hi = r & 0xFF00FF00u;
-        t[term][0] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07050301u);   // the high bytes of halves 0..3
-        t[term][1] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07050301u);   // and of halves 4..7
-        if (term < 3) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) r[i] = as_u32((as_h2(r[i]) - as_h2(hi[i])) * eight);
-        }
-    }
-    return finite;
-}
-
-// The mean of the 8 halves of a piece (fp32 sum, times 1/8) as two halves, hi + lo: 22 of the
-// fp32 sum's 24 bits.  Low half of the result: hi.
-__device__ __forceinline__ uint32_t piece_mean_hi_lo(const u4_t &v)
-{
-    const h2_t ones = h2_t{(half_t)1.0f, (half_t)1.0f};
-    float r = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; i++) r = __builtin_amdgcn_fdot2(as_h2(v[i]), ones, r, false);
-    r *= 0.125f;
-    const half_t hi = (half_t)r;
-    const half_t lo = (half_t)(r - (float)hi);
-    return as_u32(h2_t{hi, lo});
-}
-
-struct Q8Gather {
-    u2_t g0, s0, g1, s1;
-};
-
-// lane_base = (lane % 32) * 8; the tables start at LDS address 0
-__device__ __forceinline__ void q8_gather(Q8Gather &o, uint32_t w, uint32_t lane_base)
-{
-    const uint32_t w7 = w & 0x7FFF7FFFu;                 // sign-row index must not see the shift bit
-    o.g0 = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u) + kSSignBytes);
-    o.s0 = lds_read8(__builtin_amdgcn_perm(w7, lane_base, 0x0C0C0500u));
-    o.g1 = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u) + kSSignBytes);
-    o.s1 = lds_read8(__builtin_amdgcn_perm(w7, lane_base, 0x0C0C0700u));
-}
-
-__device__ __forceinline__ long q8_pack(uint32_t lo, uint32_t hi)
-{
-    return (long)(((unsigned long)hi << 32) | (unsigned long)lo);
-}
-
-// One 256-wide k step for the first nv (uniform, 1 <= nv <= R) of R row tiles; same item order
-// as stream_step.  xaddr: this lane's x terms of the step (16 bytes per word pair: the B
-// operands of its two codes), x8addr: the means of its 8 codes (8 halves: hi or lo, by column).
-template <int R>
-__device__ __forceinline__ void q8_step(const u4_t (&cw)[R], uint32_t xaddr, uint32_t x8addr, uint32_t lane_base,
-                                        f4_t (&acc)[R][2], f4_t (&accd)[R], int nv)
-{
-    // All 16 table gathers of a tile's step and the reads of x go out before the first MFMA
-    // (8-byte results: 48 registers), so the wave meets the LDS latency once per step and tile,
-    // not once per word; with two tiles the reads of x serve both.
-    u4_t xq[4];
-    xq[0] = lds_read16(xaddr);
-    xq[1] = lds_read16(xaddr + 16);
-    xq[2] = lds_read16(xaddr + 32);
-    xq[3] = lds_read16(xaddr + 48);
-    const u4_t x8 = lds_read16(x8addr);
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        if (r > 0 && r >= nv) break;   // tiles past nv: nothing to do (uniform)
-        Q8Gather g[4];
-#pragma unroll
-        for (int t2 = 0; t2 < 4; t2++) q8_gather(g[t2], cw[r][t2], lane_base);
-        // two words = four codes = 32 consecutive k of the lane's 64: one 16x16x128 MFMA (32
-        // bytes per lane and operand, A fp8, B bf8, no scaling), which does four times the work
-        // of the 16x16x32 form in twice its time
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const Q8Gather &b0 = g[2 * h], &b1 = g[2 * h + 1];
-            const i8_t a = i8_t{(int)(b0.g0[0] ^ b0.s0[0]), (int)(b0.g0[1] ^ b0.s0[1]), (int)(b0.g1[0] ^ b0.s1[0]),
-                                (int)(b0.g1[1] ^ b0.s1[1]), (int)(b1.g0[0] ^ b1.s0[0]), (int)(b1.g0[1] ^ b1.s0[1]),
-                                (int)(b1.g1[0] ^ b1.s1[0]), (int)(b1.g1[1] ^ b1.s1[1])};
-            const u4_t &x0 = xq[2 * h], &x1 = xq[2 * h + 1];
-            const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
-            acc[r][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[r][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
-        }
-        // the shift term, in 16-bit arithmetic: +-2.0 per code (a code word with everything but its
-        // shift bits replaced by the bits of 2.0) against the means
-        const u4_t a8 = (cw[r] & 0x80008000u) | 0x40004000u;
-        accd[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8_t, a8), __builtin_bit_cast(h8_t, x8), accd[r], 0, 0, 0);
-    }
-}
-
-template <int R, int W, int D, bool kPacked>
-__global__ __launch_bounds__(64 * W) void gemv_q8_kernel(const uint16_t *__restrict__ x,
-                                                         const uint16_t *__restrict__ codes,
-                                                         const void *__restrict__ grid, float scale,
-                                                         uint16_t *__restrict__ y, int M, int N, int K,
-                                                         int tiles_q, int tiles_r)
-{
-    static_assert(R == 1 || R == 2, "a partial row block is handled as one tile");
-    static_assert(W == 16, "the table staging below assumes 1024 threads");
-    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);   // two parities, see q8_red_bytes
-    const int red_par = q8_red_bytes(R, W, M) / 32;                    // float4 per parity
-    unsigned char *xt = smem_raw + kSTablesBytes + q8_red_bytes(R, W, M);
-    // the means: rows 2 m (hi) and 2 m + 1 (lo) of K / 8 halves; the shift term has an accumulator of
-    // its own, where they sit in columns 4 m and 4 m + 1
-    const int xt_pitch = K + 16, x8_pitch = (K >> 2) + 16;
-    unsigned char *x8t = xt + 4 * M * xt_pitch;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int c16 = lane & 15;
-    const int q = lane >> 4;
-    const int n_steps = K >> 8;
-    const int row_bytes = K >> 2;
-    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;
-
-    // ---- prologue: the loads with nothing queued in front of them first (grid rows, the first
-    // pieces of x), then the code stream, then the tables and the terms of x while the code
-    // loads fly.  The three kinds of staging go to different waves - grid rows to waves 0-3 (one
-    // row per thread), sign rows to waves 4-7, x to everybody - because every instruction of
-    // the prologue is paid once per wave that runs it, needed or not.
-    u4_t grow = u4_t{0u, 0u, 0u, 0u};
-    if (wave < 4) grow = reinterpret_cast<const u4_t *>(grid)[tid];
-    const int row_chunks = K >> 3;                     // 16-byte pieces per row of x
-    const int n_pieces = M * row_chunks;               // x is [M][K] contiguous: piece p sits at x + 16 p
-    u4_t xnext = tid < n_pieces ? reinterpret_cast<const u4_t *>(x)[tid] : u4_t{0u, 0u, 0u, 0u};
-
-    const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;   // k steps of this wave per row block
-    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
-    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
-    const int nb_wg = (t1 - t0 + R - 1) / R;
-
-    const int n_tiles_all = (N + 15) >> 4;
-    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_tiles_all * 16 : N) * row_bytes), 0x00020000);
-    int voff[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) voff[r] = kPacked ? lane * 16 + r * n_steps * 1024 : (16 * r + c16) * row_bytes + q * 16;
-    constexpr int kOut = (int)0x80000000;
-    int pf_blk = 0, pf_j = 0;
-    auto issue = [&](u4_t (&cwd)[R]) {
-        const bool ok = pf_blk < nb_wg && n_sw > 0;
-        const int tb = t0 + pf_blk * R;
-        const int soff = !ok ? kOut
-                         : kPacked ? (tb * n_steps + wave + pf_j * W) * 1024
-                                   : tb * 16 * row_bytes + (wave + pf_j * W) * 64;
-#pragma unroll
-        for (int r = 0; r < R; r++)   // tiles of a partial block that belong to the next workgroup: no access
-            cwd[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], (r == 0 || tb + r < t1) ? soff : kOut, 0);
-        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
-    };
-
-    u4_t cw[D][R];
-#pragma unroll
-    for (int d = 0; d < D; d++) issue(cw[d]);
-
-    bool fits = true;   // stays true while x is finite and the grid fits fp8
-    if (wave >= 4 && wave < 8) {
-        // sign rows: 128 rows of 16 slots (16 bytes = two copies each); thread t of these 256 writes
-        // 8 slots of row t / 2 (16 neighbouring lanes hit 16 different slot positions)
-        const int t = tid - 256, row = t >> 1;
-        const u2_t sb = sign_bytes((uint32_t)row);
-        const uint32_t sg = lds_addr(smem_raw) + (uint32_t)((row * 16 + (t & 1) * 8 + (row & 7)) * 16);   // slot i ^ (row % 8)
-#pragma unroll
-        for (int i = 0; i < 8; i++) lds_write16(sg ^ (uint32_t)(i * 16), u4_t{sb[0], sb[1], sb[0], sb[1]});
-    }
-    __builtin_amdgcn_sched_barrier(0);   // keep the sign rows ahead of the waits for the loads
-
-    // x -> its four terms, and the means of every 8 values -> theirs.  One piece per thread and
-    // trip, the next one already on its way.
-    {
-        int m = 0, c = tid;
-        for (int p = tid; p < n_pieces; p += 64 * W) {
-            const u4_t v = xnext;
-            if (p + 64 * W < n_pieces) xnext = reinterpret_cast<const u4_t *>(x)[p + 64 * W];
-            while (c >= row_chunks) { c -= row_chunks; m++; }
-            u2_t t[4];
-            fits = split_piece_bf8(v, t) && fits;
-            const uint32_t mb = piece_mean_hi_lo(v);
-#pragma unroll
-            for (int term = 0; term < 4; term++) *reinterpret_cast<u2_t *>(xt + (m * 4 + term) * xt_pitch + c * 8) = t[term];
-            reinterpret_cast<uint16_t *>(x8t + (2 * m) * x8_pitch)[c] = (uint16_t)mb;
-            reinterpret_cast<uint16_t *>(x8t + (2 * m + 1) * x8_pitch)[c] = (uint16_t)(mb >> 16);
-            c += 64 * W;
-        }
-    }
-    if (wave < 4) {
-        // grid rows: thread tid converts row tid and writes its 16 slots (two copies each)
-        bool exact;
-        const u2_t g8 = grid_row_fp8(grow, exact);
-        fits = fits && exact;
-        const uint32_t gg = lds_addr(smem_raw) + (uint32_t)(kSSignBytes + (tid * 16 + (tid & 15)) * 16);   // slot i ^ (tid % 16)
-#pragma unroll
-        for (int i = 0; i < 16; i++) lds_write16(gg ^ (uint32_t)(i * 16), u4_t{g8[0], g8[1], g8[0], g8[1]});
-    }
-    // the vote: every wave publishes whether one of its rows or pieces failed, in a word of its own (so
-    // nothing needs clearing first), and after the barrier every wave reads all of them
-    uint32_t *votes = reinterpret_cast<uint32_t *>(x8t + 2 * M * x8_pitch);
-    const bool wave_bad = __builtin_amdgcn_ballot_w64(!fits) != 0;
-    if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
-    __syncthreads();
-    if (__builtin_amdgcn_ballot_w64(votes[lane & (W - 1)] != 0) != 0) {
-        // a grid value does not fit 8 bits, or x is not finite: the 16-bit kernel takes over (it
-        // builds its own tables)
-        gemv_stream_body<R, W, 2, kPacked, 4>(x, codes, grid, scale, y, M, N, K, tiles_q, tiles_r);
-        return;
-    }
-
-    // B operand addresses of this lane: column c16 = 4 m + term (column 0 for the idle ones)
-    const int col = c16 < 4 * M ? c16 : 0;
-    const int row8 = (c16 < 4 * M && (c16 & 3) < 2) ? 2 * (c16 >> 2) + (c16 & 3) : 0;   // hi or lo of x row c16 / 4
-    const uint32_t xlane = lds_addr(xt) + (uint32_t)(col * xt_pitch + q * 64);
-    const uint32_t x8lane = lds_addr(x8t) + (uint32_t)(row8 * x8_pitch + q * 16);
-
-    f4_t acc[R][2];
-#pragma unroll
-    for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = f4_t{0.f, 0.f, 0.f, 0.f};
-    // weights of this lane's column: 8^-t with t = c16 % 4 for the terms of x, 1 for the two halves
-    // of the means; columns that hold nothing count as zero
-    const float x_weight = c16 < 4 * M ? __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)(c16 & 3) * 3u << 23)) : 0.f;
-    const float mean_weight = (c16 < 4 * M && (c16 & 3) < 2) ? 1.f : 0.f;
-    f4_t accd[R];   // the shift term
-#pragma unroll
-    for (int r = 0; r < R; r++) accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
-
-    auto finish_block = [&](int blk) {
-        f4_t *rp = red + (blk & 1) * red_par;
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            // the four term columns of an x row are added first, each with the weight of its term:
-            // lane 4 m gets columns 4 m .. 4 m + 3
-            f4_t v = (acc[r][0] + acc[r][1]) * x_weight + accd[r] * mean_weight;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                v[e] = dpp_shr_add<0x101>(v[e]);   // row_shl:1
-                v[e] = dpp_shr_add<0x102>(v[e]);   // row_shl:2
-            }
-            if ((c16 & 3) == 0 && c16 < 4 * M) rp[(wave * R + r) * 4 * M + q * M + (c16 >> 2)] = v;
-            acc[r][0] = acc[r][1] = accd[r] = f4_t{0.f, 0.f, 0.f, 0.f};
-        }
-        __syncthreads();
-        for (int p = wave; p < R * M; p += W) {
-            const int r = p / M, m = p - r * M;
-            f4_t v = f4_t{0.f, 0.f, 0.f, 0.f};
-            if (c16 < W) v = rp[(c16 * R + r) * 4 * M + q * M + m];
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
-            const int tile = t0 + blk * R + r;
-            const int n = tile * 16 + 4 * q;
-            if (c16 == 15 && tile < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
-                h4_t o;
-#pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
-                *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
-            }
-        }
-    };
-
-    if (n_sw == 0) {
-        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
-        return;
-    }
-
-    const int n_items = nb_wg * n_sw;
-    int blk = 0, j = 0;
-    for (int i0 = 0; i0 < n_items; i0 += D) {
-#pragma unroll
-        for (int d = 0; d < D; d++) {
-            if (i0 + d < n_items) {
-                const uint32_t step = (uint32_t)(wave + j * W);
-                const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
-                q8_step<R>(cw[d], xlane + step * 256u, x8lane + step * 64u, lane_base, acc, accd, nv);
-                if (++j >= n_sw) {
-                    j = 0;
-                    finish_block(blk);
-                    blk++;
-                }
-            }
-            issue(cw[d]);
-        }
-    }
-}
-
-// ------------------------------------------------------------------ batch 1 on 8-bit operands, x staged in chunks
-// gemv_q8_kernel's arithmetic (fp8 weights by two 8-byte gathers and two exclusive ors per code, x
-// as four bf8 terms, the shift term through the per-code means) for ONE row of x of any length: the
-// terms of x are staged 4096 values (16 k steps, one per wave) at a time into two LDS buffers taken
-// in turn, the chunk after the current one being split while the current one is multiplied, so
-//   * the launch starts multiplying after 512 pieces of x have been split, not after all of them,
-//     and the rest of the splitting runs beside the code stream;
-//   * the LDS holds 37 KB of x however long x is (K = 28672 needs 129 KB in one piece).
-// A workgroup walks its tiles in groups of up to T; within a group it goes chunk by chunk, and
-// in a chunk wave w does k step 16 c + w of every tile of the group with the same two registers
-// of B operands.  One barrier per chunk hands the x buffers over; the partial sums of the T tiles
-// meet once per group.  The code stream is one load per tile in flight per wave, refilled as soon
-// as the tile's step of the chunk is done.
-// LDS map: tables as in gemv_q8_kernel, partial sums [16 waves][T * 16 + 1] float4, two x buffers
-// (4 term rows of 4096 + 16 bytes, 2 rows of means of 1024 + 16 bytes), one flag word.
-constexpr int kQcChunkK = 4096;
-constexpr int kQcTermPitch = kQcChunkK + 16, kQcMeanPitch = kQcChunkK / 4 + 16;
-constexpr int kQcXBuf = 4 * kQcTermPitch + 2 * kQcMeanPitch;
-__host__ __device__ constexpr int qc_red_bytes(int T) { return 16 * (T * 16 + 1) * 16; }
-__host__ __device__ constexpr int qc_lds_bytes(int T) { return kSTablesBytes + qc_red_bytes(T) + 2 * kQcXBuf + 64; }
-
-// the four bf8 terms of a piece of x (8 halves) and the mean of the 8 as hi + lo halves; returns
-// whether all 8 are finite (their fp32 sum is finite exactly when they all are)
-__device__ __forceinline__ bool qc_split_piece(const u4_t &v, u2_t (&t)[4], uint32_t &mean_hi_lo)
-{
-    const h2_t ones = h2_t{(half_t)1.0f, (half_t)1.0f};
-    float r = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; i++) r = __builtin_amdgcn_fdot2(as_h2(v[i]), ones, r, false);
-    const bool finite = (__builtin_bit_cast(uint32_t, r) & 0x7F800000u) != 0x7F800000u;
-    r *= 0.125f;
-    const half_t hi = (half_t)r;
-    const half_t lo = (half_t)(r - (float)hi);
-    mean_hi_lo = as_u32(h2_t{hi, lo});
-    const h2_t eight = h2_t{(half_t)8.0f, (half_t)8.0f};
-    u4_t rem = v;
-#pragma unroll
-    for (int term = 0; term < 4; term++) {
-        t[term][0] = __builtin_amdgcn_perm(rem[1], rem[0], 0x07050301u);   // the high bytes of halves 0..3
-        t[term][1] = __builtin_amdgcn_perm(rem[3], rem[2], 0x07050301u);   // and of halves 4..7
-        if (term < 3) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) rem[i] = as_u32((as_h2(rem[i]) - as_h2(rem[i] & 0xFF00FF00u)) * eight);
-        }
-    }
-    return finite;
-}
-
-template <int T, int DC, bool kPacked>
-__global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restrict__ x,
-                                                        const uint16_t *__restrict__ codes,
-                                                        const void *__restrict__ grid, float scale,
-                                                        uint16_t *__restrict__ y, int N, int K, int tiles_q, int tiles_r)
-{
-    constexpr int W = 16;
-    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);
-    unsigned char *xbuf = smem_raw + kSTablesBytes + qc_red_bytes(T);
-    uint32_t *flags = reinterpret_cast<uint32_t *>(xbuf + 2 * kQcXBuf);   // [0 .. 15]: one vote per wave; [0] doubles as the running flag
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int c16 = lane & 15;
-    const int q = lane >> 4;
-    const int n_steps = K >> 8;
-    const int n_chunks = (n_steps + W - 1) / W;
-    const int row_bytes = K >> 2;
-    const int n_pieces = K >> 3;
-    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;
-
-    // ---- prologue: grid rows to waves 8-11, sign rows to waves 12-15, the first chunk of x to waves 0-7
-    u4_t grow = u4_t{0u, 0u, 0u, 0u};
-    if (wave >= 8 && wave < 12) grow = reinterpret_cast<const u4_t *>(grid)[tid - 512];
-    u4_t xpiece = u4_t{0u, 0u, 0u, 0u};
-    if (wave < 8 && tid < n_pieces) xpiece = reinterpret_cast<const u4_t *>(x)[tid];
-
-    // this workgroup's tiles [t0, t1), walked in n_groups groups of up to T tiles whose sizes differ by
-    // at most one (7 tiles with T = 3: 3 + 2 + 2, not 3 + 3 + 1: a group of one leaves a wave a single
-    // load in flight)
-    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
-    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
-    const int n_groups = (t1 - t0 + T - 1) / T;
-    // (t1 - t0) / n_groups without a division, which would stand between the kernel's start and its first loads:
-    // with T = 3 the groups of two or more are of 2 or 3 tiles, of 3 only if all are
-    static_assert(T == 3, "the group sizes below are those of T = 3");
-    const int g_base = n_groups <= 1 ? t1 - t0 : (t1 - t0 == 3 * n_groups ? 3 : 2);
-    const int g_rem = n_groups <= 1 ? 0 : t1 - t0 - g_base * n_groups;
-    const int total = n_groups * n_chunks;   // chunks to go through, over all groups
-
-    const int n_tiles_all = (N + 15) >> 4;
-    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_tiles_all * 16 : N) * row_bytes), 0x00020000);
-    const int voff = kPacked ? lane * 16 : c16 * row_bytes + q * 16;
-    constexpr int kOut = (int)0x80000000;
-    // Scalar byte offset of the code word of (group g, chunk c, tile 0 of the group) for this wave, or the
-    // out-of-range offset when the group or the wave's step of the chunk does not exist; tile t of the
-    // group lies t * tile_stride further on.  Out of range: zeros, no memory access.
-    const int tile_stride = kPacked ? n_steps * 1024 : 16 * row_bytes;
-    auto chunk_offset = [&](int g, int c, int &gn) {
-        const int gt0 = t0 + g * g_base + (g < g_rem ? g : g_rem), step = c * W + wave;
-        gn = g < n_groups && step < n_steps ? g_base + (g < g_rem ? 1 : 0) : 0;
-        return kPacked ? (gt0 * n_steps + step) * 1024 : gt0 * tile_stride + step * 64;
-    };
-    auto issue = [&](u4_t &cwd, int base, int gn, int t) {
-        cwd = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, t < gn ? base + t * tile_stride : kOut, 0);
-    };
-    // the ring: DC chunks deep, one slot per tile of the group
-    u4_t cw[DC][T];
-    {
-        int g = 0, c = 0;
-#pragma unroll
-        for (int d = 0; d < DC; d++) {
-            int gn;
-            const int base = chunk_offset(g, c, gn);
-#pragma unroll
-            for (int t = 0; t < T; t++) issue(cw[d][t], base, gn, t);
-            if (++c == n_chunks) { c = 0; g++; }
-        }
-    }
-
-    // one piece of x -> its terms and means in buffer `buf` (piece p of the chunk); returns finite
-    auto stage_piece = [&](const u4_t &v, int buf, int p) {
-        u2_t tm[4];
-        uint32_t mb;
-        const bool fin = qc_split_piece(v, tm, mb);
-        unsigned char *xb = xbuf + buf * kQcXBuf;
-#pragma unroll
-        for (int term = 0; term < 4; term++) *reinterpret_cast<u2_t *>(xb + term * kQcTermPitch + p * 8) = tm[term];
-        reinterpret_cast<uint16_t *>(xb + 4 * kQcTermPitch)[p] = (uint16_t)mb;
-        reinterpret_cast<uint16_t *>(xb + 4 * kQcTermPitch + kQcMeanPitch)[p] = (uint16_t)(mb >> 16);
-        return fin;
-    };
-
-    bool fits = true;   // stays true while x is finite and the grid fits fp8
-    if (wave >= 12) {
-        // sign rows: 128 rows of 16 slots (16 bytes = two copies each); thread t of these 256 writes
-        // 8 slots of row t / 2 (16 neighbouring lanes hit 16 different slot positions)
-        const int t = tid - 768, row = t >> 1;
-        const u2_t sb = sign_bytes((uint32_t)row);
-        // slot i ^ (row % 8) of the thread's eight: one exclusive or per address
-        const uint32_t sg = lds_addr(smem_raw) + (uint32_t)((row * 16 + (t & 1) * 8 + (row & 7)) * 16);
-#pragma unroll
-        for (int i = 0; i < 8; i++) lds_write16(sg ^ (uint32_t)(i * 16), u4_t{sb[0], sb[1], sb[0], sb[1]});
-    } else if (wave >= 8) {
-        bool exact;
-        const u2_t g8 = grid_row_fp8(grow, exact);
-        fits = exact;
-        const int r = tid - 512;
-        const uint32_t gg = lds_addr(smem_raw) + (uint32_t)(kSSignBytes + (r * 16 + (r & 15)) * 16);   // slot i ^ (r % 16)
-#pragma unroll
-        for (int i = 0; i < 16; i++) lds_write16(gg ^ (uint32_t)(i * 16), u4_t{g8[0], g8[1], g8[0], g8[1]});
-    } else {
-        fits = stage_piece(xpiece, 0, tid);
-    }
-    // the vote: every wave publishes whether something of its own failed, in a word of its own (so
-    // nothing needs clearing first), and after the barrier every wave reads all of them
-    {
-        const bool wave_bad = __builtin_amdgcn_ballot_w64(!fits) != 0;
-        if (lane == 0) flags[wave] = wave_bad ? 1u : 0u;
-    }
-    __syncthreads();
-    // a grid value that does not fit 8 bits, or (here or in a later chunk) an x that is not finite: the
-    // 16-bit kernel does the whole call over, at the end of this function
-    bool hand_over = __builtin_amdgcn_ballot_w64(flags[lane & (W - 1)] != 0) != 0;
-
-    // B operands of this lane: columns 0 .. 7 = term c16 % 4 of the first or the second MFMA's 32 bytes
-    // of the wave's k step, columns 8 and 9 = the means (hi, lo); the other columns repeat 2 .. 7.
-    // Wave w always does step w of a chunk, so the address only depends on the buffer.
-    const bool mean_col = c16 == 8 || c16 == 9;
-    const uint32_t xlane = lds_addr(xbuf) + (mean_col ? (uint32_t)(4 * kQcTermPitch + (c16 - 8) * kQcMeanPitch + q * 16 + wave * 64)
-                                                      : (uint32_t)((c16 & 3) * kQcTermPitch + q * 64 + ((c16 >> 2) & 1) * 32 + wave * 256));
-
-    f4_t acc[T][2], accd[T];
-#pragma unroll
-    for (int t = 0; t < T; t++) acc[t][0] = acc[t][1] = accd[t] = f4_t{0.f, 0.f, 0.f, 0.f};
-    const float d_scale = c16 == 0 ? 1.f : c16 == 1 ? 8.f : 0.f;
-
-    // With one or two chunks all of x stays resident once staged (chunk c in buffer c); longer x goes
-    // through the two buffers in turn and is staged again for every group.
-    const bool resident = n_chunks <= 2;
-    int g = 0, c = 0;            // group and chunk of the chunk being multiplied
-    int pg = 0, pc = 0;          // ... of the chunk DC further on, whose code words refill the slots
-#pragma unroll
-    for (int d = 0; d < DC; d++)
-        if (++pc == n_chunks) { pc = 0; pg++; }
-    bool barrier_in_group = true;   // the prologue's
-
-    // one chunk; kSlot: its ring slot (static).  Every path issues exactly T code loads (tiles and
-    // steps that do not exist load nothing and get zeros), so the wait counters stay exact.
-    auto chunk = [&](auto slot_tag, int gc) {
-        constexpr int kSlot = decltype(slot_tag)::value;
-        const bool exists = DC == 1 || gc < total;   // only a second chunk of an unrolled pair may lie past the end
-        const int gn = g_base + (g < g_rem ? 1 : 0);
-        const int ntg = exists ? gn : 0;                          // tiles of this group (uniform)
-        const bool last_c = c + 1 == n_chunks;
-        const int xb_cur = resident ? c : gc & 1;
-        // the chunk after this one: if its x is not in LDS yet, half of the waves split it while everybody
-        // multiplies, waves 0-7 and 8-15 taking turns
-        const int ng = last_c ? g + 1 : g, nc = last_c ? 0 : c + 1;
-        const bool stage_next = exists && gc + 1 < total && (!resident || gc + 1 < n_chunks);
-        const bool stager = stage_next && wave < 8;   // the waves the arbiter prefers: they are through their steps first
-        const int sp = tid & 511;
-        if (stager) {
-            const int p = nc * 512 + sp;
-            xpiece = p < n_pieces ? reinterpret_cast<const u4_t *>(x)[p] : u4_t{0u, 0u, 0u, 0u};
-        }
-        const bool step_ok = exists && c * W + wave < n_steps;
-        int p_gn;                                                 // the refills: chunk DC further on
-        const int p_base = chunk_offset(pg, pc, p_gn);
-        u4_t x0 = u4_t{0u, 0u, 0u, 0u}, x1 = x0;
-        if (step_ok) {
-            const uint32_t xa = xlane + (uint32_t)(xb_cur * kQcXBuf);
-            x0 = lds_read16(xa);
-            x1 = lds_read16(xa + 16);
-        }
-        const i8_t xb = i8_t{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
-#pragma unroll
-        for (int t = 0; t < T; t++) {
-            if (step_ok && t < ntg) {   // uniform
-                Q8Gather gt[4];
-#pragma unroll
-                for (int t2 = 0; t2 < 4; t2++) q8_gather(gt[t2], cw[kSlot][t][t2], lane_base);
-                u4_t a8;   // +-2.0 per code, the shift term's A operand: the code words' shift bits over the bits of 2.0
-#pragma unroll
-                for (int i = 0; i < 4; i++) a8[i] = bfi(0x80008000u, cw[kSlot][t][i], 0x40004000u);
-#pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    const Q8Gather &b0 = gt[2 * h], &b1 = gt[2 * h + 1];
-                    const i8_t a = i8_t{(int)(b0.g0[0] ^ b0.s0[0]), (int)(b0.g0[1] ^ b0.s0[1]), (int)(b0.g1[0] ^ b0.s1[0]),
-                                        (int)(b0.g1[1] ^ b0.s1[1]), (int)(b1.g0[0] ^ b1.s0[0]), (int)(b1.g0[1] ^ b1.s0[1]),
-                                        (int)(b1.g1[0] ^ b1.s1[0]), (int)(b1.g1[1] ^ b1.s1[1])};
-                    acc[t][h] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb, acc[t][h], 0 /* A: fp8 */, 1 /* B: bf8 */, 0, 0, 0, 0);
-                }
-                accd[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8_t, a8), __builtin_bit_cast(h8_t, x0), accd[t], 0, 0, 0);
-            }
-            issue(cw[kSlot][t], p_base, p_gn, t);                  // the slot's next code word
-        }
-        if (stager && !stage_piece(xpiece, resident ? nc : (gc + 1) & 1, sp)) flags[0] = 1u;
-        if (!exists) return;
-        const bool group_end = last_c;
-        if (group_end) {
-            // `red` still holds the sums of the group before while its reducers read them: a barrier has
-            // to lie between their read and this write
-            if (!barrier_in_group) __syncthreads();
-            // the group's partial sums: 4 columns per (wave, tile, quarter) - term t of the first MFMAs
-            // (column t) plus term t of the second (column 4 + t); the shift term's columns 8 and 9 ride
-            // in slots 0 and 1, the second times 8 to meet the weight 1/8 it gets from the reducer
-#pragma unroll
-            for (int t = 0; t < T; t++) {
-                if (t >= ntg) break;
-                f4_t v;
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    v[e] = dpp_shl_add<4>(acc[t][0][e], acc[t][1][e]) + dpp_shl_add<8>(0.f, accd[t][e]) * d_scale;
-                if (c16 < 4) red[wave * (T * 16 + 1) + (t * 4 + q) * 4 + c16] = v;
-                acc[t][0] = acc[t][1] = accd[t] = f4_t{0.f, 0.f, 0.f, 0.f};
-            }
-        }
-        barrier_in_group = !group_end && (barrier_in_group || stage_next);
-        if (stage_next || group_end) {
-            __syncthreads();   // hands the x buffers over and / or gathers the group's partial sums
-            if (stage_next && __builtin_amdgcn_ballot_w64(flags[0] != 0) != 0) hand_over = true;
-        }
-        if (group_end && !hand_over && wave < ntg) {
-            // wave t adds up tile t: lane (w, quarter) takes wave w's 4 columns with their weights 8^-c,
-            // then the 16 lanes of a row are added with DPP shifts
-            const f4_t *src = red + c16 * (T * 16 + 1) + (wave * 4 + q) * 4;
-            f4_t v = src[0];
-#pragma unroll
-            for (int cc = 1; cc < 4; cc++) v += src[cc] * __builtin_bit_cast(float, 0x3F800000u - ((uint32_t)cc * 3u << 23));
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
-            const int gt0 = t0 + g * g_base + (g < g_rem ? g : g_rem);
-            const int n = (gt0 + wave) * 16 + 4 * q;
-            if (c16 == 15 && n < N) {   // N % 4 == 0, so the four rows are in range together
-                h4_t o;
-#pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
-                *reinterpret_cast<h4_t *>(y + n) = o;
-            }
-        }
-        if (++c == n_chunks) { c = 0; g++; }
-        if (++pc == n_chunks) { pc = 0; pg++; }
-    };
-
-    for (int gc = 0; gc < total && !hand_over; gc += DC) {
-        chunk(std::integral_constant<int, 0>{}, gc);
-        if constexpr (DC > 1) {
-            if (!hand_over) chunk(std::integral_constant<int, 1>{}, gc + 1);
-        }
-    }
-    if (hand_over) {
-        __syncthreads();   // everybody has read the flags before the LDS is laid out anew
-        gemv_stream_body<1, W, 2, kPacked, 4>(x, codes, grid, scale, y, 1, N, K, tiles_q, tiles_r);
-    }
-}
-
-// ------------------------------------------------------------------ small-batch matrix-vector path
-// M <= 32 when x does not fit in LDS beside the tables (M * K too large).  Same tables, same
-// decode, same persistent workgroups and split-K as the streaming kernel; the difference is
-// where B comes from: x is read from global memory (L2) into registers, one 256-wide step at
-// a time.  Because vector-memory results return in order, x and codes of a step travel as ONE
-// prefetch unit (x first, then the codes), D units deep: an x load never waits behind codes
-// that are needed later than it is.  All loads are raw buffer loads whose offset is out of
-// range past the end (zeros, no memory access), so no branch surrounds them and the wait
-// counters stay exact.  MT = number of 16-row tiles of x (M <= 16 * MT).
-template <int R, int MT>
-__device__ __forceinline__ void regx_step(const u4_t (&cw)[R], const u4_t (&xb)[MT][8], uint32_t lane_base,
-                                          uint32_t quarter_bits, f4_t (&acc)[R][MT][2], int nv)
-{
-    constexpr int kItems = 4 * R;
-    StreamGather buf[2];
-    stream_gather(buf[0], cw[0][0], lane_base, quarter_bits);
-#pragma unroll
-    for (int i = 0; i < kItems; i++) {
-        const int t2 = i / R, r = i % R;
-        if (i + 1 < kItems) {
-            const int nt2 = (i + 1) / R, nr = (i + 1) % R;
-            if (nr == 0 || nr < nv) stream_gather(buf[(i + 1) & 1], cw[nr][nt2], lane_base, quarter_bits);
-        }
-        if (r == 0 || r < nv) {   // tiles past nv (uniform) belong to the next workgroup
-            const StreamGather &b = buf[i & 1];
-            const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-                acc[r][mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[mt][2 * t2]), acc[r][mt][0], 0, 0, 0);
-            const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-                acc[r][mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[mt][2 * t2 + 1]), acc[r][mt][1], 0, 0, 0);
-        }
-    }
-}
-
-template <int R, int W, int MT, int D, bool kPacked>
-__global__ __launch_bounds__(64 * W) void gemv_regx_kernel(const uint16_t *__restrict__ x,
-                                                           const uint16_t *__restrict__ codes,
-                                                           const void *__restrict__ grid, float scale,
-                                                           uint16_t *__restrict__ y, int M, int N, int K,
-                                                           int tiles_q, int tiles_r)
-{
-    static_assert(R >= 1 && R <= 4, "row tiles per block");
-    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    typedef f4_t red_t[W][R * MT][kWave];
-    red_t *red = reinterpret_cast<red_t *>(smem_raw + kSTablesBytes);   // red[parity]
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int c16 = lane & 15;
-    const int q = lane >> 4;
-    const int n_steps = K >> 8;
-    const int row_bytes = K >> 2;
-    const uint32_t lane_base = (uint32_t)c16 * 16u;
-    const uint32_t quarter_bits = 0x34003400u;
-
-    const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid & 255];
-
-    const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;
-    // contiguous, balanced range of 16-row tiles per workgroup, as in the streaming kernel
-    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
-    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
-    const int nb_wg = (t1 - t0 + R - 1) / R;
-
-    // row-major or packed codes, addressed as in the streaming kernel
-    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
-    const __amdgpu_buffer_rsrc_t xrsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, M * K * 2, 0x00020000);
-    constexpr int kOut = (int)0x80000000;
-    int voff[R], xoff[MT];
-#pragma unroll
-    for (int r = 0; r < R; r++) voff[r] = kPacked ? lane * 16 + r * n_steps * 1024 : (16 * r + c16) * row_bytes + q * 16;
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-        const int m = 16 * mt + c16;
-        xoff[mt] = m < M ? (m * K + 64 * q) * 2 : kOut;   // columns past M: zeros, no memory access
-    }
-
-    struct Unit {
-        u4_t cw[R];
-        u4_t xb[MT][8];
-    };
-    int pf_blk = 0, pf_j = 0;
-    auto issue = [&](Unit &u) {
-        const bool ok = pf_blk < nb_wg && n_sw > 0;
-        const int step = wave + pf_j * W;
-        const int xs_off = ok ? step * 512 : kOut;
-        const int tb = t0 + pf_blk * R;
-        const int soff = !ok ? kOut : kPacked ? (tb * n_steps + step) * 1024 : tb * 16 * row_bytes + step * 64;
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-            for (int t = 0; t < 8; t++)
-                u.xb[mt][t] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff[mt] + t * 16, xs_off, 0);
-#pragma unroll
-        for (int r = 0; r < R; r++)
-            u.cw[r] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], (r == 0 || tb + r < t1) ? soff : kOut, 0);
-        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
-    };
-
-    Unit ring[D];
-#pragma unroll
-    for (int d = 0; d < D; d++) issue(ring[d]);
-
-    // tables (sign rows need no load; grid rows from the fetch above)
-    {
-        constexpr int kPerRow = 64 * W / 128, kCopies = 16 / kPerRow;
-        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw);
-        const int srow = tid / kPerRow, sc0 = (tid % kPerRow) * kCopies;
-        const u4_t sv = sign_row((uint32_t)srow);
-#pragma unroll
-        for (int i = 0; i < kCopies; i++) sg[srow * 16 + ((sc0 + i + srow) & 15)] = sv;   // 16 lanes, 16 bank groups
-        constexpr int kCopiesPer = 4096 / (64 * W);
-        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes);
-        const int row = tid & 255, c0 = (tid >> 8) * kCopiesPer;
-#pragma unroll
-        for (int i = 0; i < kCopiesPer; i++) gg[row * 16 + ((c0 + i + tid) & 15)] = grow;   // 16 lanes, 16 bank groups
-    }
-    __syncthreads();
-
-    f4_t acc[R][MT][2];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) acc[r][mt][0] = acc[r][mt][1] = f4_t{0.f, 0.f, 0.f, 0.f};
-
-    // end of a row block: partial sums to LDS (double-buffered per block), one barrier, then
-    // the first R * MT waves add up one (row tile, m tile) each and store it
-    auto finish_block = [&](int blk) {
-        const int par = blk & 1;
-#pragma unroll
-        for (int r = 0; r < R; r++)
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++) {
-                red[par][wave][r * MT + mt][lane] = acc[r][mt][0] + acc[r][mt][1];
-                acc[r][mt][0] = acc[r][mt][1] = f4_t{0.f, 0.f, 0.f, 0.f};
-            }
-        __syncthreads();
-        for (int tile = wave; tile < R * MT; tile += W) {
-            f4_t sacc = red[par][0][tile][lane];
-#pragma unroll
-            for (int w = 1; w < W; w++) sacc += red[par][w][tile][lane];
-            const int r = tile / MT, mt = tile % MT;
-            const int m = 16 * mt + c16;
-            const int rt = t0 + blk * R + r;
-            const int n = rt * 16 + 4 * q;
-            if (m < M && rt < t1 && n < N) {   // N % 4 == 0, so the four rows are in range together
-                h4_t o;
-#pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (half_t)(sacc[e] * scale);
-                *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
-            }
-        }
-    };
-
-    if (n_sw == 0) {
-        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
-        return;
-    }
-    const int n_items = nb_wg * n_sw;
-    int blk = 0, j = 0;
-    for (int i0 = 0; i0 < n_items; i0 += D) {
-#pragma unroll
-        for (int d = 0; d < D; d++) {
-            if (i0 + d < n_items) {
-                regx_step<R, MT>(ring[d].cw, ring[d].xb, lane_base, quarter_bits, acc, t1 - (t0 + blk * R));
-                if (++j >= n_sw) {
-                    j = 0;
-                    finish_block(blk);
-                    blk++;
-                }
-            }
-            issue(ring[d]);
-        }
-    }
-}
-
-// ------------------------------------------------------------------ matrix-matrix path
-// Block tile BN (n) x BM (m) x 64 (k) with WN x WM waves, each wave TN x TM tiles of
-// v_mfma_f32_32x32x16_f16 (A = decoded W rows, B = x rows, fp32 accumulate).  A wide n keeps
-// x re-reads down (x is fetched once per BN output columns) and a tall m amortises the decode.
-//
-// The k loop is software-pipelined three deep so that the matrix unit never waits for
-// staging: while the MFMAs of tile kt run out of LDS buffer kt%2, the same waves decode tile
-// kt+1 (whose codes and x already sit in registers) into buffer (kt+1)%2 - a quarter of that
-// work after each group of MFMAs, in the matrix unit's shadow - and the global loads of tiles
-// kt+2 .. kt+4 are in flight.  One barrier per k tile.  LDS rows are 144 bytes apart (9 bank groups),
-// so the 16 lanes the LDS serves per clock - 16 consecutive rows at the same k - hit 16
-// different groups.
-constexpr int kGemmBK = 64;
-constexpr int kGemmLd = kGemmBK + 8;   // halves per LDS row
-
-template <int WN, int WM, int TN, int TM>
-struct GemmCfg {
-    static constexpr int kThreads = 64 * WN * WM;
-    static constexpr int kBN = WN * TN * 32;
-    static constexpr int kBM = WM * TM * 32;
-    static constexpr int kTPR = kThreads / kBN;            // threads sharing one W row (1 or 2)
-    static constexpr int kCPT = 8 / kTPR;                  // codes per thread per k tile
-    static constexpr int kXPT = kBM * 8 / kThreads;        // 16-byte pieces of x per thread per k tile
-    static constexpr int kXTPR = 8 / kXPT;                 // threads sharing one x row
-    static_assert(kTPR == 1 || kTPR == 2, "one or two threads per W row");
-    static_assert(kXPT >= 1 && kXPT <= 8 && 8 % kXPT == 0, "x pieces per thread");
-    struct Shared {
-        DecodeTables tab;
-        uint16_t w[2][kBN][kGemmLd];
-        uint16_t x[2][kBM][kGemmLd];
-    };
-};
-
-// decode of one code with the packed delta taken from the low / high half of dd
-template <bool kHi>
-__device__ __forceinline__ u4_t gemm_decode(uint32_t code, uint32_t dd, const DecodeTables &t)
-{
-    const u4_t g = t.grid[code & 0xFFu];
-    const u4_t sg = t.sign[(code >> 8) & 0x7Fu];
-    u4_t r;
-#pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = pk_fma_bcast<kHi>(g[i], sg[i], dd);
-    return r;
-}
-
-template <int WN, int WM, int TN, int TM>
-__global__ __launch_bounds__(64 * WN * WM) void gemm_kernel(const uint16_t *__restrict__ x,
-                                                            const uint16_t *__restrict__ codes,
-                                                            const void *__restrict__ grid, float scale,
-                                                            uint16_t *__restrict__ y, int M, int N, int K, int y_vec)
-{
-    typedef GemmCfg<WN, WM, TN, TM> C;
-    extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
-    typename C::Shared &sh = *reinterpret_cast<typename C::Shared *>(gemm_smem);
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wn = wave % WN, wm = wave / WN;
-    const int n0 = blockIdx.x * C::kBN;
-    const int m0 = blockIdx.y * C::kBM;
-    const int k_tiles = K / kGemmBK;
-    const int64_t kc = K >> 3;
-
-    stage_tables<true>(sh.tab, grid, tid, C::kThreads);
-
-    // W staging: thread -> row tid / kTPR, kCPT codes of the k tile
-    const int w_row = tid / C::kTPR, w_part = tid % C::kTPR;
-    int wr = n0 + w_row;
-    wr = wr < N ? wr : N - 1;
-    const uint16_t *wsrc = codes + (int64_t)wr * kc + w_part * C::kCPT;
-    // x staging: thread -> row tid / kXTPR, kXPT pieces of 8 halves
-    const int x_row = tid / C::kXTPR, x_part = tid % C::kXTPR;
-    int xr = m0 + x_row;
-    const bool x_in = xr < M;
-    xr = x_in ? xr : M - 1;
-    const uint16_t *xsrc = x + (int64_t)xr * K + x_part * C::kXPT * 8;
-
-    struct Stage {
-        uint32_t cw[C::kCPT / 2];
-        u4_t xv[C::kXPT];
-    };
-    auto load_tile = [&](Stage &st, int kt) {
-        kt = kt < k_tiles ? kt : k_tiles - 1;    // past the end: reload the last tile (never used)
-        const uint32_t *wp = reinterpret_cast<const uint32_t *>(wsrc + (int64_t)kt * 8);
-        if (C::kCPT == 8) {
-            const u4_t v = *reinterpret_cast<const u4_t *>(wp);
-#pragma unroll
-            for (int i = 0; i < C::kCPT / 2; i++) st.cw[i] = v[i];
-        } else {
-            const u2_t v = *reinterpret_cast<const u2_t *>(wp);
-#pragma unroll
-            for (int i = 0; i < C::kCPT / 2; i++) st.cw[i] = v[i];
-        }
-#pragma unroll
-        for (int i = 0; i < C::kXPT; i++) st.xv[i] = reinterpret_cast<const u4_t *>(xsrc + (int64_t)kt * kGemmBK)[i];
-    };
-    // One quarter (q = 0..3) of a thread's staging work for LDS buffer `buf`, in two halves:
-    // the table gathers are issued before a group of MFMAs, the packed FMAs and the LDS writes
-    // run after it, in the matrix unit's shadow.
-    constexpr int kCq = C::kCPT / 4;             // codes per quarter: 1 or 2
-    struct Gathered {
-        u4_t g[kCq], sg[kCq];
-    };
-    auto stage_gather = [&](Gathered &o, const Stage &st, int q) {
-#pragma unroll
-        for (int c = 0; c < kCq; c++) {
-            const int ci = q * kCq + c;          // code index within the thread's kCPT
-            const uint32_t code = (ci & 1) ? st.cw[ci >> 1] >> 16 : st.cw[ci >> 1];
-            o.g[c] = sh.tab.grid[code & 0xFFu];
-            o.sg[c] = sh.tab.sign[(code >> 8) & 0x7Fu];
-        }
-    };
-    auto stage_finish = [&](const Gathered &o, const Stage &st, int buf, int q) {
-#pragma unroll
-        for (int c = 0; c < kCq; c++) {
-            const int ci = q * kCq + c;
-            const uint32_t dd = (st.cw[ci >> 1] & 0x80008000u) | 0x34003400u;
-            u4_t wv;
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                wv[i] = (ci & 1) ? pk_fma_bcast<true>(o.g[c][i], o.sg[c][i], dd) : pk_fma_bcast<false>(o.g[c][i], o.sg[c][i], dd);
-            *reinterpret_cast<u4_t *>(&sh.w[buf][w_row][(w_part * C::kCPT + ci) * 8]) = wv;
-        }
-        const u4_t zero = u4_t{0u, 0u, 0u, 0u};
-        if (C::kXPT >= 4) {
-#pragma unroll
-            for (int i = 0; i < C::kXPT / 4; i++) {
-                const int pi = q * (C::kXPT / 4) + i;
-                *reinterpret_cast<u4_t *>(&sh.x[buf][x_row][(x_part * C::kXPT + pi) * 8]) = x_in ? st.xv[pi] : zero;
-            }
-        } else if (q < C::kXPT) {
-            *reinterpret_cast<u4_t *>(&sh.x[buf][x_row][(x_part * C::kXPT + q) * 8]) = x_in ? st.xv[q] : zero;
-        }
-    };
-
-    // ring of four stages: tile kt+1 is staged out of ring[(kt+1)%4] while tile kt+4 is fetched
-    // into ring[kt%4], so a global load has three tiles of MFMAs to arrive
-    Stage ring[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) load_tile(ring[i], i);
-
-    f16_t acc[TN][TM];
-#pragma unroll
-    for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int j = 0; j < TM; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
-
-    const int l32 = lane & 31, kq = lane >> 5;
-    __syncthreads();   // tables ready
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-        Gathered gq;
-        stage_gather(gq, ring[0], q);
-        stage_finish(gq, ring[0], 0, q);
-    }
-    __syncthreads();   // tile 0 staged
-
-    // Compute tile kt from buffer `buf` while staging tile kt+1 (registers sn) into the other
-    // buffer and fetching tile kt+4 into sf.  Operand fragments are double-buffered in
-    // registers: those of k step ks+1 are requested before the MFMAs of step ks are issued.
-    auto read_frags = [&](h8_t (&a)[TN], h8_t (&b)[TM], int buf, int ks) {
-#pragma unroll
-        for (int i = 0; i < TN; i++)
-            a[i] = *reinterpret_cast<const h8_t *>(&sh.w[buf][(wn * TN + i) * 32 + l32][ks * 16 + kq * 8]);
-#pragma unroll
-        for (int j = 0; j < TM; j++)
-            b[j] = *reinterpret_cast<const h8_t *>(&sh.x[buf][(wm * TM + j) * 32 + l32][ks * 16 + kq * 8]);
-    };
-    auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf) {
-        const bool staging = kt + 1 < k_tiles;
-        load_tile(sf, kt + 4);
-        h8_t a[2][TN], b[2][TM];
-        read_frags(a[0], b[0], buf, 0);
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            if (ks < 3) read_frags(a[(ks + 1) & 1], b[(ks + 1) & 1], buf, ks + 1);
-            Gathered gq;
-            if (staging) stage_gather(gq, sn, ks);
-#pragma unroll
-            for (int i = 0; i < TN; i++)
-#pragma unroll
-                for (int j = 0; j < TM; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
-            if (staging) stage_finish(gq, sn, buf ^ 1, ks);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        __syncthreads();
-    };
-
-    for (int kt = 0; kt < k_tiles; kt += 4) {
-        tile(kt, 0, ring[1], ring[0]);
-        if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1]);
-        if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2]);
-        if (kt + 3 < k_tiles) tile(kt + 3, 1, ring[0], ring[3]);
-    }
-
-    // D layout of 32x32: element e of lane: row (n) = 8*(e/4) + 4*(lane/32) + e%4, column (m) = lane%32
-    const bool n_vec = (N & 3) == 0 && y_vec != 0;   // 8-byte stores need an 8-byte aligned y
-#pragma unroll
-    for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int j = 0; j < TM; j++) {
-            const int m = m0 + (wm * TM + j) * 32 + l32;
-            if (m >= M) continue;
-#pragma unroll
-            for (int e4 = 0; e4 < 4; e4++) {
-                const int n = n0 + (wn * TN + i) * 32 + 8 * e4 + 4 * kq;
-                uint16_t o[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    o[e] = __builtin_bit_cast(uint16_t, (half_t)(acc[i][j][4 * e4 + e] * scale));
-                uint16_t *dst = y + (int64_t)m * N + n;
-                if (n_vec && n + 3 < N) {
-                    u2_t v;
-                    v[0] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-                    v[1] = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
-                    *reinterpret_cast<u2_t *>(dst) = v;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (n + e < N) dst[e] = o[e];
-                }
-            }
-        }
-}
-
-// ------------------------------------------------------------------ matrix-matrix path, weights in registers
-// Block tile 256 (n) x 128 (m) x 64 (k), four waves, each wave 64 rows of W (two 32-row tiles)
-// against all 128 rows of x (four 32-row tiles): 8 accumulators of v_mfma_f32_32x32x16_f16.
-//
-// The LDS is the scarce resource of the staged kernel above (table gathers with bank
-// conflicts, W tile written and read back, operand fragments read by every wave).  Here
-//   * a wave decodes ITS 64 rows straight into A-operand registers - a lane's 8 bytes of a
-//     row are the 4 codes it feeds to the 4 MFMA k steps of the tile, any k order works as
-//     long as A and B agree - so W never touches the LDS and no decode is done twice;
-//   * the tables are the conflict-free 16-copy ones of the matrix-vector kernels (256-byte
-//     row pitch, lane reads copy lane % 16, address = one v_perm_b32);
-//   * only x goes through the LDS (coalesced global loads, rows 144 bytes apart, double
-//     buffered, one barrier per k tile), read as B fragments once per wave and k step.
-// Per k tile and wave: 32 MFMAs (1024 matrix-unit clocks) against 36 LDS instructions and
-// about 64 VALU operations, so the matrix unit is the bound.  Tile kt+1 is decoded and its x
-// written while the MFMAs of tile kt run; global loads are four tiles ahead.
-// w = g * s + d, d = low (kHi false) or high half of dd for both lanes, as plain vector code:
-// the compiler folds the broadcast into the op_sel bits and its scheduler sees a VALU
-// instruction (it cannot classify inline assembly)
-template <bool kHi>
-__device__ __forceinline__ h8_t gemm_finish(const u4_t &g, const u4_t &sg, uint32_t dd)
-{
-    const h2_t dv = as_h2(dd);
-    const h2_t d = kHi ? h2_t{dv[1], dv[1]} : h2_t{dv[0], dv[0]};
-    u4_t r;
-#pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = as_u32(__builtin_elementwise_fma(as_h2(g[i]), as_h2(sg[i]), d));
-    return __builtin_bit_cast(h8_t, r);
-}
-
-constexpr int kGrBN = 256, kGrBK = 64, kGrLd = kGrBK + 8;
-constexpr int kGrTN = 2;
-__host__ __device__ constexpr int gr_smem_bytes(int TM) { return kSTablesBytes + 2 * (32 * TM) * kGrLd * 2; }
-
-// TM = 32-row tiles of x per workgroup (block tile 256 x 32 TM): 4 for prefill, 2 and 1 for
-// shorter x.  kSplit: blockIdx.z picks a contiguous share of the k tiles and the block writes
-// fp32 partial sums to part[z][M][N] instead of y (summed, scaled and rounded by
-// splitk_reduce_kernel), so that short x still fills the chip with workgroups.
-template <int TM, bool kSplit, bool kPacked>
-__global__ __launch_bounds__(256) void gemm_reg_kernel(const uint16_t *__restrict__ x,
-                                                       const uint16_t *__restrict__ codes,
-                                                       const void *__restrict__ grid, float scale,
-                                                       uint16_t *__restrict__ y, float *__restrict__ part,
-                                                       int M, int N, int K, int splits, int y_vec)
-{
-    constexpr int kBM = 32 * TM;
-    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31, kq = lane >> 5;
-    const uint32_t lane_base = (uint32_t)(lane & 15) * 16u;
-    const uint32_t quarter_bits = 0x34003400u;
-    // Workgroups go to the 8 XCDs round robin by linear id, so with m fastest the workgroups
-    // of one XCD share a few x row blocks (which then stay in that XCD's L2) and stream the codes.
-    const int m0 = blockIdx.x * kBM;
-    const int n0 = blockIdx.y * kGrBN;
-    const int row_bytes = K >> 2;
-    constexpr int kOut = (int)0x80000000;
-    // this block's k tiles: [kt_lo, kt_lo + k_tiles)
-    int kt_lo = 0, k_tiles = K / kGrBK;
-    if (kSplit) {
-        const int z = blockIdx.z, tq = k_tiles / splits, tr = k_tiles % splits;
-        kt_lo = z * tq + (z < tr ? z : tr);
-        k_tiles = tq + (z < tr ? 1 : 0);
-    }
-
-    // tables: thread tid owns grid row tid (16 copies) and 8 of the 2048 sign slots
-    {
-        const u4_t grow = reinterpret_cast<const u4_t *>(grid)[tid];
-        u4_t *gg = reinterpret_cast<u4_t *>(smem_raw + kSSignBytes);
-        u4_t *sg = reinterpret_cast<u4_t *>(smem_raw);
-#pragma unroll
-        for (int i = 0; i < 8; i++) sg[tid + i * 256] = sign_row((uint32_t)((tid + i * 256) >> 4));
-#pragma unroll
-        for (int i = 0; i < 16; i++) gg[tid * 16 + ((i + tid) & 15)] = grow;   // 16 lanes, 16 bank groups
-    }
-
-    // global sources.  Codes: lane (row l32 of tile i, half kq) reads 8 bytes = codes 4 kq .. 4 kq + 3
-    // of the k tile.  x: load p of thread tid is piece tid % 8 (16 bytes) of row 32 p + tid / 8, so
-    // that 8 lanes cover one 128-byte line.  Both as raw buffer
-    // loads: rows past N / M and tiles past the end get zeros without a memory access.
-    // Packed codes (pack_kernel): the 16 bytes of (row, k tile) sit at
-    // (((row / 16) * (K / 256) + kt / 4) * 64 + (kt % 4) * 16 + row % 16) * 16, so the per-tile part
-    // of the offset is kt * 256 and a wave's load is two runs of 256 consecutive bytes instead
-    // of 32 pieces of 16.
-    const int n_pad = ((N + 15) >> 4) << 4;
-    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kPacked ? n_pad : N) * row_bytes), 0x00020000);
-    const __amdgpu_buffer_rsrc_t xrsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x), 0, (int)((int64_t)M * K * 2), 0x00020000);
-    // Row-major codes travel four k tiles at a time: lane (row, half kq) loads the 32 bytes of its row that
-    // hold tiles 4 j + 2 kq and 4 j + 2 kq + 1 whole, so the two lanes of a row take 64 consecutive bytes
-    // (half a cache line per visit, not 16 bytes of it), and one v_permlane32_swap per word hands lanes
-    // l and l + 32 the halves they need of each other's tiles.  Tiles past the end of the block's share read
-    // whatever follows in the row (zeros past the end of the matrix); their x is zero, so they add nothing.
-    constexpr bool kWide = !kPacked;
-    int cvoff[kGrTN];
-#pragma unroll
-    for (int i = 0; i < kGrTN; i++) {
-        const int n = n0 + wave * 64 + i * 32 + l32;
-        if (kPacked) cvoff[i] = n < n_pad ? (n >> 4) * (K >> 8) * 1024 + (n & 15) * 16 + kq * 8 : kOut;
-        else cvoff[i] = n < N ? n * row_bytes + kq * 32 : kOut;
-    }
-    // rows r and r + 8 share a group of 16 lanes: with the 144-byte pitch their 16 pieces fall in
-    // 16 different bank groups, so the LDS writes below are conflict-free like the fragment reads
-    const int x_row = ((tid >> 7) << 4) + ((tid >> 4) & 7) + (((tid >> 3) & 1) << 3), x_piece = tid & 7;
-    int xvoff[TM];
-#pragma unroll
-    for (int p = 0; p < TM; p++) {
-        const int m = m0 + 32 * p + x_row;
-        xvoff[p] = m < M ? (m * K + x_piece * 8) * 2 : kOut;
-    }
-
-    struct Stage {
-        u2_t cw[kGrTN];
-        u4_t xv[TM];
-    };
-    auto load_codes = [&](Stage &st, int kt) {   // kt counts this block's tiles (packed codes: one tile at a time)
-        const int coff = kt < k_tiles ? (kt_lo + kt) * 256 : kOut;
-#pragma unroll
-        for (int i = 0; i < kGrTN; i++) st.cw[i] = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
-    };
-    // the codes of four tiles (row-major codes): w[row tile][h] holds, once swapped, tile h of the four in
-    // words 0 and 1 and tile h + 2 in words 2 and 3
-    struct CodeTrip {
-        u4_t w[kGrTN][2];
-    };
-    auto load_trip = [&](CodeTrip &ct, int kt) {   // kt: the first of the four tiles, counted within the block
-        const int coff = kt < k_tiles ? (kt_lo + kt) * 16 : kOut;
-#pragma unroll
-        for (int i = 0; i < kGrTN; i++)
-#pragma unroll
-            for (int h = 0; h < 2; h++) ct.w[i][h] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, cvoff[i] + 16 * h, coff, 0);
-    };
-    auto swap_trip = [&](CodeTrip &ct) {
-#pragma unroll
-        for (int i = 0; i < kGrTN; i++)
-#pragma unroll
-            for (int h = 0; h < 2; h++)
-#pragma unroll
-                for (int w = 0; w < 2; w++) {
-                    const u2_t r = __builtin_amdgcn_permlane32_swap(ct.w[i][h][w], ct.w[i][h][w + 2], false, false);
-                    ct.w[i][h][w] = r[0];
-                    ct.w[i][h][w + 2] = r[1];
-                }
-    };
-    auto load_x = [&](Stage &st, int kt, int p) {
-        const int xoff = kt < k_tiles ? (kt_lo + kt) * 128 : kOut;
-        st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
-    };
-    auto load_tile = [&](Stage &st, int kt) {
-        if constexpr (!kWide) load_codes(st, kt);
-#pragma unroll
-        for (int p = 0; p < TM; p++) load_x(st, kt, p);
-    };
-    unsigned char *xs = smem_raw + kSTablesBytes;                       // [2][kBM][kGrLd] halves
-    const uint32_t xs_w = (uint32_t)(x_row * kGrLd + x_piece * 8) * 2u;                      // this thread's write slot (p = 0)
-    const uint32_t xs_r = lds_addr(xs) + (uint32_t)(l32 * kGrLd + kq * 32) * 2u;             // this lane's B fragments
-    constexpr uint32_t kXBuf = kBM * kGrLd * 2;
-
-    CodeTrip cur, nxt;   // row-major codes: the four tiles being decoded and the four after them
-    if constexpr (kWide) load_trip(nxt, 0);
-    Stage ring[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) load_tile(ring[i], i);
-
-    f16_t acc[kGrTN][TM];
-#pragma unroll
-    for (int i = 0; i < kGrTN; i++)
-#pragma unroll
-        for (int j = 0; j < TM; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
-
-    // A fragments of one k tile: [tile i][k step s], a decoded code each
-    u4_t afr[2][kGrTN][4];
-    auto x_store = [&](const Stage &st, int buf, int p) {
-        *reinterpret_cast<u4_t *>(xs + xs_w + buf * kXBuf + p * (32 * kGrLd * 2)) = st.xv[p];
-    };
-    // The decode runs as a stream of units, one per k step: unit u of a tile is word u / 2 of
-    // row tile u % 2 (two codes = two k steps of that row tile).  A step gathers the table
-    // rows of its unit and finishes (packed FMAs) the unit gathered one step earlier, so no
-    // step waits for its own gathers.
-    StreamGather g[2];
-    // unit u of tile kI of the four in `ct` (row-major codes) or of the tile in `st` (packed codes)
-    auto unit_gather = [&](StreamGather &o, const Stage &st, const CodeTrip &ct, int kI, int u) {
-        const uint32_t cwd = kWide ? ct.w[u & 1][kI & 1][2 * (kI >> 1) + (u >> 1)] : st.cw[u & 1][u >> 1];
-        stream_gather(o, cwd, lane_base, quarter_bits);
-    };
-    auto unit_finish = [&](const StreamGather &o, int abuf, int u) {
-        afr[abuf][u & 1][2 * (u >> 1)] = __builtin_bit_cast(u4_t, gemm_finish<false>(o.g0, o.s0, o.dd));
-        afr[abuf][u & 1][2 * (u >> 1) + 1] = __builtin_bit_cast(u4_t, gemm_finish<true>(o.g1, o.s1, o.dd));
-    };
-
-    __syncthreads();   // tables ready
-    if constexpr (kWide) swap_trip(nxt);
-#pragma unroll
-    for (int u = 0; u < 4; u++) {
-        unit_gather(g[u & 1], ring[0], nxt, 0, u);
-        if (u < 3) unit_finish(g[u & 1], 0, u);   // unit 3 is finished by the first step of the loop
-    }
-    if constexpr (kWide) {
-        cur = nxt;
-        load_trip(nxt, 4);
-    }
-#pragma unroll
-    for (int p = 0; p < TM; p++) x_store(ring[0], 0, p);
-    __syncthreads();   // x tile 0 staged
-
-    auto read_b = [&](u4_t (&b)[TM], int buf, int s) {
-#pragma unroll
-        for (int j = 0; j < TM; j++) b[j] = lds_read16(xs_r + buf * kXBuf + (uint32_t)(j * 32 * kGrLd * 2 + s * 16));
-    };
-    u4_t b[2][TM];   // the x fragments of the current and the next MFMA step
-    read_b(b[0], 0, 0);
-    // MFMAs of tile kt (A = afr[buf], B from x buffer buf) while tile kt+1 (registers sn) is
-    // decoded into afr[buf ^ 1] and its x written to buffer buf ^ 1, and tile kt+4 is fetched
-    // into sf.  Past the last tile sn holds zeros (out-of-range loads): decoding and storing
-    // them is harmless and keeps every step one straight line of code, which the scheduling
-    // hints below then weave into groups of one MFMA, LDS reads and VALU: with one wave per
-    // SIMD nothing else hides the non-matrix instructions.
-    constexpr int kMfma = kGrTN * TM;                       // MFMAs per k step
-    constexpr int kDsPer = (TM + 4 + kMfma - 1) / kMfma;    // LDS reads per MFMA group
-    constexpr int kValuPer = (24 + kMfma - 1) / kMfma;      // VALU per MFMA group
-    // kNext (row-major codes): which of its four tiles tile kt+1 is; 0 = the first of the four after
-    // the current ones, which then become the current ones while the loads of the four after them start
-    auto tile = [&](int kt, int buf, const Stage &sn, Stage &sf, auto next_tag) {
-        constexpr int kNext = decltype(next_tag)::value;
-        if constexpr (kWide && kNext == 0) swap_trip(nxt);
-        const CodeTrip &ct = kNext == 0 ? nxt : cur;
-#pragma unroll
-        for (int s = 0; s < 4; s++) {
-            // the global loads of tile kt+4 spread over the steps, woven between the MFMAs too
-            if (!kWide && s == 0) load_codes(sf, kt + 4);
-            if (TM == 4 && (s == 1 || s == 2)) {
-                load_x(sf, kt + 4, 2 * s - 2);
-                load_x(sf, kt + 4, 2 * s - 1);
-            }
-            if (TM < 4 && s >= 1 && s <= TM) load_x(sf, kt + 4, s - 1);
-            // unit 3 of the CURRENT tile was gathered in the last step of the previous tile
-            unit_finish(g[(s + 1) & 1], s == 0 ? buf : buf ^ 1, (s + 3) & 3);
-            unit_gather(g[s & 1], sn, ct, kNext, s);
-            if (s < 3) read_b(b[(s + 1) & 1], buf, s + 1);
-            else read_b(b[0], buf ^ 1, 0);   // step 0 of tile kt + 1: its x is in place since the barrier
-            if (kWide && kNext == 0 && s == 3) {
-                cur = nxt;
-                load_trip(nxt, kt + 5);   // tile kt + 1 is the first of the new current four
-            }
-#pragma unroll
-            for (int i = 0; i < kGrTN; i++)
-#pragma unroll
-                for (int j = 0; j < TM; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, afr[buf][i][s]),
-                                                                       __builtin_bit_cast(h8_t, b[s & 1][j]), acc[i][j], 0, 0, 0);
-            // the x of tile kt + 1 goes to the other buffer in steps 0 .. 2, ahead of the barrier
-            if (TM == 4) {
-                if (s == 0) x_store(sn, buf ^ 1, 0);
-                if (s == 1) {
-                    x_store(sn, buf ^ 1, 1);
-                    x_store(sn, buf ^ 1, 2);
-                }
-                if (s == 2) x_store(sn, buf ^ 1, 3);
-            } else if (s < TM) {
-                x_store(sn, buf ^ 1, s);
-            }
-#pragma unroll
-            for (int r = 0; r < kMfma; r++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x100, kDsPer, 0);     // LDS reads
-                __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0);   // VALU
-                if (s < 3 && (r == 1 || r == kMfma / 2)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
-                if (kWide && kNext == 0 && s == 3 && r < 2 * kGrTN) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            }
-            if (TM == 4 ? s < 3 : s < TM) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // LDS writes
-            if (TM == 4 && s == 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            // The tile's one barrier lies between steps 2 and 3, not at its end, so that no tile starts by
-            // waiting for an LDS read behind a barrier: buffer buf ^ 1 was last read in step 2 of the tile
-            // before (the fragments of its step 3), ahead of that tile's barrier, and is read again in step 3.
-            if (s == 2) __syncthreads();
-        }
-    };
-
-    // Four tiles per trip with no way out in between: a path that left the loop body early
-    // would reach the loop head with the newest loads still pending on registers the body
-    // reuses, and the wait the compiler places there for that path (all loads done) would
-    // be paid by every trip.  The up to three tiles left over run after the loop.
-    int kt = 0;
-    typedef std::integral_constant<int, 0> N0;
-    typedef std::integral_constant<int, 1> N1;
-    typedef std::integral_constant<int, 2> N2;
-    typedef std::integral_constant<int, 3> N3;
-    for (; kt + 4 <= k_tiles; kt += 4) {
-        tile(kt, 0, ring[1], ring[0], N1{});
-        tile(kt + 1, 1, ring[2], ring[1], N2{});
-        tile(kt + 2, 0, ring[3], ring[2], N3{});
-        tile(kt + 3, 1, ring[0], ring[3], N0{});
-    }
-    if (kt < k_tiles) tile(kt, 0, ring[1], ring[0], N1{});
-    if (kt + 1 < k_tiles) tile(kt + 1, 1, ring[2], ring[1], N2{});
-    if (kt + 2 < k_tiles) tile(kt + 2, 0, ring[3], ring[2], N3{});
-
-    // D layout of 32x32: element e of lane: row (n) = 8*(e/4) + 4*(lane/32) + e%4, column (m) = lane%32
-    const bool n_vec = (N & 3) == 0 && (kSplit || y_vec != 0);   // 8-byte stores need an 8-byte aligned y
-#pragma unroll
-    for (int i = 0; i < kGrTN; i++)
-#pragma unroll
-        for (int j = 0; j < TM; j++) {
-            const int m = m0 + j * 32 + l32;
-            if (m >= M) continue;
-#pragma unroll
-            for (int e4 = 0; e4 < 4; e4++) {
-                const int n = n0 + wave * 64 + i * 32 + 8 * e4 + 4 * kq;
-                if (kSplit) {
-                    float *dst = part + ((int64_t)blockIdx.z * M + m) * N + n;
-                    if (n_vec && n + 3 < N) {
-                        *reinterpret_cast<f4_t *>(dst) =
-                            f4_t{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            if (n + e < N) dst[e] = acc[i][j][4 * e4 + e];
-                    }
-                    continue;
-                }
-                uint16_t o[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    o[e] = __builtin_bit_cast(uint16_t, (half_t)(acc[i][j][4 * e4 + e] * scale));
-                uint16_t *dst = y + (int64_t)m * N + n;
-                if (n_vec && n + 3 < N) {
-                    u2_t v;
-                    v[0] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-                    v[1] = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
-                    *reinterpret_cast<u2_t *>(dst) = v;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (n + e < N) dst[e] = o[e];
-                }
-            }
-        }
-}
-
-// y = half(scale * sum_z part[z]) over M * N elements; the order of the sum is fixed, so the
-// result does not depend on how the blocks were scheduled.
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ part, uint16_t *__restrict__ y,
-                                                            int64_t mn, int splits, float scale)
-{
-    const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i4 >= mn) return;
-    if (i4 + 3 < mn && (mn & 3) == 0) {
-        f4_t sacc = *reinterpret_cast<const f4_t *>(part + i4);
-        for (int z = 1; z < splits; z++) sacc += *reinterpret_cast<const f4_t *>(part + (int64_t)z * mn + i4);
-        u2_t v;
-        v[0] = (uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sacc[0] * scale)) |
-               ((uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sacc[1] * scale)) << 16);
-        v[1] = (uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sacc[2] * scale)) |
-               ((uint32_t)__builtin_bit_cast(uint16_t, (half_t)(sacc[3] * scale)) << 16);
-        *reinterpret_cast<u2_t *>(y + i4) = v;
-    } else {
-        for (int64_t i = i4; i < mn && i < i4 + 4; i++) {
-            float sacc = part[i];
-            for (int z = 1; z < splits; z++) sacc += part[(int64_t)z * mn + i];
-            y[i] = __builtin_bit_cast(uint16_t, (half_t)(sacc * scale));
-        }
-    }
-}
-
-// ------------------------------------------------------------------ the reference's integer operator
-// out[m,n] = sum_k x[m,k] * W[n,k] in int32, W decoded to int8 from the packed int64 table
-// exactly as /root/reference/test_decode_matmul.py:29-55 (value = +-byte, then +1 or -1, kept
-// in int8).  Codes may be in the layout the reference's kernel reads
-// (/root/reference/test_decode_matmul.py:101-109: 16-row x 4-column tiles of 64 codes ordered
-// [row % 8][column % 4][row / 8]) or plain row-major.  One wave per output row, integer
-// arithmetic throughout, so the result is exact for any K (the sum wraps in int32 like the
-// reference's accumulator).  A correctness path, not a tuned one (no matrix unit).
-__device__ __forceinline__ int64_t tiled_code_index(int64_t n, int64_t j, int64_t kc)
-{
-    return ((n >> 4) * (kc >> 2) + (j >> 2)) * 64 + (n & 7) * 8 + (j & 3) * 2 + ((n >> 3) & 1);
-}
-
-__device__ __forceinline__ int wave_sum_i32(int v)
-{
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-
-// Weights of one code, exactly as the reference's scalar decode: +-byte, then +1 or -1, kept in int8.
-__device__ __forceinline__ void int8_decode_exact(uint64_t abs, uint32_t c, int (&w)[8])
-{
-    uint32_t s8 = (c >> 8) & 0x7Fu;
-    s8 |= (__builtin_popcount(s8) & 1u) << 7;
-    const int shift = (c >> 15) & 1;
-#pragma unroll
-    for (int d = 0; d < 8; d++) {
-        int8_t v = (int8_t)(abs & 0xFFu);
-        if ((s8 >> d) & 1u) v = (int8_t)(-v);
-        v = (int8_t)(shift ? v - 1 : v + 1);
-        w[d] = v;
-        abs >>= 8;
-    }
-}
-
-// kFast: every byte of the table is 2 mod 4 (the E8P table is: 4 x a half-odd value).  Then
-// negating a byte flips its upper six bits, adding 1 sets its lowest bit and subtracting 1
-// turns the low bits 10 into 01 - the whole decode is one exclusive or with a mask that depends
-// only on the code's high byte (/root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:45-65
-// uses the same property), and the 8 products of a code are two 4-way int8 dot products.
-// Otherwise (kFast false) the scalar decode above, byte by byte.  x8: x and K allow 8-byte loads.
-// Rows n_first, n_first + n_stride, ... below n_end, one wave each.
-template <bool kFast>
-__device__ __forceinline__ void int8_rows(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
-                                          const uint64_t *table, const uint64_t *masks, int32_t *__restrict__ out,
-                                          int64_t M, int64_t N, int64_t K, int tiled, bool x8, int64_t n_first,
-                                          int64_t n_stride, int64_t n_end)
-{
-    const int lane = threadIdx.x & 63;
-    const int64_t kc = K >> 3;
-    constexpr int kMC = 8;
-    for (int64_t n = n_first; n < n_end; n += n_stride) {
-        for (int64_t m0 = 0; m0 < M; m0 += kMC) {
-            int acc[kMC] = {};
-            for (int64_t j = lane; j < kc; j += kWave) {
-                const uint32_t c = codes[tiled ? tiled_code_index(n, j, kc) : n * kc + j];
-                if (kFast) {
-                    const uint64_t w8 = table[c & 0xFFu] ^ masks[c >> 8];
-                    const int wlo = (int)(uint32_t)w8, whi = (int)(uint32_t)(w8 >> 32);
-#pragma unroll
-                    for (int mm = 0; mm < kMC; mm++) {
-                        if (m0 + mm < M) {
-                            const int8_t *xr = x + (m0 + mm) * K + j * 8;
-                            int xlo, xhi;
-                            if (x8) {
-                                const u2_t v = *reinterpret_cast<const u2_t *>(xr);
-                                xlo = (int)v[0];
-                                xhi = (int)v[1];
-                            } else {
-                                xlo = (int)((uint32_t)(uint8_t)xr[0] | (uint32_t)(uint8_t)xr[1] << 8 |
-                                            (uint32_t)(uint8_t)xr[2] << 16 | (uint32_t)(uint8_t)xr[3] << 24);
-                                xhi = (int)((uint32_t)(uint8_t)xr[4] | (uint32_t)(uint8_t)xr[5] << 8 |
-                                            (uint32_t)(uint8_t)xr[6] << 16 | (uint32_t)(uint8_t)xr[7] << 24);
-                            }
-                            acc[mm] = __builtin_amdgcn_sdot4(xlo, wlo, acc[mm], false);
-                            acc[mm] = __builtin_amdgcn_sdot4(xhi, whi, acc[mm], false);
-                        }
-                    }
-                } else {
-                    int w[8];
-                    int8_decode_exact(table[c & 0xFFu], c, w);
-#pragma unroll
-                    for (int mm = 0; mm < kMC; mm++) {
-                        if (m0 + mm < M) {
-                            const int8_t *xr = x + (m0 + mm) * K + j * 8;
-#pragma unroll
-                            for (int d = 0; d < 8; d++) acc[mm] += (int)xr[d] * w[d];
-                        }
-                    }
-                }
-            }
-#pragma unroll
-            for (int mm = 0; mm < kMC; mm++) {
-                const int sum = wave_sum_i32(acc[mm]);
-                if (lane == 0 && m0 + mm < M) out[(m0 + mm) * N + n] = sum;
-            }
-        }
-    }
-}
-
-__global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
-                                                   const int64_t *__restrict__ codebook_abs,
-                                                   int32_t *__restrict__ out, int64_t M, int64_t N, int64_t K,
-                                                   int tiled, int x8)
-{
-    __shared__ uint64_t table[256];
-    __shared__ uint64_t masks[256];
-    __shared__ int slow[4];
-    const uint64_t abs = (uint64_t)codebook_abs[threadIdx.x];
-    table[threadIdx.x] = abs;
-    {
-        // mask of high byte t: sign bits t & 0x7F (the eighth by parity), shift t >> 7
-        uint32_t s8 = threadIdx.x & 0x7Fu;
-        s8 |= (__builtin_popcount(s8) & 1u) << 7;
-        uint64_t mk = (threadIdx.x >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
-#pragma unroll
-        for (int d = 0; d < 8; d++)
-            if ((s8 >> d) & 1u) mk ^= 0xFCull << (8 * d);
-        masks[threadIdx.x] = mk;
-    }
-    const bool bad = (abs & 0x0303030303030303ull) != 0x0202020202020202ull;
-    const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
-    if ((threadIdx.x & 63) == 0) slow[threadIdx.x >> 6] = wave_bad ? 1 : 0;
-    __syncthreads();
-    const int64_t n_first = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), n_stride = (int64_t)gridDim.x * 4;
-    if (slow[0] | slow[1] | slow[2] | slow[3])
-        int8_rows<false>(x, codes, table, masks, out, M, N, K, tiled, false, n_first, n_stride, N);
-    else
-        int8_rows<true>(x, codes, table, masks, out, M, N, K, tiled, x8 != 0, n_first, n_stride, N);
-}
-
-// ------------------------------------------------------------------ the integer operator on the matrix unit
-// M <= 16, K a multiple of 256, a table whose bytes are all 2 mod 4 (see int8_rows): the
-// small-batch kernel's structure (persistent workgroups over contiguous ranges of 16-row tiles,
-// k steps of 256 dealt to 8 waves, x fetched from L2 into registers with the codes as one
-// prefetch unit, partial sums through LDS) with the decode done in bytes - one 8-byte gather of
-// the table entry by the code's low byte, one of the mask by its high byte, exclusive or - and
-// v_mfma_i32_16x16x64_i8: a lane's 8 codes of a step are the A operands of four MFMAs (two codes =
-// 16 k each), B is 16 bytes of x per lane and MFMA.  Both tables hold 32 copies of every 8-byte
-// row (row pitch 256 B, lane reads copy lane % 32: no bank conflicts for any codes).  Exact:
-// int8 products, int32 sums (which wrap like the reference's accumulator).
-// Codes row-major, or in the reference's tile order (/root/reference/test_decode_matmul.py:101-109):
-// there 16 bytes hold codes (row g, columns c .. c + 3) interleaved with row g + 8's, so lanes g
-// and g + 8 load the same two pieces and each keeps its halves (one v_perm per two codes).
-// A table with any other byte is found while the tables are built, and the workgroup then does
-// its rows with the scalar decode instead.
-typedef int i4_t __attribute__((ext_vector_type(4)));
-constexpr int kI8TableBytes = 256 * 256;   // one table: 256 rows x 32 copies x 8 bytes
-
-template <int R, int W, int D, bool kTiled>
-__global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
-                                                       const int64_t *__restrict__ codebook_abs,
-                                                       int32_t *__restrict__ out, int M, int N, int K, int tiles_q,
-                                                       int tiles_r)
-{
-    static_assert(W == 8, "the table staging below assumes 512 threads");
-    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    // partial sums: two buffers taken in turn while they fit beside the tables (R <= 2), else one
-    // and a second barrier per row block
-    constexpr bool kTwoBuffers = R <= 2;
-    typedef i4_t red_t[W][R][kWave];
-    red_t *red = reinterpret_cast<red_t *>(smem_raw + 2 * kI8TableBytes);   // red[parity]
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int c16 = lane & 15;
-    const int q = lane >> 4;
-    const int n_steps = K >> 8;
-    const int row_bytes = K >> 2;
-    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;          // grid rows: [0, 64K)
-    const uint32_t lane_base2 = lane_base | 0x10000u;               // mask rows: [64K, 128K)
-
-    uint64_t entry = 0;
-    if (tid < 256) entry = (uint64_t)codebook_abs[tid];
-
-    const int n_sw = wave < n_steps ? (n_steps - wave + W - 1) / W : 0;
-    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
-    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
-    const int nb_wg = (t1 - t0 + R - 1) / R;
-
-    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kTiled ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
-    const __amdgpu_buffer_rsrc_t xrsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(x), 0, M * K, 0x00020000);
-    constexpr int kOut = (int)0x80000000;
-    // per-lane byte offsets inside a row block.  Row-major: row 16 r + c16, 16 bytes at quarter q.
-    // Tiled: the tile row of the block is 16 rows x K / 4 bytes as well, a tile (4 code columns) is
-    // 128 bytes, and lane (g = c16 % 8, quarter q) reads 16 bytes at g * 16 of tiles 2 q and 2 q + 1
-    // of the step's 8.
-    int voff[R];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-        voff[r] = kTiled ? r * 16 * row_bytes + q * 256 + (c16 & 7) * 16 : (16 * r + c16) * row_bytes + q * 16;
-    const int xoff = c16 < M ? c16 * K + 64 * q : kOut;   // columns past M: zeros, no memory access
-    const uint32_t half_sel = (c16 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
-
-    struct Unit {
-        u4_t cw[R][kTiled ? 2 : 1];
-        u4_t xb[4];
-    };
-    int pf_blk = 0, pf_j = 0;
-    auto issue = [&](Unit &u) {
-        const bool ok = pf_blk < nb_wg && n_sw > 0;
-        const int step = wave + pf_j * W;
-        const int xs_off = ok ? step * 256 : kOut;
-        const int tb = t0 + pf_blk * R;
-        const int soff = !ok ? kOut : kTiled ? tb * 16 * row_bytes + step * 1024 : tb * 16 * row_bytes + step * 64;
-#pragma unroll
-        for (int t = 0; t < 4; t++) u.xb[t] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff + t * 16, xs_off, 0);
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int so = (r == 0 || tb + r < t1) ? soff : kOut;
-            u.cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], so, 0);
-            if (kTiled) u.cw[r][kTiled ? 1 : 0] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r] + 128, so, 0);
-        }
-        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
-    };
-
-    Unit ring[D];
-#pragma unroll
-    for (int d = 0; d < D; d++) issue(ring[d]);
-
-    // tables: threads 0 .. 255 write the 32 copies of table entry tid (16 slots of two copies),
-    // threads 256 .. 511 those of the mask of high byte tid - 256
-    bool bad = false;
-    {
-        uint64_t v = entry;
-        if (tid < 256) {
-            bad = (entry & 0x0303030303030303ull) != 0x0202020202020202ull;
-        } else {
-            const uint32_t t = (uint32_t)tid - 256u;
-            uint32_t s8 = t & 0x7Fu;
-            s8 |= (__builtin_popcount(s8) & 1u) << 7;
-            v = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
-#pragma unroll
-            for (int d = 0; d < 8; d++)
-                if ((s8 >> d) & 1u) v ^= 0xFCull << (8 * d);
-        }
-        const uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
-        // tid >= 256 lands in the mask table; slot i ^ (tid % 16): 16 lanes, 16 bank groups, one exclusive or per address
-        const uint32_t rowp = lds_addr(smem_raw) + (uint32_t)((tid * 16 + (tid & 15)) * 16);
-#pragma unroll
-        for (int i = 0; i < 16; i++) lds_write16(rowp ^ (uint32_t)(i * 16), u4_t{lo, hi, lo, hi});
-    }
-    // the vote on the table: one word per wave in the partial-sum area, read by everybody after the barrier
-    uint32_t *votes = reinterpret_cast<uint32_t *>(smem_raw + 2 * kI8TableBytes);
-    const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
-    if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
-    __syncthreads();
-    const bool any_bad = __builtin_amdgcn_ballot_w64(votes[lane & (W - 1)] != 0) != 0;
-    __syncthreads();   // the votes are read before partial sums overwrite them
-    if (any_bad) {
-        // scalar decode for this workgroup's rows; the raw table goes where the partial sums would
-        uint64_t *table = reinterpret_cast<uint64_t *>(smem_raw + 2 * kI8TableBytes);
-        if (tid < 256) table[tid] = entry;
-        __syncthreads();
-        const int64_t n_end = (int64_t)t1 * 16 < N ? (int64_t)t1 * 16 : N;
-        int8_rows<false>(x, codes, table, table, out, M, N, K, kTiled ? 1 : 0, false, (int64_t)t0 * 16 + wave, W, n_end);
-        return;
-    }
-
-    i4_t acc[R][2];
-#pragma unroll
-    for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = i4_t{0, 0, 0, 0};
-
-    auto finish_block = [&](int blk) {
-        const int par = kTwoBuffers ? blk & 1 : 0;
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            red[par][wave][r][lane] = acc[r][0] + acc[r][1];
-            acc[r][0] = acc[r][1] = i4_t{0, 0, 0, 0};
-        }
-        __syncthreads();
-        for (int r = wave; r < R; r += W) {
-            i4_t sacc = red[par][0][r][lane];
-#pragma unroll
-            for (int w = 1; w < W; w++) sacc += red[par][w][r][lane];
-            const int rt = t0 + blk * R + r;
-            const int n = rt * 16 + 4 * q;
-            if (c16 < M && rt < t1 && n < N)   // N % 4 == 0, so the four rows are in range together
-                *reinterpret_cast<i4_t *>(out + (int64_t)c16 * N + n) = sacc;
-        }
-        if (!kTwoBuffers) __syncthreads();   // the next block's sums go to the same buffer
-    };
-
-    if (n_sw == 0) {
-        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
-        return;
-    }
-    const int n_items = nb_wg * n_sw;
-    int blk = 0, j = 0;
-    for (int i0 = 0; i0 < n_items; i0 += D) {
-#pragma unroll
-        for (int d = 0; d < D; d++) {
-            if (i0 + d < n_items) {
-                const Unit &u = ring[d];
-                const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    if (r > 0 && r >= nv) break;
-                    u4_t cw;   // the lane's 8 codes of the step, two per word
-                    if (kTiled) {
-                        const u4_t &a = u.cw[r][0], &b = u.cw[r][kTiled ? 1 : 0];
-                        cw = u4_t{__builtin_amdgcn_perm(a[1], a[0], half_sel), __builtin_amdgcn_perm(a[3], a[2], half_sel),
-                                  __builtin_amdgcn_perm(b[1], b[0], half_sel), __builtin_amdgcn_perm(b[3], b[2], half_sel)};
-                    } else {
-                        cw = u.cw[r][0];
-                    }
-                    u2_t g[8], m[8];
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const uint32_t w = cw[i];
-                        g[2 * i] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
-                        m[2 * i] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
-                        g[2 * i + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
-                        m[2 * i + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
-                    }
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const i4_t a = i4_t{(int)(g[2 * i][0] ^ m[2 * i][0]), (int)(g[2 * i][1] ^ m[2 * i][1]),
-                                            (int)(g[2 * i + 1][0] ^ m[2 * i + 1][0]), (int)(g[2 * i + 1][1] ^ m[2 * i + 1][1])};
-                        acc[r][i & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, __builtin_bit_cast(i4_t, u.xb[i]), acc[r][i & 1], 0, 0, 0);
-                    }
-                }
-                if (++j >= n_sw) {
-                    j = 0;
-                    finish_block(blk);
-                    blk++;
-                }
-            }
-            issue(ring[d]);
-        }
-    }
-}
-
-
-// ------------------------------------------------------------------ the integer operator, many rows of x
-// Block tile 256 (n) x 128 (m), eight waves in two groups of four.  A group is a complete
-// 256 x 128 x 64 pipeline - one wave per SIMD, each 64 rows of W (two 32-row tiles) x all 128 rows
-// of x = 8 accumulators of v_mfma_i32_32x32x32_i8 - and the two groups take the even and the odd k
-// tiles of the same output tile, so that every SIMD holds two waves working on different k tiles:
-// while one waits for its table gathers or its x fragments the other's MFMAs run.  At the end each
-// group hands the other the partial sums of one of its two row tiles through the LDS (the tables'
-// space, by then free) and stores the other one.
-// Like the half-precision gemm_reg_kernel, every wave decodes its own rows straight into A
-// operands - here that is two 8-byte gathers and two exclusive ors per code (int8x_kernel's
-// tables), eight codes per lane and k tile - and only x goes through the LDS: four buffers (two
-// per group) of 128 rows x 64 bytes, the 16-byte pieces of a row exchanged by (row / 4) % 4 so
-// that the 16 lanes the LDS serves per clock hit 16 different bank groups without padding (the
-// tables take 128 KB of the 160).  Lane (row, half h = lane / 32) takes codes 4 h .. 4 h + 3 of its
-// row's 8 in the k tile (8 consecutive bytes; in the reference's tile order, the 16 bytes of the
-// pair of rows, of which one v_perm per two codes keeps ours) and pairs them with bytes 32 h ..
-// 32 h + 31 of the x rows.
-// The decode runs one k tile ahead of the MFMAs as a stream of units (the two codes of one row tile
-// and MFMA step): a step gathers the table rows of two units and finishes (exclusive ors) the two
-// gathered a step earlier, and scheduling hints weave that between the step's eight MFMAs.  Global
-// loads run three of the group's k tiles ahead in a ring of registers; one barrier per pair of k
-// tiles (one of either group).
-// A table with a byte that is not 2 mod 4: the workgroup does its tile with the scalar decode.
-typedef int i16_t __attribute__((ext_vector_type(16)));
-constexpr int kI8gBN = 256, kI8gBM = 128, kI8gBK = 64;
-constexpr int kI8gXBuf = kI8gBM * kI8gBK;                       // one x tile, unpadded
-constexpr int kI8gSmem = 2 * kI8TableBytes + 4 * kI8gXBuf;      // 160 KB
-
-template <bool kTiled>
-__global__ __launch_bounds__(512) void int8g_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
-                                                    const int64_t *__restrict__ codebook_abs,
-                                                    int32_t *__restrict__ out, int M, int N, int K)
-{
-    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    unsigned char *xs = smem_raw + 2 * kI8TableBytes;   // x tiles: [group][buffer]
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int grp = wave >> 2, w4 = wave & 3;            // group (k tile parity) and place along n
-    const int gtid = tid & 255;
-    const int l32 = lane & 31, kq = lane >> 5;
-    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;   // grid rows: [0, 64K)
-    const uint32_t lane_base2 = lane_base | 0x10000u;        // mask rows: [64K, 128K)
-    const int m0 = blockIdx.x * kI8gBM;
-    const int n0 = blockIdx.y * kI8gBN;
-    const int row_bytes = K >> 2;
-    const int k_tiles = K / kI8gBK;
-    const int g_tiles = (k_tiles + 1) >> 1;              // tiles per group (the odd group's last may not exist)
-    constexpr int kOut = (int)0x80000000;
-
-    // global sources, as raw buffer loads (rows past N / M and tiles past the end: zeros, no access)
-    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kTiled ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
-    const __amdgpu_buffer_rsrc_t xrsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(x), 0, (int)((int64_t)M * K), 0x00020000);
-    // codes of row tile i (32 rows): row-major 8 bytes at row * K / 4 + kt * 16 + 8 h; tiled: tile
-    // (row / 16, 2 kt + h) of 128 bytes, 16 bytes at (row % 8) * 16
-    int cvoff[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int n = n0 + w4 * 64 + i * 32 + l32;
-        if (kTiled) cvoff[i] = n < N ? (n >> 4) * 16 * row_bytes + kq * 128 + (n & 7) * 16 : kOut;
-        else cvoff[i] = n < N ? n * row_bytes + kq * 8 : kOut;
-    }
-    const uint32_t half_sel = (l32 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
-    // x: thread gtid of a group loads piece gtid % 4 (16 bytes) of rows gtid / 4 and gtid / 4 + 64 of the
-    // group's tile; in the LDS piece p of row r sits at r * 64 + (p ^ (r / 4) % 4) * 16
-    int xvoff[2];
-#pragma unroll
-    for (int p = 0; p < 2; p++) {
-        const int m = m0 + (gtid >> 2) + 64 * p;
-        xvoff[p] = m < M ? m * K + (gtid & 3) * 16 : kOut;
-    }
-    unsigned char *xg = xs + grp * 2 * kI8gXBuf;   // this group's two buffers
-    unsigned char *xw_ptr = xg + (gtid >> 2) * 64 + (((gtid & 3) ^ ((gtid >> 4) & 3)) << 4);
-    const uint32_t swz = (uint32_t)(l32 >> 2) & 3u;
-    const uint32_t xr_addr = lds_addr(xg) + (uint32_t)(l32 * 64);
-    const uint32_t xr_off[2] = {(((uint32_t)kq * 2u) ^ swz) << 4, (((uint32_t)kq * 2u + 1u) ^ swz) << 4};
-
-    struct Stage {
-        u4_t cw[2];   // row-major: only the low 8 bytes are loaded
-        u4_t xv[2];
-    };
-    auto load = [&](Stage &st, int t) {   // t: the group's tile, k tile 2 t + grp
-        const int kt = 2 * t + grp;
-        const int ok = kt < k_tiles;
-        const int coff = ok ? (kTiled ? kt * 256 : kt * 16) : kOut;
-        const int xoff = ok ? kt * kI8gBK : kOut;
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            if (kTiled) {
-                st.cw[i] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, cvoff[i], coff, 0);
-            } else {
-                const u2_t v = __builtin_amdgcn_raw_buffer_load_b64(crsrc, cvoff[i], coff, 0);
-                st.cw[i] = u4_t{v[0], v[1], 0u, 0u};
-            }
-        }
-#pragma unroll
-        for (int p = 0; p < 2; p++) st.xv[p] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xvoff[p], xoff, 0);
-    };
-    auto stage_x = [&](const Stage &st, int buf) {
-#pragma unroll
-        for (int p = 0; p < 2; p++) *reinterpret_cast<u4_t *>(xw_ptr + buf * kI8gXBuf + p * 64 * 64) = st.xv[p];
-    };
-    Stage ring[3];
-#pragma unroll
-    for (int d = 0; d < 3; d++) load(ring[d], d);
-
-    // tables: threads 0 .. 255 write the 32 copies of table entry tid, threads 256 .. 511 those of
-    // the mask of high byte tid - 256 (the mask table follows the grid table: row tid either way)
-    const uint64_t entry = tid < 256 ? (uint64_t)codebook_abs[tid] : 0x0202020202020202ull;
-    {
-        uint64_t v = entry;
-        if (tid >= 256) {
-            const uint32_t t = (uint32_t)tid - 256u;
-            uint32_t s8 = t & 0x7Fu;
-            s8 |= (__builtin_popcount(s8) & 1u) << 7;
-            v = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
-#pragma unroll
-            for (int d = 0; d < 8; d++)
-                if ((s8 >> d) & 1u) v ^= 0xFCull << (8 * d);
-        }
-        u4_t *rowp = reinterpret_cast<u4_t *>(smem_raw) + tid * 16;
-        const u4_t vv = u4_t{(uint32_t)v, (uint32_t)(v >> 32), (uint32_t)v, (uint32_t)(v >> 32)};
-#pragma unroll
-        for (int i = 0; i < 16; i++) rowp[(i + tid) & 15] = vv;   // 16 lanes, 16 bank groups
-    }
-    // the vote on the table (one word per wave in the x area, read by everybody after the barrier)
-    {
-        uint32_t *votes = reinterpret_cast<uint32_t *>(xs);
-        const bool bad = (entry & 0x0303030303030303ull) != 0x0202020202020202ull;
-        const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
-        if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
-        __syncthreads();
-        const bool any_bad = (votes[0] | votes[1] | votes[2] | votes[3]) != 0;   // the table is in waves 0 - 3
-        __syncthreads();   // the votes are read before x overwrites them
-        if (any_bad) {
-            uint64_t *table = reinterpret_cast<uint64_t *>(xs);
-            if (tid < 256) table[tid] = entry;
-            __syncthreads();
-            const int64_t n_end = (int64_t)n0 + kI8gBN < N ? (int64_t)n0 + kI8gBN : N;
-            const int64_t mc = M - m0 < kI8gBM ? M - m0 : kI8gBM;
-            int8_rows<false>(x + (int64_t)m0 * K, codes, table, table, out + (int64_t)m0 * N, mc, N, K, kTiled ? 1 : 0,
-                             false, (int64_t)n0 + wave, 8, n_end);
-            return;
-        }
-    }
-
-    i16_t acc[2][4];
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
-
-    // unit u of a tile: the two codes (8 weights each) of row tile u % 2 and MFMA step u / 2
-    struct Unit {
-        u2_t g[2], k[2];
-    };
-    i4_t afr[2][2][2];   // A operands: [buffer][row tile][MFMA step]
-    auto unit_gather = [&](Unit &o, const Stage &st, int u) {
-        const int i = u & 1, s2 = u >> 1;
-        const uint32_t w = kTiled ? __builtin_amdgcn_perm(st.cw[i][2 * s2 + 1], st.cw[i][2 * s2], half_sel) : st.cw[i][s2];
-        o.g[0] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
-        o.k[0] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
-        o.g[1] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
-        o.k[1] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
-    };
-    auto unit_finish = [&](const Unit &o, int abuf, int u) {
-        afr[abuf][u & 1][u >> 1] = i4_t{(int)(o.g[0][0] ^ o.k[0][0]), (int)(o.g[0][1] ^ o.k[0][1]),
-                                        (int)(o.g[1][0] ^ o.k[1][0]), (int)(o.g[1][1] ^ o.k[1][1])};
-    };
-    Unit ga[2], gb[2];   // units 0, 1 (MFMA step 0) and 2, 3 (step 1) in flight
-
-    auto read_b = [&](u4_t (&b)[4], int buf, int s2) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) b[j] = lds_read16(xr_addr + (uint32_t)(buf * kI8gXBuf + j * 32 * 64) + xr_off[s2]);
-    };
-    stage_x(ring[0], 0);
-    unit_gather(ga[0], ring[0], 0);
-    unit_gather(ga[1], ring[0], 1);
-    unit_finish(ga[0], 0, 0);
-    unit_finish(ga[1], 0, 1);
-    unit_gather(gb[0], ring[0], 2);
-    unit_gather(gb[1], ring[0], 3);
-    __syncthreads();   // x tile 0 of either group staged
-
-    // MFMAs of the group's tile t (A = afr[buf], B from the group's x buffer buf).  Step 0 finishes the
-    // tile's own second pair of units (gathered in the last step of the tile before), gathers the first
-    // pair of tile t + 1 (registers sn), writes the x of tile t + 1 to buffer buf ^ 1 and fetches tile
-    // t + 3 into sf; step 1 finishes that pair into afr[buf ^ 1] and gathers the second.  Each step
-    // reads its own x fragments as it starts: the SIMD's other wave covers the wait.
-    auto tile = [&](int t, int buf, const Stage &sn, Stage &sf) {
-        u4_t b[4];
-        read_b(b, buf, 0);
-        unit_finish(gb[0], buf, 2);
-        unit_finish(gb[1], buf, 3);
-        unit_gather(ga[0], sn, 0);
-        unit_gather(ga[1], sn, 1);
-        stage_x(sn, buf ^ 1);
-        load(sf, t + 3);
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[buf][i][0], __builtin_bit_cast(i4_t, b[j]), acc[i][j], 0, 0, 0);
-#pragma unroll
-        for (int r = 0; r < 8; r++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // MFMA
-            if (r < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // LDS reads
-            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                // VALU
-            if (r == 4) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);    // LDS writes
-            if (r >= 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // global loads
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        read_b(b, buf, 1);
-        unit_finish(ga[0], buf ^ 1, 0);
-        unit_finish(ga[1], buf ^ 1, 1);
-        unit_gather(gb[0], sn, 2);
-        unit_gather(gb[1], sn, 3);
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[buf][i][1], __builtin_bit_cast(i4_t, b[j]), acc[i][j], 0, 0, 0);
-#pragma unroll
-        for (int r = 0; r < 8; r++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // MFMA
-            if (r < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // LDS reads
-            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                // VALU
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-    };
-
-    // both groups make the same number of trips (the barriers are the workgroup's); six tiles per trip
-    // so that ring slot and x buffer are compile-time constants
-    int t = 0;
-    for (; t + 6 <= g_tiles; t += 6) {
-        tile(t, 0, ring[1], ring[0]);
-        tile(t + 1, 1, ring[2], ring[1]);
-        tile(t + 2, 0, ring[0], ring[2]);
-        tile(t + 3, 1, ring[1], ring[0]);
-        tile(t + 4, 0, ring[2], ring[1]);
-        tile(t + 5, 1, ring[0], ring[2]);
-    }
-    if (t < g_tiles) tile(t, 0, ring[1], ring[0]);
-    if (t + 1 < g_tiles) tile(t + 1, 1, ring[2], ring[1]);
-    if (t + 2 < g_tiles) tile(t + 2, 0, ring[0], ring[2]);
-    if (t + 3 < g_tiles) tile(t + 3, 1, ring[1], ring[0]);
-    if (t + 4 < g_tiles) tile(t + 4, 0, ring[2], ring[1]);
-
-    // The two groups hold partial sums of the same 256 x 128 outputs.  Group g keeps row tile g of
-    // each of its waves' two and gets the other group's sums for it through the LDS: wave (g, w4)
-    // leaves row tile 1 - g in slot (g, w4), 16 KB of the tables' space, and adds slot (1 - g, w4).
-    {
-        int *slot_w = reinterpret_cast<int *>(smem_raw) + (grp * 4 + w4) * 4096 + lane;
-        const int *slot_r = reinterpret_cast<const int *>(smem_raw) + ((1 - grp) * 4 + w4) * 4096 + lane;
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) slot_w[(j * 16 + e) * 64] = grp == 0 ? acc[1][j][e] : acc[0][j][e];
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int v = slot_r[(j * 16 + e) * 64];
-                if (grp == 0) acc[0][j][e] += v;
-                else acc[1][j][e] += v;
-            }
-    }
-
-    // D layout of 32x32: element e of lane: row (n) = 8 * (e / 4) + 4 * (lane / 32) + e % 4, column (m) = lane % 32
-    const bool n_vec = (N & 3) == 0;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int m = m0 + j * 32 + l32;
-        if (m >= M) continue;
-#pragma unroll
-        for (int e4 = 0; e4 < 4; e4++) {
-            const int n = n0 + w4 * 64 + grp * 32 + 8 * e4 + 4 * kq;
-            int32_t *dst = out + (int64_t)m * N + n;
-            i4_t v;
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = grp == 0 ? acc[0][j][4 * e4 + e] : acc[1][j][4 * e4 + e];
-            if (n_vec && n + 3 < N) {
-                *reinterpret_cast<i4_t *>(dst) = v;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (n + e < N) dst[e] = v[e];
-            }
-        }
-    }
-}
-
-__global__ void zero_i32_kernel(int32_t *y, int64_t n)
-{
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
-        y[i] = 0;
-}
-
-// ------------------------------------------------------------------ offline repack for the streaming kernel
-// packed[((tile * n_steps + step) * 64 + lane) * 8 + e] = codes[16 tile + lane % 16][32 step + 8 (lane / 16) + e]
-// (16-bit units; rows past N are zeros).  One thread moves one 16-byte piece.
-__global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ codes, u4_t *__restrict__ packed,
-                                                   int64_t N, int64_t K, int64_t pieces)
-{
-    const int64_t n_steps = K >> 8, kc = K >> 3;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < pieces; i += (int64_t)gridDim.x * 256) {
-        const int64_t lane = i & 63, chunk = i >> 6;
-        const int64_t step = chunk % n_steps, tile = chunk / n_steps;
-        const int64_t n = tile * 16 + (lane & 15);
-        u4_t v = u4_t{0u, 0u, 0u, 0u};
-        if (n < N) v = *reinterpret_cast<const u4_t *>(codes + n * kc + step * 32 + (lane >> 4) * 8);
-        packed[i] = v;
-    }
-}
-
-// ------------------------------------------------------------------ plain read of a code matrix
-// What the memory system gives a kernel that only reads: the batch-1 kernels' launch shape (one
-// workgroup of 16 waves per compute unit over contiguous ranges of 16-row tiles, a wave's load 16
-// rows x 64 bytes, the waves of a workgroup dealing out the 256-wide k steps) with two loads in flight
-// per wave and an exclusive or in place of the decode.  The yardstick the benchmark prints beside the
-// batch-1 kernels; `sink` is written only if the bytes happen to cancel (never for random codes),
-// which keeps the loads alive.
-__global__ __launch_bounds__(1024) void read_probe_kernel(const uint16_t *__restrict__ codes, uint32_t *__restrict__ sink,
-                                                          int N, int K, int tiles_q, int tiles_r)
-{
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, q = lane >> 4;
-    const int n_steps = K >> 8, row_bytes = K >> 2;
-    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
-    const int t1 = t0 + tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
-    const __amdgpu_buffer_rsrc_t crsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(codes), 0, (int)((int64_t)N * row_bytes), 0x00020000);
-    const int voff = c16 * row_bytes + q * 16;
-    u4_t acc = u4_t{0u, 0u, 0u, 0u};
-    for (int tile = t0; tile < t1; tile++)
-        for (int step = wave; step < n_steps; step += 32) {
-            const u4_t a = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, tile * 16 * row_bytes + step * 64, 0);
-            const u4_t b = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, step + 16 < n_steps ? tile * 16 * row_bytes + (step + 16) * 64 : (int)0x80000000, 0);
-            acc ^= a ^ b;
-        }
-    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9E3779B9u && N < 0) sink[0] = acc[0];
-}
-
-// ------------------------------------------------------------------ scratch memory of the library
-// The one buffer the library owns: split-K partial sums for dmm_decode_matmul_noalloc_f16, whose
-// callers cannot allocate.  In host code the array's name is a stand-in, not a device address;
-// dmm_init asks the runtime for the address once per device and the launches pass that.
-constexpr int64_t kScratchBytes = 16ll << 20;
-static __device__ __align__(256) unsigned char scratch[kScratchBytes];
-
-// ------------------------------------------------------------------ host side
-thread_local hipEvent_t tls_start = nullptr;
-thread_local hipEvent_t tls_stop = nullptr;
-
-template <typename T>
-struct same_type { typedef T type; };
-
-// Enqueue one kernel; the status is what the launch call itself returns (no look at the
-// thread's last-error state, which may hold somebody else's stale error).  kFirst / kLast:
-// whether this launch opens / closes the span the timing events bracket (an operator call
-// that takes two kernels records start before the first and stop after the second).
-template <bool kFirst = true, bool kLast = true, typename... KArgs>
-int launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStream_t stream,
-           typename same_type<KArgs>::type... args)
-{
-    void *argv[] = {(void *)&args...};
-    if (tls_start && tls_stop)
-        return (int)hipExtLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream,
-                                       kFirst ? tls_start : nullptr, kLast ? tls_stop : nullptr, 0);
-    return (int)hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream);
-}
-
-inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
-
-// ---- per-device state, set up by dmm_init --------------------------------------------------
-constexpr int kMaxDevices = 64;
-constexpr int kLdsMax = 160 * 1024;
-
-struct DeviceState {
-    std::atomic<int> ready{0};
-    int cus = 256;
-    void *scratch = nullptr;   // this device's copy of `scratch`
-};
-DeviceState g_dev[kMaxDevices];
-std::mutex g_init_mutex;
-
-// Every kernel that needs more dynamic LDS than the default limit, or whose table addressing
-// assumes that its dynamic LDS starts at LDS address 0 (true exactly when the kernel has no
-// static LDS, which dmm_init verifies from the function's attributes).
-struct KernelInfo {
-    const void *fn;
-    int dynamic_lds;   // bytes to allow; 0 = default limit is enough
-    bool lds_base0;
-};
-
-template <typename... KArgs>
-KernelInfo kinfo(void (*k)(KArgs...), int lds, bool base0) { return KernelInfo{reinterpret_cast<const void *>(k), lds, base0}; }
-
-const std::vector<KernelInfo> &kernel_table()
-{
-    static const std::vector<KernelInfo> t = {
-#define DMM_BOTH_LAYOUTS(X) X(false), X(true)
-#define DMM_K_STREAM(P) kinfo(gemv_stream_kernel<1, 16, 2, P, 4>, kLdsMax, true), kinfo(gemv_stream_kernel<1, 16, 2, P, 1>, kLdsMax, true)
-        DMM_BOTH_LAYOUTS(DMM_K_STREAM),
-#define DMM_K_Q8(P) kinfo(gemv_q8_kernel<1, 16, 2, P>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P>, kLdsMax, true), kinfo(gemv_q8c_kernel<3, 1, P>, kLdsMax, true)
-        DMM_BOTH_LAYOUTS(DMM_K_Q8),
-#define DMM_K_REGX(P)                                                                                        \
-    kinfo(gemv_regx_kernel<1, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 1, 2, P>, kLdsMax, true),     \
-        kinfo(gemv_regx_kernel<3, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 1, 2, P>, kLdsMax, true), \
-        kinfo(gemv_regx_kernel<1, 8, 2, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, 2, P>, kLdsMax, true)
-        DMM_BOTH_LAYOUTS(DMM_K_REGX),
-#define DMM_K_GREG(P)                                                                                        \
-    kinfo(gemm_reg_kernel<1, false, P>, gr_smem_bytes(1), true), kinfo(gemm_reg_kernel<2, false, P>, gr_smem_bytes(2), true), \
-        kinfo(gemm_reg_kernel<4, false, P>, gr_smem_bytes(4), true), kinfo(gemm_reg_kernel<1, true, P>, gr_smem_bytes(1), true), \
-        kinfo(gemm_reg_kernel<2, true, P>, gr_smem_bytes(2), true), kinfo(gemm_reg_kernel<4, true, P>, gr_smem_bytes(4), true)
-        DMM_BOTH_LAYOUTS(DMM_K_GREG),
-        kinfo(gemm_kernel<4, 2, 2, 2>, (int)sizeof(GemmCfg<4, 2, 2, 2>::Shared), false),
-#define DMM_K_I8X(T)                                                                                         \
-    kinfo(int8x_kernel<1, 8, 2, T>, kLdsMax, true), kinfo(int8x_kernel<2, 8, 2, T>, kLdsMax, true),                    \
-        kinfo(int8x_kernel<3, 8, 2, T>, kLdsMax, true), kinfo(int8x_kernel<4, 8, 2, T>, kLdsMax, true),                \
-        kinfo(int8g_kernel<T>, kI8gSmem, true)
-        DMM_BOTH_LAYOUTS(DMM_K_I8X),
-#undef DMM_K_I8X
-#undef DMM_K_GREG
-#undef DMM_K_REGX
-#undef DMM_K_Q8
-#undef DMM_K_STREAM
-#undef DMM_BOTH_LAYOUTS
-    };
-    return t;
-}
-
-// One-time set-up of a device (the current one must be `dev`): compute-unit count, dynamic-LDS
-// limits, the check that the table kernels have no static LDS, and the address of `scratch`.
-int init_current_device(int dev)
-{
-    DeviceState &ds = g_dev[dev];
-    if (ds.ready.load(std::memory_order_acquire)) return DMM_OK;
-    std::lock_guard<std::mutex> lock(g_init_mutex);
-    if (ds.ready.load(std::memory_order_acquire)) return DMM_OK;
-    int v = 0;
-    hipError_t e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return (int)e;
-    ds.cus = v > 0 ? v : 256;
-    for (const KernelInfo &k : kernel_table()) {
-        if (k.lds_base0) {
-            hipFuncAttributes attr;
-            e = hipFuncGetAttributes(&attr, k.fn);
-            if (e != hipSuccess) return (int)e;
-            if (attr.sharedSizeBytes != 0) return DMM_ERR_INTERNAL;
-        }
-        if (k.dynamic_lds > 0) {
-            e = hipFuncSetAttribute(k.fn, hipFuncAttributeMaxDynamicSharedMemorySize, k.dynamic_lds);
-            if (e != hipSuccess) return (int)e;
-        }
-    }
-    void *p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess) return (int)e;
-    ds.scratch = p;
-    ds.ready.store(1, std::memory_order_release);
-    return DMM_OK;
-}
-
-// Called by every entry point that launches, after its argument checks.  A first call on a
-// device does the set-up unless the stream is being captured into a graph, where host-side
-// set-up has no business: such a caller runs dmm_init beforehand.
-int ensure_ready(hipStream_t stream, const DeviceState **out = nullptr)
-{
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
-    if (dev < 0 || dev >= kMaxDevices) return DMM_ERR_TOO_LARGE;
-    if (!g_dev[dev].ready.load(std::memory_order_acquire)) {
-        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-        if (stream && hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
-            return DMM_ERR_NOT_INITIALIZED;
-        if (int st = init_current_device(dev)) return st;
-    }
-    if (out) *out = &g_dev[dev];
-    return DMM_OK;
-}
-
-// compute units of the current device (after ensure_ready)
-int cu_count()
-{
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-    return g_dev[dev].cus;
-}
-
-int check_common(const void *x, const void *codes, const void *grid, const void *y, int64_t M,
-                 int64_t N, int64_t K)
-{
-    if (M < 0 || N < 0 || K < 0 || (K & 7)) return DMM_ERR_BAD_SHAPE;
-    if (M == 0 || N == 0) return DMM_OK;   // nothing to write; pointers may be NULL
-    if (!y || !grid) return DMM_ERR_NULL_POINTER;
-    if (K > 0 && (!x || !codes)) return DMM_ERR_NULL_POINTER;
-    if (!aligned(x, 2) || !aligned(codes, 2) || !aligned(grid, 2) || !aligned(y, 2)) return DMM_ERR_MISALIGNED;
-    if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return DMM_ERR_TOO_LARGE;
-    return DMM_OK;
-}
-
-bool gemv_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
-             int64_t K)
-{
-    return M >= 1 && M <= 32 && K >= 256 && (K & 255) == 0 && K <= (1 << 23) && N * (K >> 2) < (1LL << 31) &&
-           (N & 3) == 0 && aligned(x, 16) &&
-           aligned(codes, 16) && aligned(grid, 16) && aligned(y, 8);
-}
-
-bool gemm_ok(const void *x, const void *codes, const void *grid, const void *, int64_t M, int64_t N,
-             int64_t K)
-{
-    return M >= 1 && N >= 1 && K >= 64 && (K & 63) == 0 && aligned(x, 16) && aligned(codes, 16) &&
-           aligned(grid, 16) && M <= 65535LL * 128;
-}
-
-template <int R, int W, int D, bool kPacked = false>
-int launch_gemv_stream(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                       int64_t N, int64_t K, hipStream_t stream)
-{
-    const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)stream_x_bytes(M, K);
-    const int64_t n_tiles = (N + 15) / 16;
-    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    if (M <= 4)   // four pieces of x per LDS read
-        return launch(gemv_stream_kernel<R, W, D, kPacked, 4>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
-                      (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N,
-                      (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
-    return launch(gemv_stream_kernel<R, W, D, kPacked, 1>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
-                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
-                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
-}
-
-// tables, partial sums and x fit in the 160 KB of LDS, and every byte offset of the code
-// matrix fits the 31 bits the buffer addressing is used with
-template <int R, int W>
-bool gemv_q8_ok(int64_t M, int64_t N, int64_t K)
-{
-    return M <= 4 && (int64_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + q8_x_bytes(M, K) <= kLdsMax &&
-           N * (K >> 2) < (1LL << 31);
-}
-
-template <int R, int W, int D, bool kPacked = false>
-int launch_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                   int64_t N, int64_t K, hipStream_t stream)
-{
-    // the 8-bit layout is the larger one, so the 16-bit kernel it may hand over to fits as well
-    const size_t shmem = (size_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
-    const int64_t n_tiles = (N + 15) / 16;
-    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_q8_kernel<R, W, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
-                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
-                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
-}
-
-// the chunked 8-bit kernel: one row of x of any length the 16-bit kernel could take over (its x in LDS)
-bool gemv_q8c_ok(int64_t M, int64_t N, int64_t K)
-{
-    return M == 1 && (int64_t)kSTablesBytes + stream_red_bytes(1, 16, 1) + stream_x_bytes(1, K) <= kLdsMax &&
-           N * (K >> 2) < (1LL << 31);
-}
-
-// groups of up to three tiles, one code load per tile in flight per wave (four tiles per group spill
-// registers; two chunks in flight per wave were no faster)
-template <bool kPacked>
-int launch_gemv_q8c(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t N, int64_t K,
-                    hipStream_t stream)
-{
-    constexpr int T = 3;
-    size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(1, 16, 1) + (size_t)stream_x_bytes(1, K);   // the 16-bit hand-over
-    if (shmem < (size_t)qc_lds_bytes(T)) shmem = qc_lds_bytes(T);
-    const int64_t n_tiles = (N + 15) / 16;
-    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_q8c_kernel<T, 1, kPacked>, dim3((unsigned)wgs), dim3(1024), shmem, stream, (const uint16_t *)x,
-                  (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)N, (int)K, (int)(n_tiles / wgs),
-                  (int)(n_tiles % wgs));
-}
-
-template <int R, int W>
-bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
-{
-    return M <= 16 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + stream_x_bytes(M, K) <= kLdsMax &&
-           N * (K >> 2) < (1LL << 31);
-}
-
-template <int R, int W, int MT, int D, bool kPacked = false>
-int launch_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                     int64_t N, int64_t K, hipStream_t stream)
-{
-    const size_t shmem = (size_t)kSTablesBytes + 2 * W * R * MT * kWave * 16;
-    const int64_t n_tiles = (N + 15) / 16;
-    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_regx_kernel<R, W, MT, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
-                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
-                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
-}
-
-// Whether the operator may pick the 8-bit kernel: dmm_set_gemv_8bit, or DMM_GEMV_8BIT=0 in the
-// environment (read once, at the first call that needs it) for hosts that cannot call it.
-std::atomic<int> g_gemv_q8{-1};
-
-inline bool gemv_q8_enabled()
-{
-    int on = g_gemv_q8.load(std::memory_order_relaxed);
-    if (on < 0) {
-        const char *e = getenv("DMM_GEMV_8BIT");
-        on = (e && e[0] == '0') ? 0 : 1;
-        int expected = -1;
-        if (!g_gemv_q8.compare_exchange_strong(expected, on)) on = expected;   // a setter came first
-    }
-    return on == 1;
-}
-
-// The 8-bit kernels.  One row of x: the chunked kernel.  Two to four rows: one row tile at a time, the
-// code stream three loads deep per wave when a workgroup has more than two row tiles to walk
-// through, two deep for shorter launches (where a larger first burst only delays the first tile).
-template <bool kPacked>
-int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                int64_t N, int64_t K, hipStream_t stream)
-{
-    if (M == 1) return launch_gemv_q8c<kPacked>(x, codes, grid, scale, y, N, K, stream);
-    const int64_t n_tiles = (N + 15) / 16;
-    if (n_tiles > 2 * cu_count()) return launch_gemv_q8<1, 16, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    return launch_gemv_q8<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-}
-
-// whether an 8-bit kernel can take the shape at all (grid and x permitting, which the kernel finds out)
-bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok(M, N, K) : gemv_q8_ok<1, 16>(M, N, K); }
-
-// The choice among the matrix-vector kernels.  The 8-bit kernels where they apply and pay: one row of x
-// from more than two row tiles per workgroup on, and at exactly two for long x (measured as launches of
-// one HIP graph on rotating code buffers, the two kernels taking turns, 8-bit against 16-bit kernel, us
-// per launch: 8192 -> 10240 7.9 / 8.7, 8192 -> 9216 7.9 / 8.7, 8192 -> 28672 15.3 / 16.6, 4096 -> 22016
-// 8.7 / 10.9; two tiles: 28672 -> 8192 15.5 / 16.2, 16384 -> 8192 10.4 / 10.6, 12288 -> 8192 8.5 / 8.6,
-// 8192 -> 8192 7.0 / 7.0, 4096 -> 8192 5.3 / 5.3, 5120 -> 8192 6.2 / 5.7; below two tiles the 16-bit
-// kernel wins, 5120 -> 5120 6.2 / 5.6, 11008 -> 4096 6.9 / 5.5, its prologue being the cheaper one), two
-// to four rows from more than three tiles on.  A grid that does not fit fp8 costs them a second table
-// build, and the 16-bit kernel's y is the correctly rounded one.  Otherwise the 16-bit streaming
-// kernel, one tile at a time; the register-x kernel when x does not fit the LDS.
-enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
-
-GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
-{
-    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const bool long_launch = M == 1 ? n_tiles > 2 * cus || (n_tiles == 2 * cus && K >= 12288) : n_tiles > 3 * cus;
-    if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
-    if (gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
-    return kGemvRegx;
-}
-
-// The register-x kernel for M <= 16 reads the x slice of a k step once per row block, so the row
-// block should be the workgroup's whole share of tiles when that is 1 .. 4 tiles, and otherwise
-// the size that needs the fewest blocks.
-template <bool kPacked>
-int run_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                  int64_t N, int64_t K, hipStream_t stream)
-{
-    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
-    int best = 1;
-    for (int r = 2; r <= 4; r++)
-        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
-    switch (best) {
-        case 1: return launch_gemv_regx<1, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        case 2: return launch_gemv_regx<2, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        case 3: return launch_gemv_regx<3, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        default: return launch_gemv_regx<4, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    }
-}
-
-// M = 17 .. 32: two x tiles per wave leave registers for one or two row tiles (three spill)
-template <bool kPacked>
-int run_gemv_regx2(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                   int64_t N, int64_t K, hipStream_t stream)
-{
-    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;
-    if (share == 1) return launch_gemv_regx<1, 8, 2, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    return launch_gemv_regx<2, 8, 2, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-}
-
-template <bool kPacked>
-int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-             int64_t N, int64_t K, hipStream_t stream)
-{
-    if (M > 16) return run_gemv_regx2<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    switch (pick_gemv(M, N, K)) {
-        case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        default: return run_gemv_regx<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    }
-}
-
-template <int TM, bool kSplit, bool kPacked>
-int launch_gemm_reg_tm(const void *x, const void *codes, const void *grid, float scale, void *y, float *part,
-                       int64_t M, int64_t N, int64_t K, int splits, hipStream_t stream)
-{
-    dim3 g((unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)((N + kGrBN - 1) / kGrBN), (unsigned)splits);
-    return launch<true, !kSplit>(gemm_reg_kernel<TM, kSplit, kPacked>, g, dim3(256), gr_smem_bytes(TM), stream,
-                                 (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, part, (int)M,
-                                 (int)N, (int)K, splits, aligned(y, 8) ? 1 : 0);
-}
-
-// rows of x per block: 32, 64 or 128
-inline int gemm_reg_tm(int64_t M) { return M <= 32 ? 1 : M <= 64 ? 2 : 4; }
-
-template <bool kPacked = false>
-int launch_gemm_reg(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                    int64_t N, int64_t K, hipStream_t stream)
-{
-    switch (gemm_reg_tm(M)) {
-        case 1: return launch_gemm_reg_tm<1, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
-        case 2: return launch_gemm_reg_tm<2, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
-        default: return launch_gemm_reg_tm<4, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
-    }
-}
-
-// How many ways to split K so that the blocks about fill the chip: as many as fit the CU count
-// without starting a second round, each with at least 4 k tiles, and no more than the
-// workspace holds partial sums for.  1 = no split.
-int splitk_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, int cus)
-{
-    const int tm = gemm_reg_tm(M);
-    const int64_t tiles = ((M + 32 * tm - 1) / (32 * tm)) * ((N + kGrBN - 1) / kGrBN);
-    int64_t splits = cus / tiles;
-    const int64_t k_tiles = K / kGrBK;
-    if (splits > k_tiles / 4) splits = k_tiles / 4;
-    if (splits > 64) splits = 64;
-    const int64_t per_split = M * N * 4;
-    if (per_split > 0 && splits * per_split > workspace_bytes) splits = workspace_bytes / per_split;
-    return splits < 2 ? 1 : (int)splits;
-}
-
-template <bool kPacked = false>
-int launch_gemm_splitk(const void *x, const void *codes, const void *grid, float scale, void *y, void *workspace,
-                       int splits, int64_t M, int64_t N, int64_t K, hipStream_t stream)
-{
-    float *part = reinterpret_cast<float *>(workspace);
-    int st;
-    switch (gemm_reg_tm(M)) {
-        case 1: st = launch_gemm_reg_tm<1, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
-        case 2: st = launch_gemm_reg_tm<2, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
-        default: st = launch_gemm_reg_tm<4, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
-    }
-    if (st != 0) return st;
-    const int64_t mn = M * N;
-    const int64_t blocks = (mn + 1023) / 1024;
-    return launch<false, true>(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const float *)part,
-                               (uint16_t *)y, mn, splits, scale);
-}
-
-// the register-operand kernel addresses codes and x through 31-bit buffer offsets
-bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
-{
-    return N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31) && N <= 65535LL * kGrBN;
-}
-
-// Smallest M that takes the split-K path when a workspace is given (up to M = 16 the
-// matrix-vector kernels are as fast or faster).
-constexpr int kSplitKMinM = 17;
-
-bool splitk_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
-               int64_t K)
-{
-    return M >= kSplitKMinM && gemm_ok(x, codes, grid, y, M, N, K) && gemm_reg_ok(M, N, K) && aligned(y, 8);
-}
-
-// The register-operand kernel where its offsets fit, else the LDS-staged one (256 x 128, 8 waves)
-int run_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-             int64_t N, int64_t K, hipStream_t stream)
-{
-    if (gemm_reg_ok(M, N, K)) return launch_gemm_reg(x, codes, grid, scale, y, M, N, K, stream);
-    typedef GemmCfg<4, 2, 2, 2> C;
-    dim3 g((unsigned)((N + C::kBN - 1) / C::kBN), (unsigned)((M + C::kBM - 1) / C::kBM));
-    return launch(gemm_kernel<4, 2, 2, 2>, g, dim3(C::kThreads), sizeof(typename C::Shared), stream,
-                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
-                  aligned(y, 8) ? 1 : 0);
-}
-
-// y = 0 when K == 0 (empty sum), any M, N.
-__global__ void zero_kernel(uint16_t *y, int64_t n)
-{
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
-        y[i] = 0;
-}
-
-int run_generic(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                int64_t N, int64_t K, hipStream_t stream)
-{
-    if (K == 0) {
-        int64_t n = M * N;
-        unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
-        return launch(zero_kernel, dim3(blocks), dim3(256), 0, stream, (uint16_t *)y, n);
-    }
-    int64_t blocks = (N + 3) / 4;
-    if (blocks > 65535 * 16) blocks = 65535 * 16;
-    return launch(generic_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t *)x,
-                  (const uint16_t *)codes, grid, scale, (uint16_t *)y, M, N, K);
-}
-
-template <int R, bool kTiled, bool kFirst, bool kLast>
-int launch_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
-                 hipStream_t stream)
-{
-    constexpr int W = 8, D = 2;
-    const size_t shmem = (size_t)2 * kI8TableBytes + (R <= 2 ? 2 : 1) * W * R * kWave * 16;
-    const int64_t n_tiles = (N + 15) / 16;
-    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch<kFirst, kLast>(int8x_kernel<R, W, D, kTiled>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
-                                 (const int8_t *)x, (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M,
-                                 (int)N, (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
-}
-
-// Which kernel the integer operator takes for 16-byte aligned buffers.  Many rows of x: the
-// matrix-matrix kernel costs about K * 11.5 ns per round of one 256 x 128 tile per CU (47 us at
-// K = 4096) however few of its tiles exist, the matrix-vector kernel about 3 us plus its code
-// bytes at 3.5 TB/s per 16 rows of x; the cheaper estimate wins (M = 64 at 4096 x 4096: four
-// matrix-vector launches, 20 us; M = 256: one matrix-matrix launch, 47 us against 75).
-enum Int8Kind { kInt8Scalar, kInt8Gemv, kInt8Gemm };
-Int8Kind pick_int8(int64_t M, int64_t N, int64_t K, int cus)
-{
-    if (M < 1 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31) || K > (1 << 17))
-        return kInt8Scalar;
-    if (M > 16 && M * K < (1LL << 31)) {
-        const int64_t tiles = ((M + kI8gBM - 1) / kI8gBM) * ((N + kI8gBN - 1) / kI8gBN);
-        const double t_gemm = 3.0 + (double)((tiles + cus - 1) / cus) * (double)K * 0.0115;
-        const double t_gemv = (double)((M + 15) / 16) * (3.0 + (double)N * (double)(K >> 2) / 3.5e6);
-        if (t_gemm < t_gemv) return kInt8Gemm;
-    }
-    return kInt8Gemv;
-}
-
-template <bool kTiled>
-int launch_int8g(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
-                 hipStream_t stream)
-{
-    dim3 g((unsigned)((M + kI8gBM - 1) / kI8gBM), (unsigned)((N + kI8gBN - 1) / kI8gBN));
-    return launch(int8g_kernel<kTiled>, g, dim3(512), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
-                  (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
-}
-
-// one launch for up to 16 rows of x; first / last: position in the operator call's sequence of
-// launches, for the timing events
-template <bool kTiled>
-int run_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
-              bool first, bool last, hipStream_t stream)
-{
-    // row block = the workgroup's share of tiles when that is one to four, else the size that needs
-    // the fewest blocks (x is fetched once per row block), as for the half-precision kernel
-    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;
-    int best = 1;
-    for (int r = 2; r <= 4; r++)
-        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
-#define DMM_I8X(RR)                                                                                         \
-    (first ? (last ? launch_int8x<RR, kTiled, true, true>(x, codes, cb, out, M, N, K, stream)               \
-                   : launch_int8x<RR, kTiled, true, false>(x, codes, cb, out, M, N, K, stream))              \
-           : (last ? launch_int8x<RR, kTiled, false, true>(x, codes, cb, out, M, N, K, stream)              \
-                   : launch_int8x<RR, kTiled, false, false>(x, codes, cb, out, M, N, K, stream)))
-    return best == 1 ? DMM_I8X(1) : best == 2 ? DMM_I8X(2) : best == 3 ? DMM_I8X(3) : DMM_I8X(4);
-#undef DMM_I8X
-}
-
-// CU count for the pure queries (kernel names, workspace size), which must answer without a
-// device: the current device's if it has been set up, else the MI355X's 256
-int cu_count_or_default()
-{
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-    return g_dev[dev].ready.load(std::memory_order_acquire) ? g_dev[dev].cus : 256;
-}
-
-// the operator's dispatch once the arguments are checked and the device is ready
-int dispatch_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M, int64_t N,
-                 int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t s)
-{
-    if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K)) {
-        const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
-        if (splits >= 2) return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, s);
-    }
-    if (gemv_ok(x, codes, grid, y, M, N, K)) return run_gemv<false>(x, codes, grid, scale, y, M, N, K, s);
-    if (gemm_ok(x, codes, grid, y, M, N, K)) return run_gemm(x, codes, grid, scale, y, M, N, K, s);
-    return run_generic(x, codes, grid, scale, y, M, N, K, s);
-}
-
-// ------------------------------------------------------------------ the operator on host memory
-// The reference's own CPU path is a scalar decode and a triple loop (/root/reference/test_decode_matmul.py:29-71);
-// this is the same thing for the half-precision form, in plain C++ for tensors that live in host
-// memory: no GPU is involved and no GPU call is made.  Not a fallback: device pointers never come
-// here, the entry points below are separate ones.  One rounding per weight (the fp32 sum of a half
-// and +-1/4 is exact), fp32 sums over k in ascending order, rows of W spread over host threads.
-inline void host_decode_row(const uint16_t *codes, const half_t *grid, int64_t kc, half_t *w)
-{
-    for (int64_t j = 0; j < kc; j++) {
-        const uint32_t c = codes[j];
-        const uint32_t idx = c & 0xFFu, s7 = (c >> 8) & 0x7Fu;
-        const uint32_t s8 = s7 | ((uint32_t)(__builtin_popcount(s7) & 1) << 7);
-        const float shift = (c & 0x8000u) ? -0.25f : 0.25f;
-        for (int d = 0; d < 8; d++) {
-            const float g = (float)grid[idx * 8 + d];
-            w[j * 8 + d] = (half_t)(((s8 >> d) & 1u ? -g : g) + shift);
-        }
-    }
-}
-
-template <typename F>
-void host_parallel_rows(int64_t n_rows, int64_t work_per_row, F body)
-{
-    unsigned threads = std::thread::hardware_concurrency();
-    if (threads == 0) threads = 1;
-    if (threads > 16) threads = 16;
-    if (n_rows * work_per_row < (1 << 20) || n_rows < 2) threads = 1;
-    if ((int64_t)threads > n_rows) threads = (unsigned)n_rows;
-    if (threads == 1) {
-        body(0, n_rows);
-        return;
-    }
-    std::vector<std::thread> pool;
-    for (unsigned t = 0; t < threads; t++)
-        pool.emplace_back([=] { body(n_rows * t / threads, n_rows * (t + 1) / threads); });
-    for (auto &th : pool) th.join();
-}
+#include "dmm_tables.h"
+#include "dmm_gemv_f16.h"
+#include "dmm_gemv_q8.h"
+#include "dmm_gemv_small.h"
+#include "dmm_gemm.h"
+#include "dmm_int8.h"
+#include "dmm_aux.h"
+#include "dmm_host.h"
 
 }  // namespace dmm
 

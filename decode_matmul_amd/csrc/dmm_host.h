@@ -1,0 +1,585 @@
+// The library scratch memory and the host side: launch plumbing, per-device set-up, argument
+// checks, dispatch and the operator on host memory.
+// Part of libdmm: included by dmm.hip inside namespace dmm, in this order; not a
+// translation unit of its own.
+
+// ------------------------------------------------------------------ scratch memory of the library
+// The one buffer the library owns: split-K partial sums for dmm_decode_matmul_noalloc_f16, whose
+// callers cannot allocate.  In host code the array's name is a stand-in, not a device address;
+// dmm_init asks the runtime for the address once per device and the launches pass that.
+constexpr int64_t kScratchBytes = 16ll << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+// ------------------------------------------------------------------ host side
+thread_local hipEvent_t tls_start = nullptr;
+thread_local hipEvent_t tls_stop = nullptr;
+
+template <typename T>
+struct same_type { typedef T type; };
+
+// Enqueue one kernel; the status is what the launch call itself returns (no look at the
+// thread's last-error state, which may hold somebody else's stale error).  kFirst / kLast:
+// whether this launch opens / closes the span the timing events bracket (an operator call
+// that takes two kernels records start before the first and stop after the second).
+template <bool kFirst = true, bool kLast = true, typename... KArgs>
+int launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStream_t stream,
+           typename same_type<KArgs>::type... args)
+{
+    void *argv[] = {(void *)&args...};
+    if (tls_start && tls_stop)
+        return (int)hipExtLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream,
+                                       kFirst ? tls_start : nullptr, kLast ? tls_stop : nullptr, 0);
+    return (int)hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream);
+}
+
+inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---- per-device state, set up by dmm_init --------------------------------------------------
+constexpr int kMaxDevices = 64;
+constexpr int kLdsMax = 160 * 1024;
+
+struct DeviceState {
+    std::atomic<int> ready{0};
+    int cus = 256;
+    void *scratch = nullptr;   // this device's copy of `scratch`
+};
+DeviceState g_dev[kMaxDevices];
+std::mutex g_init_mutex;
+
+// Every kernel that needs more dynamic LDS than the default limit, or whose table addressing
+// assumes that its dynamic LDS starts at LDS address 0 (true exactly when the kernel has no
+// static LDS, which dmm_init verifies from the function's attributes).
+struct KernelInfo {
+    const void *fn;
+    int dynamic_lds;   // bytes to allow; 0 = default limit is enough
+    bool lds_base0;
+};
+
+template <typename... KArgs>
+KernelInfo kinfo(void (*k)(KArgs...), int lds, bool base0) { return KernelInfo{reinterpret_cast<const void *>(k), lds, base0}; }
+
+const std::vector<KernelInfo> &kernel_table()
+{
+    static const std::vector<KernelInfo> t = {
+#define DMM_BOTH_LAYOUTS(X) X(false), X(true)
+#define DMM_K_STREAM(P) kinfo(gemv_stream_kernel<1, 16, 2, P, 4>, kLdsMax, true), kinfo(gemv_stream_kernel<1, 16, 2, P, 1>, kLdsMax, true)
+        DMM_BOTH_LAYOUTS(DMM_K_STREAM),
+#define DMM_K_Q8(P) kinfo(gemv_q8_kernel<1, 16, 2, P>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P>, kLdsMax, true), kinfo(gemv_q8c_kernel<3, 1, P>, kLdsMax, true)
+        DMM_BOTH_LAYOUTS(DMM_K_Q8),
+#define DMM_K_REGX(P)                                                                                        \
+    kinfo(gemv_regx_kernel<1, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 1, 2, P>, kLdsMax, true),     \
+        kinfo(gemv_regx_kernel<3, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 1, 2, P>, kLdsMax, true), \
+        kinfo(gemv_regx_kernel<1, 8, 2, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, 2, P>, kLdsMax, true)
+        DMM_BOTH_LAYOUTS(DMM_K_REGX),
+#define DMM_K_GREG(P)                                                                                        \
+    kinfo(gemm_reg_kernel<1, false, P>, gr_smem_bytes(1), true), kinfo(gemm_reg_kernel<2, false, P>, gr_smem_bytes(2), true), \
+        kinfo(gemm_reg_kernel<4, false, P>, gr_smem_bytes(4), true), kinfo(gemm_reg_kernel<1, true, P>, gr_smem_bytes(1), true), \
+        kinfo(gemm_reg_kernel<2, true, P>, gr_smem_bytes(2), true), kinfo(gemm_reg_kernel<4, true, P>, gr_smem_bytes(4), true)
+        DMM_BOTH_LAYOUTS(DMM_K_GREG),
+        kinfo(gemm_kernel<4, 2, 2, 2>, (int)sizeof(GemmCfg<4, 2, 2, 2>::Shared), false),
+#define DMM_K_I8X(T)                                                                                         \
+    kinfo(int8x_kernel<1, 8, 2, T>, kLdsMax, true), kinfo(int8x_kernel<2, 8, 2, T>, kLdsMax, true),                    \
+        kinfo(int8x_kernel<3, 8, 2, T>, kLdsMax, true), kinfo(int8x_kernel<4, 8, 2, T>, kLdsMax, true),                \
+        kinfo(int8g_kernel<T>, kI8gSmem, true)
+        DMM_BOTH_LAYOUTS(DMM_K_I8X),
+#undef DMM_K_I8X
+#undef DMM_K_GREG
+#undef DMM_K_REGX
+#undef DMM_K_Q8
+#undef DMM_K_STREAM
+#undef DMM_BOTH_LAYOUTS
+    };
+    return t;
+}
+
+// One-time set-up of a device (the current one must be `dev`): compute-unit count, dynamic-LDS
+// limits, the check that the table kernels have no static LDS, and the address of `scratch`.
+int init_current_device(int dev)
+{
+    DeviceState &ds = g_dev[dev];
+    if (ds.ready.load(std::memory_order_acquire)) return DMM_OK;
+    std::lock_guard<std::mutex> lock(g_init_mutex);
+    if (ds.ready.load(std::memory_order_acquire)) return DMM_OK;
+    int v = 0;
+    hipError_t e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return (int)e;
+    ds.cus = v > 0 ? v : 256;
+    for (const KernelInfo &k : kernel_table()) {
+        if (k.lds_base0) {
+            hipFuncAttributes attr;
+            e = hipFuncGetAttributes(&attr, k.fn);
+            if (e != hipSuccess) return (int)e;
+            if (attr.sharedSizeBytes != 0) return DMM_ERR_INTERNAL;
+        }
+        if (k.dynamic_lds > 0) {
+            e = hipFuncSetAttribute(k.fn, hipFuncAttributeMaxDynamicSharedMemorySize, k.dynamic_lds);
+            if (e != hipSuccess) return (int)e;
+        }
+    }
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    ds.scratch = p;
+    ds.ready.store(1, std::memory_order_release);
+    return DMM_OK;
+}
+
+// Called by every entry point that launches, after its argument checks.  A first call on a
+// device does the set-up unless the stream is being captured into a graph, where host-side
+// set-up has no business: such a caller runs dmm_init beforehand.
+int ensure_ready(hipStream_t stream, const DeviceState **out = nullptr)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return DMM_ERR_TOO_LARGE;
+    if (!g_dev[dev].ready.load(std::memory_order_acquire)) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (stream && hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+            return DMM_ERR_NOT_INITIALIZED;
+        if (int st = init_current_device(dev)) return st;
+    }
+    if (out) *out = &g_dev[dev];
+    return DMM_OK;
+}
+
+// compute units of the current device (after ensure_ready)
+int cu_count()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    return g_dev[dev].cus;
+}
+
+int check_common(const void *x, const void *codes, const void *grid, const void *y, int64_t M,
+                 int64_t N, int64_t K)
+{
+    if (M < 0 || N < 0 || K < 0 || (K & 7)) return DMM_ERR_BAD_SHAPE;
+    if (M == 0 || N == 0) return DMM_OK;   // nothing to write; pointers may be NULL
+    if (!y || !grid) return DMM_ERR_NULL_POINTER;
+    if (K > 0 && (!x || !codes)) return DMM_ERR_NULL_POINTER;
+    if (!aligned(x, 2) || !aligned(codes, 2) || !aligned(grid, 2) || !aligned(y, 2)) return DMM_ERR_MISALIGNED;
+    if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return DMM_ERR_TOO_LARGE;
+    return DMM_OK;
+}
+
+bool gemv_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
+             int64_t K)
+{
+    return M >= 1 && M <= 32 && K >= 256 && (K & 255) == 0 && K <= (1 << 23) && N * (K >> 2) < (1LL << 31) &&
+           (N & 3) == 0 && aligned(x, 16) &&
+           aligned(codes, 16) && aligned(grid, 16) && aligned(y, 8);
+}
+
+bool gemm_ok(const void *x, const void *codes, const void *grid, const void *, int64_t M, int64_t N,
+             int64_t K)
+{
+    return M >= 1 && N >= 1 && K >= 64 && (K & 63) == 0 && aligned(x, 16) && aligned(codes, 16) &&
+           aligned(grid, 16) && M <= 65535LL * 128;
+}
+
+template <int R, int W, int D, bool kPacked = false>
+int launch_gemv_stream(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                       int64_t N, int64_t K, hipStream_t stream)
+{
+    const size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + (size_t)stream_x_bytes(M, K);
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    if (M <= 4)   // four pieces of x per LDS read
+        return launch(gemv_stream_kernel<R, W, D, kPacked, 4>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                      (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N,
+                      (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    return launch(gemv_stream_kernel<R, W, D, kPacked, 1>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+// tables, partial sums and x fit in the 160 KB of LDS, and every byte offset of the code
+// matrix fits the 31 bits the buffer addressing is used with
+template <int R, int W>
+bool gemv_q8_ok(int64_t M, int64_t N, int64_t K)
+{
+    return M <= 4 && (int64_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + q8_x_bytes(M, K) <= kLdsMax &&
+           N * (K >> 2) < (1LL << 31);
+}
+
+template <int R, int W, int D, bool kPacked = false>
+int launch_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                   int64_t N, int64_t K, hipStream_t stream)
+{
+    // the 8-bit layout is the larger one, so the 16-bit kernel it may hand over to fits as well
+    const size_t shmem = (size_t)kSTablesBytes + q8_red_bytes(R, W, (int)M) + (size_t)q8_x_bytes(M, K);
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(gemv_q8_kernel<R, W, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+// the chunked 8-bit kernel: one row of x of any length the 16-bit kernel could take over (its x in LDS)
+bool gemv_q8c_ok(int64_t M, int64_t N, int64_t K)
+{
+    return M == 1 && (int64_t)kSTablesBytes + stream_red_bytes(1, 16, 1) + stream_x_bytes(1, K) <= kLdsMax &&
+           N * (K >> 2) < (1LL << 31);
+}
+
+// groups of up to three tiles, one code load per tile in flight per wave (four tiles per group spill
+// registers; two chunks in flight per wave were no faster)
+template <bool kPacked>
+int launch_gemv_q8c(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t N, int64_t K,
+                    hipStream_t stream)
+{
+    constexpr int T = 3;
+    size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(1, 16, 1) + (size_t)stream_x_bytes(1, K);   // the 16-bit hand-over
+    if (shmem < (size_t)qc_lds_bytes(T)) shmem = qc_lds_bytes(T);
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(gemv_q8c_kernel<T, 1, kPacked>, dim3((unsigned)wgs), dim3(1024), shmem, stream, (const uint16_t *)x,
+                  (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)N, (int)K, (int)(n_tiles / wgs),
+                  (int)(n_tiles % wgs));
+}
+
+template <int R, int W>
+bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
+{
+    return M <= 16 && (int64_t)kSTablesBytes + stream_red_bytes(R, W, (int)M) + stream_x_bytes(M, K) <= kLdsMax &&
+           N * (K >> 2) < (1LL << 31);
+}
+
+template <int R, int W, int MT, int D, bool kPacked = false>
+int launch_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                     int64_t N, int64_t K, hipStream_t stream)
+{
+    const size_t shmem = (size_t)kSTablesBytes + 2 * W * R * MT * kWave * 16;
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(gemv_regx_kernel<R, W, MT, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+// Whether the operator may pick the 8-bit kernel: dmm_set_gemv_8bit, or DMM_GEMV_8BIT=0 in the
+// environment (read once, at the first call that needs it) for hosts that cannot call it.
+std::atomic<int> g_gemv_q8{-1};
+
+inline bool gemv_q8_enabled()
+{
+    int on = g_gemv_q8.load(std::memory_order_relaxed);
+    if (on < 0) {
+        const char *e = getenv("DMM_GEMV_8BIT");
+        on = (e && e[0] == '0') ? 0 : 1;
+        int expected = -1;
+        if (!g_gemv_q8.compare_exchange_strong(expected, on)) on = expected;   // a setter came first
+    }
+    return on == 1;
+}
+
+// The 8-bit kernels.  One row of x: the chunked kernel.  Two to four rows: one row tile at a time, the
+// code stream three loads deep per wave when a workgroup has more than two row tiles to walk
+// through, two deep for shorter launches (where a larger first burst only delays the first tile).
+template <bool kPacked>
+int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                int64_t N, int64_t K, hipStream_t stream)
+{
+    if (M == 1) return launch_gemv_q8c<kPacked>(x, codes, grid, scale, y, N, K, stream);
+    const int64_t n_tiles = (N + 15) / 16;
+    if (n_tiles > 2 * cu_count()) return launch_gemv_q8<1, 16, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    return launch_gemv_q8<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+}
+
+// whether an 8-bit kernel can take the shape at all (grid and x permitting, which the kernel finds out)
+bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok(M, N, K) : gemv_q8_ok<1, 16>(M, N, K); }
+
+// The choice among the matrix-vector kernels.  The 8-bit kernels where they apply and pay: one row of x
+// from more than two row tiles per workgroup on, and at exactly two for long x (measured as launches of
+// one HIP graph on rotating code buffers, the two kernels taking turns, 8-bit against 16-bit kernel, us
+// per launch: 8192 -> 10240 7.9 / 8.7, 8192 -> 9216 7.9 / 8.7, 8192 -> 28672 15.3 / 16.6, 4096 -> 22016
+// 8.7 / 10.9; two tiles: 28672 -> 8192 15.5 / 16.2, 16384 -> 8192 10.4 / 10.6, 12288 -> 8192 8.5 / 8.6,
+// 8192 -> 8192 7.0 / 7.0, 4096 -> 8192 5.3 / 5.3, 5120 -> 8192 6.2 / 5.7; below two tiles the 16-bit
+// kernel wins, 5120 -> 5120 6.2 / 5.6, 11008 -> 4096 6.9 / 5.5, its prologue being the cheaper one), two
+// to four rows from more than three tiles on.  A grid that does not fit fp8 costs them a second table
+// build, and the 16-bit kernel's y is the correctly rounded one.  Otherwise the 16-bit streaming
+// kernel, one tile at a time; the register-x kernel when x does not fit the LDS.
+enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
+
+GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
+{
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const bool long_launch = M == 1 ? n_tiles > 2 * cus || (n_tiles == 2 * cus && K >= 12288) : n_tiles > 3 * cus;
+    if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
+    if (gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
+    return kGemvRegx;
+}
+
+// The register-x kernel for M <= 16 reads the x slice of a k step once per row block, so the row
+// block should be the workgroup's whole share of tiles when that is 1 .. 4 tiles, and otherwise
+// the size that needs the fewest blocks.
+template <bool kPacked>
+int run_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                  int64_t N, int64_t K, hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
+    int best = 1;
+    for (int r = 2; r <= 4; r++)
+        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
+    switch (best) {
+        case 1: return launch_gemv_regx<1, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case 2: return launch_gemv_regx<2, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case 3: return launch_gemv_regx<3, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return launch_gemv_regx<4, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    }
+}
+
+// M = 17 .. 32: two x tiles per wave leave registers for one or two row tiles (three spill)
+template <bool kPacked>
+int run_gemv_regx2(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                   int64_t N, int64_t K, hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;
+    if (share == 1) return launch_gemv_regx<1, 8, 2, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    return launch_gemv_regx<2, 8, 2, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+}
+
+template <bool kPacked>
+int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+             int64_t N, int64_t K, hipStream_t stream)
+{
+    if (M > 16) return run_gemv_regx2<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    switch (pick_gemv(M, N, K)) {
+        case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return run_gemv_regx<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    }
+}
+
+template <int TM, bool kSplit, bool kPacked>
+int launch_gemm_reg_tm(const void *x, const void *codes, const void *grid, float scale, void *y, float *part,
+                       int64_t M, int64_t N, int64_t K, int splits, hipStream_t stream)
+{
+    dim3 g((unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)((N + kGrBN - 1) / kGrBN), (unsigned)splits);
+    return launch<true, !kSplit>(gemm_reg_kernel<TM, kSplit, kPacked>, g, dim3(256), gr_smem_bytes(TM), stream,
+                                 (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, part, (int)M,
+                                 (int)N, (int)K, splits, aligned(y, 8) ? 1 : 0);
+}
+
+// rows of x per block: 32, 64 or 128
+inline int gemm_reg_tm(int64_t M) { return M <= 32 ? 1 : M <= 64 ? 2 : 4; }
+
+template <bool kPacked = false>
+int launch_gemm_reg(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                    int64_t N, int64_t K, hipStream_t stream)
+{
+    switch (gemm_reg_tm(M)) {
+        case 1: return launch_gemm_reg_tm<1, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+        case 2: return launch_gemm_reg_tm<2, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+        default: return launch_gemm_reg_tm<4, false, kPacked>(x, codes, grid, scale, y, nullptr, M, N, K, 1, stream);
+    }
+}
+
+// How many ways to split K so that the blocks about fill the chip: as many as fit the CU count
+// without starting a second round, each with at least 4 k tiles, and no more than the
+// workspace holds partial sums for.  1 = no split.
+int splitk_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, int cus)
+{
+    const int tm = gemm_reg_tm(M);
+    const int64_t tiles = ((M + 32 * tm - 1) / (32 * tm)) * ((N + kGrBN - 1) / kGrBN);
+    int64_t splits = cus / tiles;
+    const int64_t k_tiles = K / kGrBK;
+    if (splits > k_tiles / 4) splits = k_tiles / 4;
+    if (splits > 64) splits = 64;
+    const int64_t per_split = M * N * 4;
+    if (per_split > 0 && splits * per_split > workspace_bytes) splits = workspace_bytes / per_split;
+    return splits < 2 ? 1 : (int)splits;
+}
+
+template <bool kPacked = false>
+int launch_gemm_splitk(const void *x, const void *codes, const void *grid, float scale, void *y, void *workspace,
+                       int splits, int64_t M, int64_t N, int64_t K, hipStream_t stream)
+{
+    float *part = reinterpret_cast<float *>(workspace);
+    int st;
+    switch (gemm_reg_tm(M)) {
+        case 1: st = launch_gemm_reg_tm<1, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+        case 2: st = launch_gemm_reg_tm<2, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+        default: st = launch_gemm_reg_tm<4, true, kPacked>(x, codes, grid, scale, y, part, M, N, K, splits, stream); break;
+    }
+    if (st != 0) return st;
+    const int64_t mn = M * N;
+    const int64_t blocks = (mn + 1023) / 1024;
+    return launch<false, true>(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const float *)part,
+                               (uint16_t *)y, mn, splits, scale);
+}
+
+// the register-operand kernel addresses codes and x through 31-bit buffer offsets
+bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
+{
+    return N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31) && N <= 65535LL * kGrBN;
+}
+
+// Smallest M that takes the split-K path when a workspace is given (up to M = 16 the
+// matrix-vector kernels are as fast or faster).
+constexpr int kSplitKMinM = 17;
+
+bool splitk_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
+               int64_t K)
+{
+    return M >= kSplitKMinM && gemm_ok(x, codes, grid, y, M, N, K) && gemm_reg_ok(M, N, K) && aligned(y, 8);
+}
+
+// The register-operand kernel where its offsets fit, else the LDS-staged one (256 x 128, 8 waves)
+int run_gemm(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+             int64_t N, int64_t K, hipStream_t stream)
+{
+    if (gemm_reg_ok(M, N, K)) return launch_gemm_reg(x, codes, grid, scale, y, M, N, K, stream);
+    typedef GemmCfg<4, 2, 2, 2> C;
+    dim3 g((unsigned)((N + C::kBN - 1) / C::kBN), (unsigned)((M + C::kBM - 1) / C::kBM));
+    return launch(gemm_kernel<4, 2, 2, 2>, g, dim3(C::kThreads), sizeof(typename C::Shared), stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  aligned(y, 8) ? 1 : 0);
+}
+
+// y = 0 when K == 0 (empty sum), any M, N.
+__global__ void zero_kernel(uint16_t *y, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        y[i] = 0;
+}
+
+int run_generic(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                int64_t N, int64_t K, hipStream_t stream)
+{
+    if (K == 0) {
+        int64_t n = M * N;
+        unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+        return launch(zero_kernel, dim3(blocks), dim3(256), 0, stream, (uint16_t *)y, n);
+    }
+    int64_t blocks = (N + 3) / 4;
+    if (blocks > 65535 * 16) blocks = 65535 * 16;
+    return launch(generic_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t *)x,
+                  (const uint16_t *)codes, grid, scale, (uint16_t *)y, M, N, K);
+}
+
+template <int R, bool kTiled, bool kFirst, bool kLast>
+int launch_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+                 hipStream_t stream)
+{
+    constexpr int W = 8, D = 2;
+    const size_t shmem = (size_t)2 * kI8TableBytes + (R <= 2 ? 2 : 1) * W * R * kWave * 16;
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch<kFirst, kLast>(int8x_kernel<R, W, D, kTiled>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                                 (const int8_t *)x, (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M,
+                                 (int)N, (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+// Which kernel the integer operator takes for 16-byte aligned buffers.  Many rows of x: the
+// matrix-matrix kernel costs about K * 11.5 ns per round of one 256 x 128 tile per CU (47 us at
+// K = 4096) however few of its tiles exist, the matrix-vector kernel about 3 us plus its code
+// bytes at 3.5 TB/s per 16 rows of x; the cheaper estimate wins (M = 64 at 4096 x 4096: four
+// matrix-vector launches, 20 us; M = 256: one matrix-matrix launch, 47 us against 75).
+enum Int8Kind { kInt8Scalar, kInt8Gemv, kInt8Gemm };
+Int8Kind pick_int8(int64_t M, int64_t N, int64_t K, int cus)
+{
+    if (M < 1 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31) || K > (1 << 17))
+        return kInt8Scalar;
+    if (M > 16 && M * K < (1LL << 31)) {
+        const int64_t tiles = ((M + kI8gBM - 1) / kI8gBM) * ((N + kI8gBN - 1) / kI8gBN);
+        const double t_gemm = 3.0 + (double)((tiles + cus - 1) / cus) * (double)K * 0.0115;
+        const double t_gemv = (double)((M + 15) / 16) * (3.0 + (double)N * (double)(K >> 2) / 3.5e6);
+        if (t_gemm < t_gemv) return kInt8Gemm;
+    }
+    return kInt8Gemv;
+}
+
+template <bool kTiled>
+int launch_int8g(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+                 hipStream_t stream)
+{
+    dim3 g((unsigned)((M + kI8gBM - 1) / kI8gBM), (unsigned)((N + kI8gBN - 1) / kI8gBN));
+    return launch(int8g_kernel<kTiled>, g, dim3(512), kI8gSmem, stream, (const int8_t *)x, (const uint16_t *)codes,
+                  (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
+}
+
+// one launch for up to 16 rows of x; first / last: position in the operator call's sequence of
+// launches, for the timing events
+template <bool kTiled>
+int run_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+              bool first, bool last, hipStream_t stream)
+{
+    // row block = the workgroup's share of tiles when that is one to four, else the size that needs
+    // the fewest blocks (x is fetched once per row block), as for the half-precision kernel
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;
+    int best = 1;
+    for (int r = 2; r <= 4; r++)
+        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
+#define DMM_I8X(RR)                                                                                         \
+    (first ? (last ? launch_int8x<RR, kTiled, true, true>(x, codes, cb, out, M, N, K, stream)               \
+                   : launch_int8x<RR, kTiled, true, false>(x, codes, cb, out, M, N, K, stream))              \
+           : (last ? launch_int8x<RR, kTiled, false, true>(x, codes, cb, out, M, N, K, stream)              \
+                   : launch_int8x<RR, kTiled, false, false>(x, codes, cb, out, M, N, K, stream)))
+    return best == 1 ? DMM_I8X(1) : best == 2 ? DMM_I8X(2) : best == 3 ? DMM_I8X(3) : DMM_I8X(4);
+#undef DMM_I8X
+}
+
+// CU count for the pure queries (kernel names, workspace size), which must answer without a
+// device: the current device's if it has been set up, else the MI355X's 256
+int cu_count_or_default()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    return g_dev[dev].ready.load(std::memory_order_acquire) ? g_dev[dev].cus : 256;
+}
+
+// the operator's dispatch once the arguments are checked and the device is ready
+int dispatch_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M, int64_t N,
+                 int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K)) {
+        const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
+        if (splits >= 2) return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, s);
+    }
+    if (gemv_ok(x, codes, grid, y, M, N, K)) return run_gemv<false>(x, codes, grid, scale, y, M, N, K, s);
+    if (gemm_ok(x, codes, grid, y, M, N, K)) return run_gemm(x, codes, grid, scale, y, M, N, K, s);
+    return run_generic(x, codes, grid, scale, y, M, N, K, s);
+}
+
+// ------------------------------------------------------------------ the operator on host memory
+// The reference's own CPU path is a scalar decode and a triple loop (/root/reference/test_decode_matmul.py:29-71);
+// this is the same thing for the half-precision form, in plain C++ for tensors that live in host
+// memory: no GPU is involved and no GPU call is made.  Not a fallback: device pointers never come
+// here, the entry points below are separate ones.  One rounding per weight (the fp32 sum of a half
+// and +-1/4 is exact), fp32 sums over k in ascending order, rows of W spread over host threads.
+inline void host_decode_row(const uint16_t *codes, const half_t *grid, int64_t kc, half_t *w)
+{
+    for (int64_t j = 0; j < kc; j++) {
+        const uint32_t c = codes[j];
+        const uint32_t idx = c & 0xFFu, s7 = (c >> 8) & 0x7Fu;
+        const uint32_t s8 = s7 | ((uint32_t)(__builtin_popcount(s7) & 1) << 7);
+        const float shift = (c & 0x8000u) ? -0.25f : 0.25f;
+        for (int d = 0; d < 8; d++) {
+            const float g = (float)grid[idx * 8 + d];
+            w[j * 8 + d] = (half_t)(((s8 >> d) & 1u ? -g : g) + shift);
+        }
+    }
+}
+
+template <typename F>
+void host_parallel_rows(int64_t n_rows, int64_t work_per_row, F body)
+{
+    unsigned threads = std::thread::hardware_concurrency();
+    if (threads == 0) threads = 1;
+    if (threads > 16) threads = 16;
+    if (n_rows * work_per_row < (1 << 20) || n_rows < 2) threads = 1;
+    if ((int64_t)threads > n_rows) threads = (unsigned)n_rows;
+    if (threads == 1) {
+        body(0, n_rows);
+        return;
+    }
+    std::vector<std::thread> pool;
+    for (unsigned t = 0; t < threads; t++)
+        pool.emplace_back([=] { body(n_rows * t / threads, n_rows * (t + 1) / threads); });
+    for (auto &th : pool) th.join();
+}

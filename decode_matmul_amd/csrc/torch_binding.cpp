@@ -1,5 +1,5 @@
 // PyTorch-ROCm operator over the C ABI of libdmm.so.  Host code only: no device code is
-// compiled here, the kernels live in dmm.hip behind include/dmm.h.
+// compiled here, the kernels live in dmm.hip and the dmm_*.h files it includes, behind include/dmm.h.
 //
 // Mirrors the operator boundary of the reference,
 // /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:178-239: one module, a function
