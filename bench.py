@@ -374,6 +374,8 @@ def main():
         out["gemv_7b_step"] = gemv_7b_step(torch, lib, capi, workload, dev, rand_codes)
         out["gemv_7b_shapes"] = gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes)
         out["small_batch"] = small_batch(torch, lib, capi, workload, dev, stream, rand_codes)
+        out["small_batch_70b"] = small_batch(torch, lib, capi, workload, dev, stream, rand_codes,
+                                             shapes=workload.LLAMA2_70B, batches=(2, 4, 8, 16))
         out["integer_operator"] = integer_operator(torch, lib, capi, workload, dev, stream, rand_codes)
         out["prefill"] = prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes)
         out["cpu_baseline"] = cpu_baseline(torch, workload)
@@ -609,12 +611,15 @@ def gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes):
     return rows
 
 
-def small_batch(torch, lib, capi, workload, dev, stream, rand_codes):
+def small_batch(torch, lib, capi, workload, dev, stream, rand_codes, shapes=None, batches=(4, 8, 16, 32)):
+    """A few rows of x (the small-batch configuration's shapes by default; the headline's shapes
+    as a second leg): kernel durations by events, every launch on the next of enough code
+    buffers to stay out of the Infinity Cache."""
     rows = []
-    for K, N in workload.SMALL_BATCH:
-        copies = 24
+    for K, N in (workload.SMALL_BATCH if shapes is None else shapes):
+        copies = max(2, -(-320 * 1000000 // workload.code_bytes(N, K)))
         codes = rand_codes(N, K, copies, 7)
-        for M in (4, 8, 16, 32):
+        for M in batches:
             x, _, grid, scale = workload.make_inputs(M, 8, K, seed=0)
             x, grid = x.to(dev), grid.to(dev)
             y = torch.empty(M, N, dtype=torch.float16, device=dev)

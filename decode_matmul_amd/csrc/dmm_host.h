@@ -66,9 +66,11 @@ const std::vector<KernelInfo> &kernel_table()
         DMM_BOTH_LAYOUTS(DMM_K_STREAM),
 #define DMM_K_Q8(P) kinfo(gemv_q8_kernel<1, 16, 2, P>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P>, kLdsMax, true), kinfo(gemv_q8c_kernel<3, 1, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_Q8),
-#define DMM_K_REGX(P)                                                                                        \
-    kinfo(gemv_regx_kernel<1, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 1, 2, P>, kLdsMax, true),     \
-        kinfo(gemv_regx_kernel<3, 8, 1, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 1, 2, P>, kLdsMax, true), \
+#define DMM_K_REGX_XI(P, XI)                                                                                            \
+    kinfo(gemv_regx_kernel<1, 8, 1, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 1, 2, P, XI>, kLdsMax, true),     \
+        kinfo(gemv_regx_kernel<3, 8, 1, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 1, 2, P, XI>, kLdsMax, true)
+#define DMM_K_REGX(P)                                                                      \
+    DMM_K_REGX_XI(P, 2), DMM_K_REGX_XI(P, 4), DMM_K_REGX_XI(P, 8),                            \
         kinfo(gemv_regx_kernel<1, 8, 2, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, 2, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_REGX),
 #define DMM_K_GREG(P)                                                                                        \
@@ -85,6 +87,7 @@ const std::vector<KernelInfo> &kernel_table()
 #undef DMM_K_I8X
 #undef DMM_K_GREG
 #undef DMM_K_REGX
+#undef DMM_K_REGX_XI
 #undef DMM_K_Q8
 #undef DMM_K_STREAM
 #undef DMM_BOTH_LAYOUTS
@@ -246,14 +249,15 @@ bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
            N * (K >> 2) < (1LL << 31);
 }
 
-template <int R, int W, int MT, int D, bool kPacked = false>
+// XI > 0: the x of a step goes through one 8 KB piece of LDS per wave, which also carries the partial sums
+template <int R, int W, int MT, int D, bool kPacked = false, int XI = 0>
 int launch_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                      int64_t N, int64_t K, hipStream_t stream)
 {
-    const size_t shmem = (size_t)kSTablesBytes + 2 * W * R * MT * kWave * 16;
+    const size_t shmem = (size_t)kSTablesBytes + (XI > 0 ? W * kRegxPiece : 2 * W * R * MT * kWave * 16);
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_regx_kernel<R, W, MT, D, kPacked>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+    return launch(gemv_regx_kernel<R, W, MT, D, kPacked, XI>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
@@ -311,6 +315,19 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
     return kGemvRegx;
 }
 
+// XI: load instructions per slice of x, two rows each
+template <bool kPacked, int XI>
+int run_gemv_regx_r(int r, const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
+                    int64_t N, int64_t K, hipStream_t stream)
+{
+    switch (r) {
+        case 1: return launch_gemv_regx<1, 8, 1, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
+        case 2: return launch_gemv_regx<2, 8, 1, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
+        case 3: return launch_gemv_regx<3, 8, 1, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return launch_gemv_regx<4, 8, 1, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
+    }
+}
+
 // The register-x kernel for M <= 16 reads the x slice of a k step once per row block, so the row
 // block should be the workgroup's whole share of tiles when that is 1 .. 4 tiles, and otherwise
 // the size that needs the fewest blocks.
@@ -323,12 +340,9 @@ int run_gemv_regx(const void *x, const void *codes, const void *grid, float scal
     int best = 1;
     for (int r = 2; r <= 4; r++)
         if ((share + r - 1) / r < (share + best - 1) / best) best = r;
-    switch (best) {
-        case 1: return launch_gemv_regx<1, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        case 2: return launch_gemv_regx<2, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        case 3: return launch_gemv_regx<3, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        default: return launch_gemv_regx<4, 8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    }
+    return M <= 4 ? run_gemv_regx_r<kPacked, 2>(best, x, codes, grid, scale, y, M, N, K, stream)
+         : M <= 8 ? run_gemv_regx_r<kPacked, 4>(best, x, codes, grid, scale, y, M, N, K, stream)
+                  : run_gemv_regx_r<kPacked, 8>(best, x, codes, grid, scale, y, M, N, K, stream);
 }
 
 // M = 17 .. 32: two x tiles per wave leave registers for one or two row tiles (three spill)

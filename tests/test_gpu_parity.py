@@ -611,14 +611,15 @@ def test_matrix_matrix_with_y_only_2_byte_aligned(M, N, K):
 
 
 # ----------------------------------------------------------------- small-batch kernel, row blocks
-@pytest.mark.parametrize("M,K", [(8, 4096), (16, 4096), (3, 28672), (12, 1024 * 5)])
+@pytest.mark.parametrize("M,K", [(8, 4096), (16, 4096), (3, 28672), (12, 1024 * 5), (2, 28672), (5, 16384), (9, 8192)])
 @pytest.mark.parametrize("share", [1, 2, 3, 4, 5, 7, 8])
 def test_small_batch_row_block_sizes(M, K, share):
     """The register-x kernel takes one to four row tiles per block, chosen from the most tiles
     a workgroup gets (`share`): every choice, with workgroups whose last block is partial and
-    an N that is no multiple of 16.  Reference: the library's own decode (pinned bit for bit
-    against the oracle above) times x in fp32 on the GPU, plus the oracle itself on the first
-    and last rows."""
+    an N that is no multiple of 16; and every width of the x slice it moves through the LDS (up
+    to 4, 8 and 16 rows of x, full and with rows to spare).  y lies between guard bands.
+    Reference: the library's own decode (pinned bit for bit against the oracle above) times x
+    in fp32 on the GPU, plus the oracle itself on the first and last rows."""
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     N = 16 * (cus * share - 37) - 4
     assert capi.lib().dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_regx_kernel"
@@ -627,9 +628,12 @@ def test_small_batch_row_block_sizes(M, K, share):
     g.manual_seed(1000 * M + share)
     codes = torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=DEV)
     xd, gd = dev(x), dev(grid)
-    y = c_matmul(xd, codes, gd, scale, "gemv")
+    buf = torch.full((64 + M * N + 64,), -7.0, dtype=torch.float16, device=DEV)
+    y = buf[64:64 + M * N].view(M, N)
+    c_matmul(xd, codes, gd, scale, "gemv", out=y)
     W = c_decode(codes, gd)
     torch.cuda.synchronize()
+    assert torch.all(buf[:64] == -7.0) and torch.all(buf[64 + M * N:] == -7.0)
     ref = (xd.float() @ W.float().T) * scale
     assert_close_to_oracle(y, ref.cpu().numpy(), "regx M=%d N=%d K=%d" % (M, N, K))
     rows = torch.from_numpy(np.r_[0:24, N - 24:N]).to(DEV)
