@@ -13,6 +13,10 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 // ------------------------------------------------------------------ host side
 thread_local hipEvent_t tls_start = nullptr;
 thread_local hipEvent_t tls_stop = nullptr;
+// an operator call made of several whole launches (rows of x in two halves) narrows the span of
+// the timing events from outside: its first launch records only the start, its last only the stop
+thread_local bool tls_span_first = true;
+thread_local bool tls_span_last = true;
 
 template <typename T>
 struct same_type { typedef T type; };
@@ -28,7 +32,8 @@ int launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStr
     void *argv[] = {(void *)&args...};
     if (tls_start && tls_stop)
         return (int)hipExtLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream,
-                                       kFirst ? tls_start : nullptr, kLast ? tls_stop : nullptr, 0);
+                                       kFirst && tls_span_first ? tls_start : nullptr,
+                                       kLast && tls_span_last ? tls_stop : nullptr, 0);
     return (int)hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream);
 }
 
@@ -360,7 +365,22 @@ template <bool kPacked>
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
-    if (M > 16) return run_gemv_regx2<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    if (M > 16) {
+        // 17 .. 32 rows of x.  The two-tile kernel still loads x fragment by fragment; from 8 MB of codes
+        // on, two launches of the 16-row kernels are faster although they read the codes twice (graph
+        // launches, one call of 32 rows against two of 16, us: 8192 -> 28672 67.5 / 49.4, 28672 -> 8192
+        // 61.5 / 50.2, 8192 -> 10240 36.1 / 27.0, 11008 -> 4096 24.3 / 20.8, 4096 -> 11008 20.6 / 19.2).
+        if (N * (K >> 2) < (8LL << 20)) return run_gemv_regx2<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        const bool outer_first = tls_span_first, outer_last = tls_span_last;
+        tls_span_last = false;
+        int st = run_gemv<kPacked>(x, codes, grid, scale, y, 16, N, K, stream);
+        tls_span_first = false;
+        tls_span_last = outer_last;
+        if (st == DMM_OK)
+            st = run_gemv<kPacked>((const uint16_t *)x + 16 * K, codes, grid, scale, (uint16_t *)y + 16 * N, M - 16, N, K, stream);
+        tls_span_first = outer_first;
+        return st;
+    }
     switch (pick_gemv(M, N, K)) {
         case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);

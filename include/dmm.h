@@ -119,7 +119,8 @@ int dmm_decode_matmul_noalloc_f16(const void *x, const void *codes, const void *
  * returns DMM_ERR_UNSUPPORTED outside its domain instead of falling back:
  *   dmm_gemv_f16     M <= 32, K % 256 == 0, N % 4 == 0, 16-byte aligned x/codes/grid,
  *                    8-byte aligned y.  Decoded registers feed the MFMA unit directly;
- *                    HBM-bound on the code bytes N*K/4.
+ *                    HBM-bound on the code bytes N*K/4.  One kernel launch, except for
+ *                    17 <= M with 8 MB of codes or more: two (rows 0 .. 15, then the rest).
  *   dmm_gemm_f16     K % 64 == 0, 16-byte aligned x/codes/grid.  Decoded tiles staged in
  *                    LDS, fp16 MFMA with fp32 accumulate.
  *   dmm_generic_f16  any K % 8 == 0, 2-byte alignment: wave-per-row dot products with a

@@ -641,6 +641,49 @@ def test_small_batch_row_block_sizes(M, K, share):
     assert_close_to_oracle(y[:, rows], want, "regx M=%d N=%d K=%d, oracle rows" % (M, N, K))
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 4112, 8192), (24, 2052, 28672), (32, 8200, 4096), (31, 11008, 4096)])
+def test_17_to_32_rows_of_x_on_a_large_code_matrix(M, N, K):
+    """From 8 MB of codes on, 17 .. 32 rows of x are two launches of the 16-row kernels (rows
+    0 .. 15, then the rest, which may be a single row on the 8-bit kernel): same tolerance, y
+    between guard bands, and the timing hook spans both launches."""
+    x, _, grid, scale = workload.make_inputs(M, 8, K, seed=M)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(M * 31 + 5)
+    codes = torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=DEV)
+    xd, gd = dev(x), dev(grid)
+    buf = torch.full((64 + M * N + 64,), -7.0, dtype=torch.float16, device=DEV)
+    y = buf[64:64 + M * N].view(M, N)
+    c_matmul(xd, codes, gd, scale, "gemv", out=y)
+    W = c_decode(codes, gd)
+    torch.cuda.synchronize()
+    assert torch.all(buf[:64] == -7.0) and torch.all(buf[64 + M * N:] == -7.0)
+    ref = (xd.float() @ W.float().T) * scale
+    assert_close_to_oracle(y, ref.cpu().numpy(), "two launches M=%d N=%d K=%d" % (M, N, K))
+    # the same rows as calls of their own give the same bits
+    y0 = c_matmul(xd[:16].contiguous(), codes, gd, scale, "gemv")
+    y1 = c_matmul(xd[16:].contiguous(), codes, gd, scale, "gemv")
+    torch.cuda.synchronize()
+    assert torch.equal(y[:16], y0) and torch.equal(y[16:], y1)
+    # the hook's events bracket the whole call: longer than either half alone
+    lib = capi.lib()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+
+    def timed(xpart, ypart):
+        lib.dmm_set_kernel_events(ev[0].cuda_event, ev[1].cuda_event)
+        try:
+            c_matmul(xpart, codes, gd, scale, "gemv", out=ypart)
+        finally:
+            lib.dmm_set_kernel_events(None, None)
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1])
+    for e in ev:
+        e.record()
+    torch.cuda.synchronize()
+    whole = min(timed(xd, y) for _ in range(3))
+    first = min(timed(xd[:16].contiguous(), y0) for _ in range(3))
+    assert whole > first * 1.2, (whole, first)
+
+
 # ----------------------------------------------------------------- seeded random shapes
 def _random_shapes(n, seed):
     rng = np.random.default_rng(seed)
