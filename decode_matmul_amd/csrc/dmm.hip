@@ -233,13 +233,16 @@ int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *
     hipStream_t s = (hipStream_t)stream;
     const bool mm_ok = gemm_ok(x, packed, grid, y, M, N, K) && gemm_reg_ok(M, ((N + 15) / 16) * 16, K);
     const bool mv_ok = gemv_ok(x, packed, grid, y, M, N, K);
-    if (!mm_ok && !mv_ok) return DMM_ERR_UNSUPPORTED;
+    const bool rows_ok = gemv_rows_ok(x, packed, grid, y, M, N, K);   // more than 32 rows, 16 at a time
+    if (!mm_ok && !rows_ok) return DMM_ERR_UNSUPPORTED;
     if ((st = ensure_ready(s))) return st;
     if (workspace && workspace_bytes > 0 && mm_ok && M >= kSplitKMinM && aligned(y, 8)) {
         const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
         if (splits >= 2) return launch_gemm_splitk<true>(x, packed, grid, scale, y, workspace, splits, M, N, K, s);
     }
     if (mv_ok) return run_gemv<true>(x, packed, grid, scale, y, M, N, K, s);
+    if (rows_ok && (!mm_ok || passes_beat_gemm(M, N, K, cu_count())))
+        return run_gemv_regx<true>(x, packed, grid, scale, y, M, N, K, s);
     return launch_gemm_reg<true>(x, packed, grid, scale, y, M, N, K, s);
 }
 

@@ -13,10 +13,6 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 // ------------------------------------------------------------------ host side
 thread_local hipEvent_t tls_start = nullptr;
 thread_local hipEvent_t tls_stop = nullptr;
-// an operator call made of several whole launches (rows of x in two halves) narrows the span of
-// the timing events from outside: its first launch records only the start, its last only the stop
-thread_local bool tls_span_first = true;
-thread_local bool tls_span_last = true;
 
 template <typename T>
 struct same_type { typedef T type; };
@@ -32,8 +28,7 @@ int launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStr
     void *argv[] = {(void *)&args...};
     if (tls_start && tls_stop)
         return (int)hipExtLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream,
-                                       kFirst && tls_span_first ? tls_start : nullptr,
-                                       kLast && tls_span_last ? tls_stop : nullptr, 0);
+                                       kFirst ? tls_start : nullptr, kLast ? tls_stop : nullptr, 0);
     return (int)hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, argv, shmem, stream);
 }
 
@@ -71,12 +66,10 @@ const std::vector<KernelInfo> &kernel_table()
         DMM_BOTH_LAYOUTS(DMM_K_STREAM),
 #define DMM_K_Q8(P) kinfo(gemv_q8_kernel<1, 16, 2, P>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P>, kLdsMax, true), kinfo(gemv_q8c_kernel<3, 1, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_Q8),
-#define DMM_K_REGX_XI(P, XI)                                                                                            \
-    kinfo(gemv_regx_kernel<1, 8, 1, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 1, 2, P, XI>, kLdsMax, true),     \
-        kinfo(gemv_regx_kernel<3, 8, 1, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 1, 2, P, XI>, kLdsMax, true)
-#define DMM_K_REGX(P)                                                                      \
-    DMM_K_REGX_XI(P, 2), DMM_K_REGX_XI(P, 4), DMM_K_REGX_XI(P, 8),                            \
-        kinfo(gemv_regx_kernel<1, 8, 2, 2, P>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, 2, P>, kLdsMax, true)
+#define DMM_K_REGX_XI(P, XI)                                                                                      \
+    kinfo(gemv_regx_kernel<1, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, P, XI>, kLdsMax, true),     \
+        kinfo(gemv_regx_kernel<3, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 2, P, XI>, kLdsMax, true)
+#define DMM_K_REGX(P) DMM_K_REGX_XI(P, 2), DMM_K_REGX_XI(P, 4), DMM_K_REGX_XI(P, 8)
         DMM_BOTH_LAYOUTS(DMM_K_REGX),
 #define DMM_K_GREG(P)                                                                                        \
     kinfo(gemm_reg_kernel<1, false, P>, gr_smem_bytes(1), true), kinfo(gemm_reg_kernel<2, false, P>, gr_smem_bytes(2), true), \
@@ -171,12 +164,21 @@ int check_common(const void *x, const void *codes, const void *grid, const void 
     return DMM_OK;
 }
 
+// what the matrix-vector kernels can take at all: any number of rows of x goes through the small-batch
+// kernel 16 at a time (the operator sends more than 32 there only when that beats the matrix-matrix kernel)
+bool gemv_rows_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
+                  int64_t K)
+{
+    return M >= 1 && M <= 4096 && M * K < (1LL << 30) && K >= 256 && (K & 255) == 0 && K <= (1 << 23) &&
+           N * (K >> 2) < (1LL << 31) && (N & 3) == 0 && aligned(x, 16) && aligned(codes, 16) && aligned(grid, 16) &&
+           aligned(y, 8);
+}
+
+// the domain of the explicit matrix-vector entry points
 bool gemv_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
              int64_t K)
 {
-    return M >= 1 && M <= 32 && K >= 256 && (K & 255) == 0 && K <= (1 << 23) && N * (K >> 2) < (1LL << 31) &&
-           (N & 3) == 0 && aligned(x, 16) &&
-           aligned(codes, 16) && aligned(grid, 16) && aligned(y, 8);
+    return gemv_rows_ok(x, codes, grid, y, M, N, K) && M <= 32;
 }
 
 bool gemm_ok(const void *x, const void *codes, const void *grid, const void *, int64_t M, int64_t N,
@@ -254,15 +256,15 @@ bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
            N * (K >> 2) < (1LL << 31);
 }
 
-// XI > 0: the x of a step goes through one 8 KB piece of LDS per wave, which also carries the partial sums
-template <int R, int W, int MT, int D, bool kPacked = false, int XI = 0>
+// the x of a step goes through one 8 KB piece of LDS per wave, which also carries the partial sums
+template <int R, int W, int D, bool kPacked, int XI>
 int launch_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                      int64_t N, int64_t K, hipStream_t stream)
 {
-    const size_t shmem = (size_t)kSTablesBytes + (XI > 0 ? W * kRegxPiece : 2 * W * R * MT * kWave * 16);
+    const size_t shmem = (size_t)kSTablesBytes + W * kRegxPiece;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_regx_kernel<R, W, MT, D, kPacked, XI>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+    return launch(gemv_regx_kernel<R, W, D, kPacked, XI>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
@@ -326,14 +328,14 @@ int run_gemv_regx_r(int r, const void *x, const void *codes, const void *grid, f
                     int64_t N, int64_t K, hipStream_t stream)
 {
     switch (r) {
-        case 1: return launch_gemv_regx<1, 8, 1, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
-        case 2: return launch_gemv_regx<2, 8, 1, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
-        case 3: return launch_gemv_regx<3, 8, 1, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
-        default: return launch_gemv_regx<4, 8, 1, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
+        case 1: return launch_gemv_regx<1, 8, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
+        case 2: return launch_gemv_regx<2, 8, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
+        case 3: return launch_gemv_regx<3, 8, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return launch_gemv_regx<4, 8, 2, kPacked, XI>(x, codes, grid, scale, y, M, N, K, stream);
     }
 }
 
-// The register-x kernel for M <= 16 reads the x slice of a k step once per row block, so the row
+// The small-batch kernel reads the x slice of a k step once per row block and pass, so the row
 // block should be the workgroup's whole share of tiles when that is 1 .. 4 tiles, and otherwise
 // the size that needs the fewest blocks.
 template <bool kPacked>
@@ -350,37 +352,11 @@ int run_gemv_regx(const void *x, const void *codes, const void *grid, float scal
                   : run_gemv_regx_r<kPacked, 8>(best, x, codes, grid, scale, y, M, N, K, stream);
 }
 
-// M = 17 .. 32: two x tiles per wave leave registers for one or two row tiles (three spill)
-template <bool kPacked>
-int run_gemv_regx2(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
-                   int64_t N, int64_t K, hipStream_t stream)
-{
-    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;
-    if (share == 1) return launch_gemv_regx<1, 8, 2, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-    return launch_gemv_regx<2, 8, 2, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-}
-
 template <bool kPacked>
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
-    if (M > 16) {
-        // 17 .. 32 rows of x.  The two-tile kernel still loads x fragment by fragment; from 8 MB of codes
-        // on, two launches of the 16-row kernels are faster although they read the codes twice (graph
-        // launches, one call of 32 rows against two of 16, us: 8192 -> 28672 67.5 / 49.4, 28672 -> 8192
-        // 61.5 / 50.2, 8192 -> 10240 36.1 / 27.0, 11008 -> 4096 24.3 / 20.8, 4096 -> 11008 20.6 / 19.2).
-        if (N * (K >> 2) < (8LL << 20)) return run_gemv_regx2<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
-        const bool outer_first = tls_span_first, outer_last = tls_span_last;
-        tls_span_last = false;
-        int st = run_gemv<kPacked>(x, codes, grid, scale, y, 16, N, K, stream);
-        tls_span_first = false;
-        tls_span_last = outer_last;
-        if (st == DMM_OK)
-            st = run_gemv<kPacked>((const uint16_t *)x + 16 * K, codes, grid, scale, (uint16_t *)y + 16 * N, M - 16, N, K, stream);
-        tls_span_first = outer_first;
-        return st;
-    }
+    if (M > 16) return run_gemv_regx<kPacked>(x, codes, grid, scale, y, M, N, K, stream);   // 16 rows per pass
     switch (pick_gemv(M, N, K)) {
         case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
@@ -567,6 +543,21 @@ int cu_count_or_default()
     return g_dev[dev].ready.load(std::memory_order_acquire) ? g_dev[dev].cus : 256;
 }
 
+// More than 32 rows of x and no workspace.  The matrix-matrix kernel costs about K * 6.9 ns (x tiles
+// of up to 64 rows) or K * 10.4 ns (128 rows) per round of one 256-row tile per CU, however few of its
+// tiles exist; the small-batch kernel about 1.5 us plus the code bytes at 3 TB/s (they come from the
+// caches after the first pass) per 16 rows of x.  The cheaper estimate wins.  Graph launches, us,
+// matrix-matrix / passes: M = 64 11008 -> 4096 74.7 / 30.2, 28672 -> 8192 186.7 / 95.6, 8192 -> 28672
+// 57.7 / 79.6; M = 128 4096 -> 11008 47.6 / 41.7, 8192 -> 10240 86.1 / 71.5, 8192 -> 28672 88.2 / 150.2.
+bool passes_beat_gemm(int64_t M, int64_t N, int64_t K, int cus)
+{
+    const int tm = gemm_reg_tm(M);
+    const int64_t tiles = ((M + 32 * tm - 1) / (32 * tm)) * ((N + kGrBN - 1) / kGrBN);
+    const double t_gemm = 3.0 + (double)((tiles + cus - 1) / cus) * (double)K * (tm == 4 ? 0.0104 : 0.0069);
+    const double t_pass = 2.0 + (double)((M + 15) / 16) * (1.5 + (double)N * (double)(K >> 2) / 3.0e6);
+    return t_pass < t_gemm;
+}
+
 // the operator's dispatch once the arguments are checked and the device is ready
 int dispatch_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M, int64_t N,
                  int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t s)
@@ -576,6 +567,8 @@ int dispatch_f16(const void *x, const void *codes, const void *grid, float scale
         if (splits >= 2) return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, s);
     }
     if (gemv_ok(x, codes, grid, y, M, N, K)) return run_gemv<false>(x, codes, grid, scale, y, M, N, K, s);
+    if (gemv_rows_ok(x, codes, grid, y, M, N, K) && passes_beat_gemm(M, N, K, cu_count()))
+        return run_gemv_regx<false>(x, codes, grid, scale, y, M, N, K, s);
     if (gemm_ok(x, codes, grid, y, M, N, K)) return run_gemm(x, codes, grid, scale, y, M, N, K, s);
     return run_generic(x, codes, grid, scale, y, M, N, K, s);
 }

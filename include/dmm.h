@@ -78,7 +78,10 @@ int dmm_decode_f16(const void *codes, const void *grid, void *W,
  * [256,8], scalar scale, y half [M,N], all row-major and contiguous.  The only shape
  * demand is K % 8 == 0 (the reference's M%8, N%16, K%2048 demands,
  * decode_matmul_cuda.cu:195-207, do not apply).  Chooses the kernel from M, the shape and
- * the pointer alignments; y is fully overwritten (no caller zeroing). */
+ * the pointer alignments; y is fully overwritten (no caller zeroing).  A few dozen to a few
+ * hundred rows of x give the matrix-matrix kernel too few tiles to fill the chip; without a
+ * workspace (below) such a call runs as passes of the small-batch kernel, 16 rows of x each,
+ * where a cost estimate says that is faster. */
 int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, float scale,
                           void *y, int64_t M, int64_t N, int64_t K, void *stream);
 
@@ -119,8 +122,9 @@ int dmm_decode_matmul_noalloc_f16(const void *x, const void *codes, const void *
  * returns DMM_ERR_UNSUPPORTED outside its domain instead of falling back:
  *   dmm_gemv_f16     M <= 32, K % 256 == 0, N % 4 == 0, 16-byte aligned x/codes/grid,
  *                    8-byte aligned y.  Decoded registers feed the MFMA unit directly;
- *                    HBM-bound on the code bytes N*K/4.  One kernel launch, except for
- *                    17 <= M with 8 MB of codes or more: two (rows 0 .. 15, then the rest).
+ *                    HBM-bound on the code bytes N*K/4 (more than 16 rows of x: every
+ *                    workgroup walks its rows of W once per 16 rows of x, so the codes come
+ *                    from HBM once and from the caches after that).
  *   dmm_gemm_f16     K % 64 == 0, 16-byte aligned x/codes/grid.  Decoded tiles staged in
  *                    LDS, fp16 MFMA with fp32 accumulate.
  *   dmm_generic_f16  any K % 8 == 0, 2-byte alignment: wave-per-row dot products with a

@@ -641,11 +641,14 @@ def test_small_batch_row_block_sizes(M, K, share):
     assert_close_to_oracle(y[:, rows], want, "regx M=%d N=%d K=%d, oracle rows" % (M, N, K))
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 4112, 8192), (24, 2052, 28672), (32, 8200, 4096), (31, 11008, 4096)])
-def test_17_to_32_rows_of_x_on_a_large_code_matrix(M, N, K):
-    """From 8 MB of codes on, 17 .. 32 rows of x are two launches of the 16-row kernels (rows
-    0 .. 15, then the rest, which may be a single row on the 8-bit kernel): same tolerance, y
-    between guard bands, and the timing hook spans both launches."""
+@pytest.mark.parametrize("M,N,K", [(17, 4112, 8192), (24, 2052, 28672), (32, 8200, 4096), (31, 11008, 4096),
+                                   (20, 500, 2304), (48, 1028, 4096), (64, 4096, 11008), (100, 2052, 8192),
+                                   (128, 4112, 4096), (33, 16 * 300 - 4, 28672)])
+def test_more_than_16_rows_of_x_in_passes(M, N, K):
+    """More than 16 rows of x go through the small-batch kernel 16 at a time inside one launch
+    (every workgroup walks its row blocks once per 16 rows); beyond 32 rows the operator takes
+    that route where it beats the matrix-matrix kernel, as on these shapes.  Same tolerance, y
+    between guard bands, a last pass with rows to spare."""
     x, _, grid, scale = workload.make_inputs(M, 8, K, seed=M)
     g = torch.Generator(device=DEV)
     g.manual_seed(M * 31 + 5)
@@ -653,35 +656,31 @@ def test_17_to_32_rows_of_x_on_a_large_code_matrix(M, N, K):
     xd, gd = dev(x), dev(grid)
     buf = torch.full((64 + M * N + 64,), -7.0, dtype=torch.float16, device=DEV)
     y = buf[64:64 + M * N].view(M, N)
-    c_matmul(xd, codes, gd, scale, "gemv", out=y)
+    c_matmul(xd, codes, gd, scale, "gemv" if M <= 32 else "auto", out=y)
     W = c_decode(codes, gd)
     torch.cuda.synchronize()
     assert torch.all(buf[:64] == -7.0) and torch.all(buf[64 + M * N:] == -7.0)
     ref = (xd.float() @ W.float().T) * scale
-    assert_close_to_oracle(y, ref.cpu().numpy(), "two launches M=%d N=%d K=%d" % (M, N, K))
-    # the same rows as calls of their own give the same bits
-    y0 = c_matmul(xd[:16].contiguous(), codes, gd, scale, "gemv")
-    y1 = c_matmul(xd[16:].contiguous(), codes, gd, scale, "gemv")
-    torch.cuda.synchronize()
-    assert torch.equal(y[:16], y0) and torch.equal(y[16:], y1)
-    # the hook's events bracket the whole call: longer than either half alone
-    lib = capi.lib()
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-
-    def timed(xpart, ypart):
-        lib.dmm_set_kernel_events(ev[0].cuda_event, ev[1].cuda_event)
-        try:
-            c_matmul(xpart, codes, gd, scale, "gemv", out=ypart)
-        finally:
-            lib.dmm_set_kernel_events(None, None)
+    assert_close_to_oracle(y, ref.cpu().numpy(), "passes M=%d N=%d K=%d" % (M, N, K))
+    rows = torch.from_numpy(np.r_[0:24, N - 24:N]).to(DEV)
+    want = orc.matmul_f32(x.numpy(), orc.decode_f16(codes[rows].cpu().numpy(), grid.numpy()), scale)
+    assert_close_to_oracle(y[:, rows], want, "passes M=%d N=%d K=%d, oracle rows" % (M, N, K))
+    # rows 16 p .. of x as a call of their own on the same kernel give the same bits
+    if M <= 32 and capi.lib().dmm_gemv_kernel_name(M - 16, N, K) == b"dmm::gemv_regx_kernel":
+        y1 = c_matmul(xd[16:].contiguous(), codes, gd, scale, "gemv")
         torch.cuda.synchronize()
-        return ev[0].elapsed_time(ev[1])
-    for e in ev:
-        e.record()
+        assert torch.equal(y[16:], y1)
+    # packed codes take the same route and give the same bits
+    packed = torch.empty(capi.lib().dmm_packed_bytes(N, K), dtype=torch.uint8, device=DEV)
+    capi.check("dmm_pack_codes", capi.lib().dmm_pack_codes(codes.data_ptr(), packed.data_ptr(), N, K,
+                                                           torch.cuda.current_stream().cuda_stream))
+    y2 = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
+    capi.check("dmm_decode_matmul_packed_f16",
+               capi.lib().dmm_decode_matmul_packed_f16(xd.data_ptr(), packed.data_ptr(), gd.data_ptr(), float(scale),
+                                                       y2.data_ptr(), M, N, K, None, 0,
+                                                       torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
-    whole = min(timed(xd, y) for _ in range(3))
-    first = min(timed(xd[:16].contiguous(), y0) for _ in range(3))
-    assert whole > first * 1.2, (whole, first)
+    assert torch.equal(y2, y)
 
 
 # ----------------------------------------------------------------- seeded random shapes
@@ -785,14 +784,15 @@ def test_packed_codes_bit_identical(M, N, K):
 @pytest.mark.parametrize("M,N,K", [(40, 300, 512), (64, 1024, 1024), (200, 771, 2304), (2048, 4096, 4096),
                                    (130, 52, 256), (33, 4100, 1024)])
 def test_packed_codes_matrix_matrix_bit_identical(M, N, K):
-    """The MFMA kernel on packed codes, with and without a split-K workspace: the bits of the
-    row-major calls."""
+    """The operator on packed codes for many rows of x (the MFMA kernel, or passes of the
+    small-batch kernel where those are cheaper), with and without a split-K workspace: the
+    bits of the row-major calls that take the same route."""
     x, codes, grid, scale = workload.make_inputs(M, N, K, seed=N + K + M)
     xd, cd, gd = dev(x), dev(codes), dev(grid)
     lib = capi.lib()
     pk = dmm.pack_codes(cd)
     stream = torch.cuda.current_stream().cuda_stream
-    y_ref = c_matmul(xd, cd, gd, scale, "gemm")
+    y_ref = c_matmul(xd, cd, gd, scale, "auto")
     y = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
     capi.check("dmm_decode_matmul_packed_f16",
                lib.dmm_decode_matmul_packed_f16(xd.data_ptr(), pk.data_ptr(), gd.data_ptr(), scale, y.data_ptr(),
