@@ -278,17 +278,9 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
     if (kind == kInt8Gemm)
         return tiled ? launch_int8g<true>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream)
                      : launch_int8g<false>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream);
-    if (kind == kInt8Gemv) {
-        for (int64_t m0 = 0; m0 < M; m0 += 16) {   // up to 16 rows of x per launch
-            const int64_t mc = M - m0 < 16 ? M - m0 : 16;
-            const int8_t *xs = (const int8_t *)x + m0 * K;
-            int32_t *os = (int32_t *)out + m0 * N;
-            const int e = tiled ? run_int8x<true>(xs, codes, codebook_abs, os, mc, N, K, m0 == 0, m0 + 16 >= M, (hipStream_t)stream)
-                                : run_int8x<false>(xs, codes, codebook_abs, os, mc, N, K, m0 == 0, m0 + 16 >= M, (hipStream_t)stream);
-            if (e) return e;
-        }
-        return DMM_OK;
-    }
+    if (kind == kInt8Gemv)   // 16 rows of x per pass of the one launch
+        return tiled ? run_int8x<true>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream)
+                     : run_int8x<false>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream);
     int64_t blocks = (N + 3) / 4;
     if (blocks > 65535 * 16) blocks = 65535 * 16;
     return launch(int8_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const int8_t *)x,

@@ -322,6 +322,19 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
     return kGemvRegx;
 }
 
+// Row tiles per block of the small-batch kernels (half precision and integer): the workgroup's whole share
+// of tiles when that is one to four, else the size (<= 4) that needs the fewest blocks - the x slice of a
+// k step is fetched once per row block and pass.
+inline int small_batch_row_block(int64_t n_tiles, int64_t cus, int64_t *blocks = nullptr)
+{
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
+    int best = 1;
+    for (int r = 2; r <= 4; r++)
+        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
+    if (blocks) *blocks = (share + best - 1) / best;
+    return best;
+}
+
 // XI: load instructions per slice of x, two rows each
 template <bool kPacked, int XI>
 int run_gemv_regx_r(int r, const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
@@ -342,11 +355,7 @@ template <bool kPacked>
 int run_gemv_regx(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                   int64_t N, int64_t K, hipStream_t stream)
 {
-    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
-    int best = 1;
-    for (int r = 2; r <= 4; r++)
-        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
+    const int best = small_batch_row_block((N + 15) / 16, cu_count());
     return M <= 4 ? run_gemv_regx_r<kPacked, 2>(best, x, codes, grid, scale, y, M, N, K, stream)
          : M <= 8 ? run_gemv_regx_r<kPacked, 4>(best, x, codes, grid, scale, y, M, N, K, stream)
                   : run_gemv_regx_r<kPacked, 8>(best, x, codes, grid, scale, y, M, N, K, stream);
@@ -471,7 +480,7 @@ int run_generic(const void *x, const void *codes, const void *grid, float scale,
                   (const uint16_t *)codes, grid, scale, (uint16_t *)y, M, N, K);
 }
 
-template <int R, bool kTiled, bool kFirst, bool kLast>
+template <int R, bool kTiled>
 int launch_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
                  hipStream_t stream)
 {
@@ -479,25 +488,37 @@ int launch_int8x(const void *x, const void *codes, const void *cb, void *out, in
     const size_t shmem = (size_t)2 * kI8TableBytes + (R <= 2 ? 2 : 1) * W * R * kWave * 16;
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch<kFirst, kLast>(int8x_kernel<R, W, D, kTiled>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
-                                 (const int8_t *)x, (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M,
-                                 (int)N, (int)K, (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    return launch(int8x_kernel<R, W, D, kTiled>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream, (const int8_t *)x,
+                  (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K,
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
 
-// Which kernel the integer operator takes for 16-byte aligned buffers.  Many rows of x: the
-// matrix-matrix kernel costs about K * 11.5 ns per round of one 256 x 128 tile per CU (47 us at
-// K = 4096) however few of its tiles exist, the matrix-vector kernel about 3 us plus its code
-// bytes at 3.5 TB/s per 16 rows of x; the cheaper estimate wins (M = 64 at 4096 x 4096: four
-// matrix-vector launches, 20 us; M = 256: one matrix-matrix launch, 47 us against 75).
+// Which kernel the integer operator takes for 16-byte aligned buffers.  More than 16 rows of x are
+// passes of the matrix-vector kernel (16 rows each, the codes from the caches after the first) or one
+// launch of the matrix-matrix kernel; the cheaper estimate wins.  A pass costs each wave its k steps
+// (K / 256 over 8 waves, per row block) at 0.85 us + 0.17 us per row tile of the block; the
+// matrix-matrix kernel K * 5.2 ns per round of one 256 x 128 tile per CU when few CUs have a tile,
+// rising to K * 8.8 ns with all of them busy (the clock drops).  Graph launches, us, passes /
+// matrix-matrix: 4096 x 4096 M = 128 20.2 / 29.5, M = 256 36.2 / 30.2; 11008 -> 4096 M = 128 48.6 / 63.1,
+// M = 256 90.2 / 63.9; 8192 -> 28672 M = 32 33.7 / 48.7, M = 64 54.5 / 48.6; 28672 -> 8192 M = 128
+// 131.6 / 149.3, M = 256 255.2 / 149.8.
 enum Int8Kind { kInt8Scalar, kInt8Gemv, kInt8Gemm };
 Int8Kind pick_int8(int64_t M, int64_t N, int64_t K, int cus)
 {
-    if (M < 1 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31) || K > (1 << 17))
+    if (M < 1 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31) || K > (1 << 17) ||
+        M * K >= (1LL << 31))
         return kInt8Scalar;
-    if (M > 16 && M * K < (1LL << 31)) {
-        const int64_t tiles = ((M + kI8gBM - 1) / kI8gBM) * ((N + kI8gBN - 1) / kI8gBN);
-        const double t_gemm = 3.0 + (double)((tiles + cus - 1) / cus) * (double)K * 0.0115;
-        const double t_gemv = (double)((M + 15) / 16) * (3.0 + (double)N * (double)(K >> 2) / 3.5e6);
+    if (M > 16) {
+        int64_t tiles = ((M + kI8gBM - 1) / kI8gBM) * ((N + kI8gBN - 1) / kI8gBN);
+        double t_gemm = 5.0;
+        for (; tiles > 0; tiles -= cus) {
+            const double fill = tiles >= cus ? 1.0 : (double)tiles / (double)cus;
+            t_gemm += (double)K * (0.0052 + 0.0036 * fill * fill);
+        }
+        int64_t blocks = 1;
+        const int r = small_batch_row_block((N + 15) / 16, cus, &blocks);
+        const double t_pass = (double)(blocks * (((K >> 8) + 7) / 8)) * (0.85 + 0.17 * r);
+        const double t_gemv = 3.0 + (double)N * (double)(K >> 2) / 8.0e6 + (double)((M + 15) / 16) * t_pass;
         if (t_gemm < t_gemv) return kInt8Gemm;
     }
     return kInt8Gemv;
@@ -512,26 +533,17 @@ int launch_int8g(const void *x, const void *codes, const void *cb, void *out, in
                   (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
 }
 
-// one launch for up to 16 rows of x; first / last: position in the operator call's sequence of
-// launches, for the timing events
+// any number of rows of x, 16 per pass
 template <bool kTiled>
 int run_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
-              bool first, bool last, hipStream_t stream)
+              hipStream_t stream)
 {
-    // row block = the workgroup's share of tiles when that is one to four, else the size that needs
-    // the fewest blocks (x is fetched once per row block), as for the half-precision kernel
-    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;
-    int best = 1;
-    for (int r = 2; r <= 4; r++)
-        if ((share + r - 1) / r < (share + best - 1) / best) best = r;
-#define DMM_I8X(RR)                                                                                         \
-    (first ? (last ? launch_int8x<RR, kTiled, true, true>(x, codes, cb, out, M, N, K, stream)               \
-                   : launch_int8x<RR, kTiled, true, false>(x, codes, cb, out, M, N, K, stream))              \
-           : (last ? launch_int8x<RR, kTiled, false, true>(x, codes, cb, out, M, N, K, stream)              \
-                   : launch_int8x<RR, kTiled, false, false>(x, codes, cb, out, M, N, K, stream)))
-    return best == 1 ? DMM_I8X(1) : best == 2 ? DMM_I8X(2) : best == 3 ? DMM_I8X(3) : DMM_I8X(4);
-#undef DMM_I8X
+    switch (small_batch_row_block((N + 15) / 16, cu_count())) {
+        case 1: return launch_int8x<1, kTiled>(x, codes, cb, out, M, N, K, stream);
+        case 2: return launch_int8x<2, kTiled>(x, codes, cb, out, M, N, K, stream);
+        case 3: return launch_int8x<3, kTiled>(x, codes, cb, out, M, N, K, stream);
+        default: return launch_int8x<4, kTiled>(x, codes, cb, out, M, N, K, stream);
+    }
 }
 
 // CU count for the pure queries (kernel names, workspace size), which must answer without a

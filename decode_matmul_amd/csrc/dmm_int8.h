@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x,
 }
 
 // ------------------------------------------------------------------ the integer operator on the matrix unit
-// M <= 16, K a multiple of 256, a table whose bytes are all 2 mod 4 (see int8_rows): the
+// K a multiple of 256, a table whose bytes are all 2 mod 4 (see int8_rows): the
 // small-batch kernel's structure (persistent workgroups over contiguous ranges of 16-row tiles,
 // k steps of 256 dealt to 8 waves, x fetched from L2 into registers with the codes as one
 // prefetch unit, partial sums through LDS) with the decode done in bytes - one 8-byte gather of
@@ -149,7 +149,8 @@ __global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x,
 // there 16 bytes hold codes (row g, columns c .. c + 3) interleaved with row g + 8's, so lanes g
 // and g + 8 load the same two pieces and each keeps its halves (one v_perm per two codes).
 // A table with any other byte is found while the tables are built, and the workgroup then does
-// its rows with the scalar decode instead.
+// its rows with the scalar decode instead.  More than 16 rows of x: a row block is walked once
+// per 16 rows (a pass), so the codes come from HBM once and from the caches after that.
 typedef int i4_t __attribute__((ext_vector_type(4)));
 constexpr int kI8TableBytes = 256 * 256;   // one table: 256 rows x 32 copies x 8 bytes
 
@@ -198,18 +199,21 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 #pragma unroll
     for (int r = 0; r < R; r++)
         voff[r] = kTiled ? r * 16 * row_bytes + q * 256 + (c16 & 7) * 16 : (16 * r + c16) * row_bytes + q * 16;
-    const int xoff = c16 < M ? c16 * K + 64 * q : kOut;   // columns past M: zeros, no memory access
+    // pass p adds 16 p rows; rows past M lie past the end of the buffer: zeros, no memory access
+    const int xoff = c16 * K + 64 * q;
+    const int n_pass = (M + 15) >> 4;
+    const int pass_bytes = 16 * K;
     const uint32_t half_sel = (c16 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
 
     struct Unit {
         u4_t cw[R][kTiled ? 2 : 1];
         u4_t xb[4];
     };
-    int pf_blk = 0, pf_j = 0;
+    int pf_blk = 0, pf_pass = 0, pf_j = 0;
     auto issue = [&](Unit &u) {
         const bool ok = pf_blk < nb_wg && n_sw > 0;
         const int step = wave + pf_j * W;
-        const int xs_off = ok ? step * 256 : kOut;
+        const int xs_off = ok ? step * 256 + pf_pass * pass_bytes : kOut;
         const int tb = t0 + pf_blk * R;
         const int soff = !ok ? kOut : kTiled ? tb * 16 * row_bytes + step * 1024 : tb * 16 * row_bytes + step * 64;
 #pragma unroll
@@ -220,7 +224,10 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
             u.cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r], so, 0);
             if (kTiled) u.cw[r][kTiled ? 1 : 0] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff[r] + 128, so, 0);
         }
-        if (++pf_j >= n_sw) { pf_j = 0; pf_blk++; }
+        if (++pf_j >= n_sw) {
+            pf_j = 0;
+            if (++pf_pass >= n_pass) { pf_pass = 0; pf_blk++; }
+        }
     };
 
     Unit ring[D];
@@ -270,8 +277,9 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = i4_t{0, 0, 0, 0};
 
-    auto finish_block = [&](int blk) {
-        const int par = kTwoBuffers ? blk & 1 : 0;
+    int n_done = 0;   // passes over row blocks finished so far: the partial-sum buffers take turns
+    auto finish_block = [&](int blk, int pass) {
+        const int par = kTwoBuffers ? n_done++ & 1 : 0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
             red[par][wave][r][lane] = acc[r][0] + acc[r][1];
@@ -284,18 +292,20 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
             for (int w = 1; w < W; w++) sacc += red[par][w][r][lane];
             const int rt = t0 + blk * R + r;
             const int n = rt * 16 + 4 * q;
-            if (c16 < M && rt < t1 && n < N)   // N % 4 == 0, so the four rows are in range together
-                *reinterpret_cast<i4_t *>(out + (int64_t)c16 * N + n) = sacc;
+            const int m = 16 * pass + c16;
+            if (m < M && rt < t1 && n < N)   // N % 4 == 0, so the four rows are in range together
+                *reinterpret_cast<i4_t *>(out + (int64_t)m * N + n) = sacc;
         }
         if (!kTwoBuffers) __syncthreads();   // the next block's sums go to the same buffer
     };
 
     if (n_sw == 0) {
-        for (int blk = 0; blk < nb_wg; blk++) finish_block(blk);
+        for (int blk = 0; blk < nb_wg; blk++)
+            for (int pass = 0; pass < n_pass; pass++) finish_block(blk, pass);
         return;
     }
-    const int n_items = nb_wg * n_sw;
-    int blk = 0, j = 0;
+    const int n_items = nb_wg * n_pass * n_sw;
+    int blk = 0, pass = 0, j = 0;
     for (int i0 = 0; i0 < n_items; i0 += D) {
 #pragma unroll
         for (int d = 0; d < D; d++) {
@@ -331,8 +341,8 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
                 }
                 if (++j >= n_sw) {
                     j = 0;
-                    finish_block(blk);
-                    blk++;
+                    finish_block(blk, pass);
+                    if (++pass >= n_pass) { pass = 0; blk++; }
                 }
             }
             issue(ring[d]);

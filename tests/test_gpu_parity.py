@@ -471,14 +471,18 @@ def test_integer_operator_table_bytes_2_mod_4(M, N, K, tiled, x_off):
     (5, 8192 + 16, 1024, True, "any"), (3, 52, 2048, False, "any"), (16, 4096, 4096, False, "e8p"),
     # workgroup shares of 3, 4, 7 and 5 tiles: row blocks of three and four tiles, partial last blocks
     (8, 16 * (256 * 3 - 10), 256, True, "e8p"), (16, 16 * (256 * 4 - 3), 256, False, "mod4"),
-    (8, 28672, 256, True, "e8p"), (4, 16 * (256 * 5 - 1), 512, True, "any")])
+    (8, 28672, 256, True, "e8p"), (4, 16 * (256 * 5 - 1), 512, True, "any"),
+    # more than 16 rows of x in passes of the one launch, a last pass with rows to spare
+    (24, 16 * 130, 2048, True, "e8p"), (33, 1028, 8192, False, "mod4"), (64, 4096, 4096, True, "e8p"),
+    (100, 2052, 1024, False, "any"), (48, 16 * (256 * 3 - 10), 512, True, "mod4")])
 def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     """K a multiple of 256 with 16-byte aligned buffers runs on v_mfma_i32_16x16x64_i8: one or
-    several tiles per workgroup with partial last blocks, more than 16 rows of x (several
-    launches), both code layouts, N no multiple of 16 (row-major), and a table with bytes that are
-    not 2 mod 4, which every workgroup must notice and serve with the scalar decode.  Exact
-    against the oracle's restatement of /root/reference/test_decode_matmul.py:58-71."""
-    assert capi.lib().dmm_integer_kernel_name(M, N, K) in (b"dmm::int8x_kernel", b"dmm::int8g_kernel")
+    several tiles per workgroup with partial last blocks, more than 16 rows of x (passes over
+    the row blocks inside the one launch), both code layouts, N no multiple of 16 (row-major),
+    and a table with bytes that are not 2 mod 4, which every workgroup must notice and serve
+    with the scalar decode.  Exact against the oracle's restatement of
+    /root/reference/test_decode_matmul.py:58-71."""
+    assert capi.lib().dmm_integer_kernel_name(M, N, K) == b"dmm::int8x_kernel"
     rng = np.random.default_rng(M * 977 + N + K)
     if table == "e8p":
         cb = orc.build_codebook_abs()
