@@ -77,12 +77,13 @@ const std::vector<KernelInfo> &kernel_table()
         kinfo(gemm_reg_kernel<2, true, P>, gr_smem_bytes(2), true), kinfo(gemm_reg_kernel<4, true, P>, gr_smem_bytes(4), true)
         DMM_BOTH_LAYOUTS(DMM_K_GREG),
         kinfo(gemm_kernel<4, 2, 2, 2>, (int)sizeof(GemmCfg<4, 2, 2, 2>::Shared), false),
-#define DMM_K_I8X(T)                                                                                         \
-    kinfo(int8x_kernel<1, 8, 2, T>, kLdsMax, true), kinfo(int8x_kernel<2, 8, 2, T>, kLdsMax, true),                    \
-        kinfo(int8x_kernel<3, 8, 2, T>, kLdsMax, true), kinfo(int8x_kernel<4, 8, 2, T>, kLdsMax, true),                \
-        kinfo(int8g_kernel<T>, kI8gSmem, true)
+#define DMM_K_I8X_S(T, S)                                                                                    \
+    kinfo(int8x_kernel<1, 8, 2, T, S>, kLdsMax, true), kinfo(int8x_kernel<2, 8, 2, T, S>, kLdsMax, true),              \
+        kinfo(int8x_kernel<3, 8, 2, T, S>, kLdsMax, true), kinfo(int8x_kernel<4, 8, 2, T, S>, kLdsMax, true)
+#define DMM_K_I8X(T) DMM_K_I8X_S(T, false), DMM_K_I8X_S(T, true), kinfo(int8g_kernel<T>, kI8gSmem, true)
         DMM_BOTH_LAYOUTS(DMM_K_I8X),
 #undef DMM_K_I8X
+#undef DMM_K_I8X_S
 #undef DMM_K_GREG
 #undef DMM_K_REGX
 #undef DMM_K_REGX_XI
@@ -480,28 +481,39 @@ int run_generic(const void *x, const void *codes, const void *grid, float scale,
                   (const uint16_t *)codes, grid, scale, (uint16_t *)y, M, N, K);
 }
 
+template <int R, bool kTiled, bool kSlice>
+int launch_int8x_s(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+                   hipStream_t stream)
+{
+    constexpr int W = 8, D = 2;
+    const size_t shmem = (size_t)2 * kI8TableBytes + W * kI8xPiece;
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(int8x_kernel<R, W, D, kTiled, kSlice>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream,
+                  (const int8_t *)x, (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K,
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+// More than 8 rows of x: the slice of a step goes through the LDS (graph launches, us, fragment loads /
+// slice: M = 16 28672 -> 8192 20.5 / 17.1, 11008 -> 4096 9.3 / 7.5; M = 64 67.0 / 54.1, 25.4 / 16.9; but
+// M = 1 13.9 / 17.0, 6.5 / 7.6, and level at M = 8).
 template <int R, bool kTiled>
 int launch_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
                  hipStream_t stream)
 {
-    constexpr int W = 8, D = 2;
-    const size_t shmem = (size_t)2 * kI8TableBytes + (R <= 2 ? 2 : 1) * W * R * kWave * 16;
-    const int64_t n_tiles = (N + 15) / 16;
-    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(int8x_kernel<R, W, D, kTiled>, dim3((unsigned)wgs), dim3(64 * W), shmem, stream, (const int8_t *)x,
-                  (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K,
-                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    return M > 8 ? launch_int8x_s<R, kTiled, true>(x, codes, cb, out, M, N, K, stream)
+                 : launch_int8x_s<R, kTiled, false>(x, codes, cb, out, M, N, K, stream);
 }
 
 // Which kernel the integer operator takes for 16-byte aligned buffers.  More than 16 rows of x are
 // passes of the matrix-vector kernel (16 rows each, the codes from the caches after the first) or one
 // launch of the matrix-matrix kernel; the cheaper estimate wins.  A pass costs each wave its k steps
-// (K / 256 over 8 waves, per row block) at 0.85 us + 0.17 us per row tile of the block; the
+// (K / 256 over 8 waves, per row block) at 0.35 us + 0.27 us per row tile of the block; the
 // matrix-matrix kernel K * 5.2 ns per round of one 256 x 128 tile per CU when few CUs have a tile,
 // rising to K * 8.8 ns with all of them busy (the clock drops).  Graph launches, us, passes /
-// matrix-matrix: 4096 x 4096 M = 128 20.2 / 29.5, M = 256 36.2 / 30.2; 11008 -> 4096 M = 128 48.6 / 63.1,
-// M = 256 90.2 / 63.9; 8192 -> 28672 M = 32 33.7 / 48.7, M = 64 54.5 / 48.6; 28672 -> 8192 M = 128
-// 131.6 / 149.3, M = 256 255.2 / 149.8.
+// matrix-matrix: 4096 x 4096 M = 256 28.5 / 30.3, M = 384 40.7 / 30.6; 11008 -> 4096 M = 256 60.1 / 63.5,
+// M = 384 86.3 / 64.1; 8192 -> 28672 M = 32 32.6 / 49.2, M = 64 54.7 / 48.7; 28672 -> 8192 M = 128
+// 111.5 / 148.7, M = 192 158.0 / 149.5.
 enum Int8Kind { kInt8Scalar, kInt8Gemv, kInt8Gemm };
 Int8Kind pick_int8(int64_t M, int64_t N, int64_t K, int cus)
 {
@@ -517,8 +529,8 @@ Int8Kind pick_int8(int64_t M, int64_t N, int64_t K, int cus)
         }
         int64_t blocks = 1;
         const int r = small_batch_row_block((N + 15) / 16, cus, &blocks);
-        const double t_pass = (double)(blocks * (((K >> 8) + 7) / 8)) * (0.85 + 0.17 * r);
-        const double t_gemv = 3.0 + (double)N * (double)(K >> 2) / 8.0e6 + (double)((M + 15) / 16) * t_pass;
+        const double t_pass = (double)(blocks * (((K >> 8) + 7) / 8)) * (0.35 + 0.27 * r);
+        const double t_gemv = 3.0 + (double)N * (double)(K >> 2) / 7.0e6 + (double)((M + 15) / 16) * t_pass;
         if (t_gemm < t_gemv) return kInt8Gemm;
     }
     return kInt8Gemv;

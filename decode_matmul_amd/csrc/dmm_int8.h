@@ -138,8 +138,11 @@ __global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x,
 // ------------------------------------------------------------------ the integer operator on the matrix unit
 // K a multiple of 256, a table whose bytes are all 2 mod 4 (see int8_rows): the
 // small-batch kernel's structure (persistent workgroups over contiguous ranges of 16-row tiles,
-// k steps of 256 dealt to 8 waves, x fetched from L2 into registers with the codes as one
-// prefetch unit, partial sums through LDS) with the decode done in bytes - one 8-byte gather of
+// k steps of 256 dealt to 8 waves, the x slice of a step fetched from L2 with the codes as one
+// prefetch unit - in whole lines, four rows of 256 bytes per load instruction - and turned into
+// fragments through a 4 KB piece of LDS that belongs to the wave alone, the 16-byte pieces of row m
+// exchanged by m % 16 so that neither the writes nor the reads meet a bank conflict; the same pieces
+// carry the partial sums at the end of a row block) with the decode done in bytes - one 8-byte gather of
 // the table entry by the code's low byte, one of the mask by its high byte, exclusive or - and
 // v_mfma_i32_16x16x64_i8: a lane's 8 codes of a step are the A operands of four MFMAs (two codes =
 // 16 k each), B is 16 bytes of x per lane and MFMA.  Both tables hold 32 copies of every 8-byte
@@ -154,19 +157,19 @@ __global__ __launch_bounds__(256) void int8_kernel(const int8_t *__restrict__ x,
 typedef int i4_t __attribute__((ext_vector_type(4)));
 constexpr int kI8TableBytes = 256 * 256;   // one table: 256 rows x 32 copies x 8 bytes
 
-template <int R, int W, int D, bool kTiled>
+constexpr int kI8xPiece = 4096;   // LDS bytes of a wave's own piece: 16 rows x 256 bytes
+
+// kSlice: the x of a step through the wave's piece as above (pays from about 8 rows of x on); else
+// every lane loads its own four fragments, which for a row or two of x is the cheaper way
+template <int R, int W, int D, bool kTiled, bool kSlice>
 __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
                                                        const int64_t *__restrict__ codebook_abs,
                                                        int32_t *__restrict__ out, int M, int N, int K, int tiles_q,
                                                        int tiles_r)
 {
     static_assert(W == 8, "the table staging below assumes 512 threads");
+    static_assert(R * kWave * 16 <= kI8xPiece, "the partial sums of a row block go through the wave's piece");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    // partial sums: two buffers taken in turn while they fit beside the tables (R <= 2), else one
-    // and a second barrier per row block
-    constexpr bool kTwoBuffers = R <= 2;
-    typedef i4_t red_t[W][R][kWave];
-    red_t *red = reinterpret_cast<red_t *>(smem_raw + 2 * kI8TableBytes);   // red[parity]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -199,15 +202,23 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 #pragma unroll
     for (int r = 0; r < R; r++)
         voff[r] = kTiled ? r * 16 * row_bytes + q * 256 + (c16 & 7) * 16 : (16 * r + c16) * row_bytes + q * 16;
-    // pass p adds 16 p rows; rows past M lie past the end of the buffer: zeros, no memory access
-    const int xoff = c16 * K + 64 * q;
+    // load i of a step is piece lane % 16 (16 bytes) of row 4 i + lane / 16 of the slice; pass p adds
+    // 16 p rows; rows past M lie past the end of the buffer: zeros, no memory access
+    int xcoff[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) xcoff[i] = kSlice ? (4 * i + q) * K + c16 * 16 : c16 * K + 64 * q + 16 * i;
     const int n_pass = (M + 15) >> 4;
     const int pass_bytes = 16 * K;
+    // the wave's piece of LDS: row m at m * 256, its piece p in slot p ^ m.  Writes: row 4 i + h, piece
+    // lane % 16, h = lane / 16, i.e. (xs_w ^ 64 i) + 1024 i.  Reads: row c16, piece 4 q + t, i.e. xs_r ^ 16 t.
+    const uint32_t xs_piece = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + wave * kI8xPiece);
+    const uint32_t xs_w = xs_piece + (uint32_t)(q * 256 + ((c16 ^ q) << 4));
+    const uint32_t xs_r = xs_piece + (uint32_t)(c16 * 256 + (((4 * q) ^ c16) << 4));
     const uint32_t half_sel = (c16 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
 
     struct Unit {
         u4_t cw[R][kTiled ? 2 : 1];
-        u4_t xb[4];
+        u4_t xs[4];   // the slice as loaded, or the lane's four fragments
     };
     int pf_blk = 0, pf_pass = 0, pf_j = 0;
     auto issue = [&](Unit &u) {
@@ -217,7 +228,7 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
         const int tb = t0 + pf_blk * R;
         const int soff = !ok ? kOut : kTiled ? tb * 16 * row_bytes + step * 1024 : tb * 16 * row_bytes + step * 64;
 #pragma unroll
-        for (int t = 0; t < 4; t++) u.xb[t] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff + t * 16, xs_off, 0);
+        for (int i = 0; i < 4; i++) u.xs[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff[i], xs_off, 0);
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int so = (r == 0 || tb + r < t1) ? soff : kOut;
@@ -256,15 +267,15 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 #pragma unroll
         for (int i = 0; i < 16; i++) lds_write16(rowp ^ (uint32_t)(i * 16), u4_t{lo, hi, lo, hi});
     }
-    // the vote on the table: one word per wave in the partial-sum area, read by everybody after the barrier
+    // the vote on the table: one word per wave in the area of the pieces, read by everybody after the barrier
     uint32_t *votes = reinterpret_cast<uint32_t *>(smem_raw + 2 * kI8TableBytes);
     const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
     if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
     __syncthreads();
     const bool any_bad = __builtin_amdgcn_ballot_w64(votes[lane & (W - 1)] != 0) != 0;
-    __syncthreads();   // the votes are read before partial sums overwrite them
+    __syncthreads();   // the votes are read before the first slice of x overwrites them
     if (any_bad) {
-        // scalar decode for this workgroup's rows; the raw table goes where the partial sums would
+        // scalar decode for this workgroup's rows; the raw table goes where the pieces would
         uint64_t *table = reinterpret_cast<uint64_t *>(smem_raw + 2 * kI8TableBytes);
         if (tid < 256) table[tid] = entry;
         __syncthreads();
@@ -277,26 +288,29 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = i4_t{0, 0, 0, 0};
 
-    int n_done = 0;   // passes over row blocks finished so far: the partial-sum buffers take turns
+    // end of a pass over a row block: every wave leaves its partial sums in its own piece (row tile
+    // r at lane l: byte (r * 64 + l) * 16), one barrier, the first R waves add up one row tile each
+    // and store it, and a second barrier, because the pieces take the x of the next pass next
     auto finish_block = [&](int blk, int pass) {
-        const int par = kTwoBuffers ? n_done++ & 1 : 0;
+        i4_t *own = reinterpret_cast<i4_t *>(smem_raw + 2 * kI8TableBytes + wave * kI8xPiece);
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            red[par][wave][r][lane] = acc[r][0] + acc[r][1];
+            own[r * kWave + lane] = acc[r][0] + acc[r][1];
             acc[r][0] = acc[r][1] = i4_t{0, 0, 0, 0};
         }
         __syncthreads();
         for (int r = wave; r < R; r += W) {
-            i4_t sacc = red[par][0][r][lane];
+            const i4_t *src = reinterpret_cast<const i4_t *>(smem_raw + 2 * kI8TableBytes) + r * kWave + lane;
+            i4_t sacc = src[0];
 #pragma unroll
-            for (int w = 1; w < W; w++) sacc += red[par][w][r][lane];
+            for (int w = 1; w < W; w++) sacc += src[w * (kI8xPiece / 16)];
             const int rt = t0 + blk * R + r;
             const int n = rt * 16 + 4 * q;
             const int m = 16 * pass + c16;
             if (m < M && rt < t1 && n < N)   // N % 4 == 0, so the four rows are in range together
                 *reinterpret_cast<i4_t *>(out + (int64_t)m * N + n) = sacc;
         }
-        if (!kTwoBuffers) __syncthreads();   // the next block's sums go to the same buffer
+        __syncthreads();
     };
 
     if (n_sw == 0) {
@@ -312,6 +326,17 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
             if (i0 + d < n_items) {
                 const Unit &u = ring[d];
                 const int nv = t1 - (t0 + blk * R);   // tiles of this block that are ours (uniform)
+                u4_t xf[4];
+                if constexpr (kSlice) {
+                    // the slice through the wave's piece: in as loaded, out as fragments
+#pragma unroll
+                    for (int i = 0; i < 4; i++) lds_write16((xs_w ^ (uint32_t)(64 * i)) + (uint32_t)(1024 * i), u.xs[i]);
+#pragma unroll
+                    for (int t = 0; t < 4; t++) xf[t] = lds_read16(xs_r ^ (uint32_t)(16 * t));
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) xf[t] = u.xs[t];
+                }
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     if (r > 0 && r >= nv) break;
@@ -336,7 +361,7 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
                     for (int i = 0; i < 4; i++) {
                         const i4_t a = i4_t{(int)(g[2 * i][0] ^ m[2 * i][0]), (int)(g[2 * i][1] ^ m[2 * i][1]),
                                             (int)(g[2 * i + 1][0] ^ m[2 * i + 1][0]), (int)(g[2 * i + 1][1] ^ m[2 * i + 1][1])};
-                        acc[r][i & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, __builtin_bit_cast(i4_t, u.xb[i]), acc[r][i & 1], 0, 0, 0);
+                        acc[r][i & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, __builtin_bit_cast(i4_t, xf[i]), acc[r][i & 1], 0, 0, 0);
                     }
                 }
                 if (++j >= n_sw) {

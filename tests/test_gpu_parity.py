@@ -502,7 +502,7 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
 @pytest.mark.parametrize("M,N,K,tiled,table", [
     (128, 32768, 256, True, "e8p"), (300, 16 * 1030, 512, False, "mod4"), (64, 40000, 256, False, "any"),
     (2048, 4096, 512, True, "e8p"), (200, 16 * 1030, 1280, True, "mod4"), (129, 16 * 1030, 256, True, "any"),
-    (256, 4096, 4096, True, "e8p"), (512, 2048, 8192, False, "mod4"),
+    (384, 4096, 4096, True, "e8p"), (512, 2048, 8192, False, "mod4"),
     (512, 2048, 768, False, "e8p"), (384, 4096, 2304, True, "mod4"), (640, 8192, 1536, True, "e8p")])
 def test_integer_operator_matrix_matrix(M, N, K, tiled, table):
     """Many rows of x run on the int8 matrix-matrix kernel: partial tiles in M and N, both code layouts, 4 to 128 k tiles
