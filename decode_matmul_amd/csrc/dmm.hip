@@ -236,7 +236,8 @@ int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *
     const bool rows_ok = gemv_rows_ok(x, packed, grid, y, M, N, K);   // more than 32 rows, 16 at a time
     if (!mm_ok && !rows_ok) return DMM_ERR_UNSUPPORTED;
     if ((st = ensure_ready(s))) return st;
-    if (workspace && workspace_bytes > 0 && mm_ok && M >= kSplitKMinM && aligned(y, 8)) {
+    if (workspace && workspace_bytes > 0 && mm_ok && M >= kSplitKMinM && aligned(y, 8) &&
+        !(passes_beat_splitk(M, N, K) && mv_ok)) {
         const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
         if (splits >= 2) return launch_gemm_splitk<true>(x, packed, grid, scale, y, workspace, splits, M, N, K, s);
     }
@@ -292,6 +293,7 @@ int64_t dmm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 {
     if (M < 1 || N < 1 || K < kGrBK || (K & 63) || M < kSplitKMinM || M > 65535LL * 128 || !gemm_reg_ok(M, N, K))
         return 0;
+    if (passes_beat_splitk(M, N, K)) return 0;   // the small-batch kernel takes it, without a workspace
     const int splits = splitk_plan(M, N, K, INT64_MAX, cu_count_or_default());
     return splits >= 2 ? (int64_t)splits * M * N * 4 : 0;
 }

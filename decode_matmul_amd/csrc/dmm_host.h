@@ -442,6 +442,15 @@ bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
 // matrix-vector kernels are as fast or faster).
 constexpr int kSplitKMinM = 17;
 
+// 17 .. 32 rows of x on a code matrix of up to 17 MB: two passes of the small-batch kernel beat the split
+// and its second launch, so such a shape asks for no workspace and ignores one (graph launches, us, split /
+// passes, M = 32: 4096 -> 11008 15.8 / 13.8, 11008 -> 4096 18.3 / 15.8, 8192 -> 8192 18.2 / 16.8; but
+// 8192 -> 10240 20.4 / 20.6, 8192 -> 28672 31.7 / 42.0; M = 48 at 4096 -> 11008 19.0 / 18.0, 64 20.2 / 22.3)
+inline bool passes_beat_splitk(int64_t M, int64_t N, int64_t K)
+{
+    return M <= 32 && K >= 256 && (K & 255) == 0 && (N & 3) == 0 && N * (K >> 2) <= (17LL << 20);
+}
+
 bool splitk_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
                int64_t K)
 {
@@ -586,7 +595,8 @@ bool passes_beat_gemm(int64_t M, int64_t N, int64_t K, int cus)
 int dispatch_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M, int64_t N,
                  int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
-    if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K)) {
+    if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K) &&
+        !(passes_beat_splitk(M, N, K) && gemv_ok(x, codes, grid, y, M, N, K))) {
         const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
         if (splits >= 2) return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, s);
     }

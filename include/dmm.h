@@ -93,8 +93,9 @@ int dmm_decode_matmul_f16(const void *x, const void *codes, const void *grid, fl
  * blocks per tile, each writes fp32 partial sums to the workspace and a second small kernel
  * adds them in a fixed order (results stay bit-reproducible), scales and rounds into y.
  *   dmm_workspace_bytes  the size that lets the call split as far as it would like to
- *                        (0: this shape never uses a workspace); any smaller size is legal
- *                        and only limits the split.
+ *                        (0: this shape never uses a workspace - among others up to 32 rows
+ *                        of x on up to 17 MB of codes, which the small-batch kernel serves
+ *                        faster); any smaller size is legal and only limits the split.
  *   workspace            device memory, 16-byte aligned, owned by the caller; it must not be
  *                        used by another call that may run at the same time (other stream).
  *                        NULL or workspace_bytes == 0: identical to dmm_decode_matmul_f16. */
