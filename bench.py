@@ -66,6 +66,8 @@ def parse():
                     help="run only the M = 2048 leg and print its object (for profiling the matrix-matrix kernel)")
     ap.add_argument("--integer-only", action="store_true",
                     help="run only the integer-operator leg and print its object (for profiling that kernel)")
+    ap.add_argument("--small-batch-only", action="store_true",
+                    help="run only the two small-batch legs and print their objects (for profiling the small-batch kernel)")
     ap.add_argument("--rotate-mb", type=int, default=400, help="distinct code bytes to rotate through, at least")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch 8 plain device copies of 256 MiB first (a known-size reference for scaling "
@@ -121,6 +123,12 @@ def main():
 
     if args.integer_only:
         print(json.dumps({"integer_operator": integer_operator(torch, lib, capi, workload, dev, stream, rand_codes)}))
+        return
+
+    if args.small_batch_only:
+        print(json.dumps({"small_batch": small_batch(torch, lib, capi, workload, dev, stream, rand_codes),
+                          "small_batch_70b": small_batch(torch, lib, capi, workload, dev, stream, rand_codes,
+                                                         shapes=workload.LLAMA2_70B, batches=(2, 4, 8, 16))}))
         return
 
     # ---------------------------------------------------------------- headline: 70B GEMV
