@@ -18,6 +18,7 @@
 //   dmm_tables.h      decode tables, decode of one code, standalone decoder, catch-all operator
 //   dmm_gemv_f16.h    matrix-vector helpers and the streaming kernel on 16-bit operands
 //   dmm_gemv_q8.h     matrix-vector kernels on 8-bit operands (fp8 weights, bf8 terms of x)
+//   dmm_gemv_q8d.h    batch 1 on 8-bit operands, every tile of a workgroup in registers
 //   dmm_gemv_small.h  small-batch kernel with x in registers
 //   dmm_gemm.h        matrix-matrix kernels and the split-K reduction
 //   dmm_int8.h        the reference's integer operator
@@ -53,6 +54,7 @@ constexpr int kWave = 64;
 #include "dmm_tables.h"
 #include "dmm_gemv_f16.h"
 #include "dmm_gemv_q8.h"
+#include "dmm_gemv_q8d.h"
 #include "dmm_gemv_small.h"
 #include "dmm_gemm.h"
 #include "dmm_int8.h"
@@ -172,7 +174,7 @@ const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K)
     if (M > 16) return "dmm::gemv_regx_kernel";
     switch (pick_gemv(M, N, K)) {
         case kGemvStream: return "dmm::gemv_stream_kernel";
-        case kGemvQ8: return M == 1 ? "dmm::gemv_q8c_kernel" : "dmm::gemv_q8_kernel";
+        case kGemvQ8: return M > 1 ? "dmm::gemv_q8_kernel" : gemv_q8d_ok(N) ? "dmm::gemv_q8d_kernel" : "dmm::gemv_q8c_kernel";
         default: return "dmm::gemv_regx_kernel";
     }
 }

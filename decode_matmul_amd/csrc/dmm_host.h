@@ -66,6 +66,11 @@ const std::vector<KernelInfo> &kernel_table()
         DMM_BOTH_LAYOUTS(DMM_K_STREAM),
 #define DMM_K_Q8(P) kinfo(gemv_q8_kernel<1, 16, 2, P>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P>, kLdsMax, true), kinfo(gemv_q8c_kernel<3, 1, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_Q8),
+#define DMM_K_Q8D(P)                                                                                             \
+    kinfo(gemv_q8d_kernel<1, 2, 2, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<2, 2, 4, P>, kLdsMax, true),         \
+        kinfo(gemv_q8d_kernel<3, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<4, 1, 4, P>, kLdsMax, true),     \
+        kinfo(gemv_q8d_kernel<6, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<8, 1, 4, P>, kLdsMax, true)
+        DMM_BOTH_LAYOUTS(DMM_K_Q8D),
 #define DMM_K_REGX_XI(P, XI)                                                                                      \
     kinfo(gemv_regx_kernel<1, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, P, XI>, kLdsMax, true),     \
         kinfo(gemv_regx_kernel<3, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 2, P, XI>, kLdsMax, true)
@@ -87,6 +92,7 @@ const std::vector<KernelInfo> &kernel_table()
 #undef DMM_K_GREG
 #undef DMM_K_REGX
 #undef DMM_K_REGX_XI
+#undef DMM_K_Q8D
 #undef DMM_K_Q8
 #undef DMM_K_STREAM
 #undef DMM_BOTH_LAYOUTS
@@ -250,6 +256,39 @@ int launch_gemv_q8c(const void *x, const void *codes, const void *grid, float sc
                   (int)(n_tiles % wgs));
 }
 
+// the resident-accumulator form: up to 8 tiles per workgroup, instantiated for 1, 2, 3, 4, 6 and 8
+inline bool gemv_q8d_ok(int64_t N) { return (N + 15) / 16 <= 8 * (int64_t)cu_count(); }
+
+template <int NT, int U, int D, bool kPacked>
+int launch_gemv_q8d_inst(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t N, int64_t K,
+                         hipStream_t stream)
+{
+    size_t shmem = (size_t)kSTablesBytes + stream_red_bytes(1, 16, 1) + (size_t)stream_x_bytes(1, K);   // the 16-bit hand-over
+    if (shmem < (size_t)qd_lds_bytes()) shmem = qd_lds_bytes();
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(gemv_q8d_kernel<NT, U, D, kPacked>, dim3((unsigned)wgs), dim3(1024), shmem, stream, (const uint16_t *)x,
+                  (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)N, (int)K, (int)(n_tiles / wgs),
+                  (int)(n_tiles % wgs));
+}
+
+template <bool kPacked>
+int launch_gemv_q8d(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t N, int64_t K,
+                    hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
+    switch (share) {
+        case 1: return launch_gemv_q8d_inst<1, 2, 2, kPacked>(x, codes, grid, scale, y, N, K, stream);
+        case 2: return launch_gemv_q8d_inst<2, 2, 4, kPacked>(x, codes, grid, scale, y, N, K, stream);
+        case 3: return launch_gemv_q8d_inst<3, 1, 3, kPacked>(x, codes, grid, scale, y, N, K, stream);
+        case 4: return launch_gemv_q8d_inst<4, 1, 4, kPacked>(x, codes, grid, scale, y, N, K, stream);
+        case 5:
+        case 6: return launch_gemv_q8d_inst<6, 1, 3, kPacked>(x, codes, grid, scale, y, N, K, stream);
+        default: return launch_gemv_q8d_inst<8, 1, 4, kPacked>(x, codes, grid, scale, y, N, K, stream);
+    }
+}
+
 template <int R, int W>
 bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
 {
@@ -293,6 +332,7 @@ template <bool kPacked>
 int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
                 int64_t N, int64_t K, hipStream_t stream)
 {
+    if (M == 1 && gemv_q8d_ok(N)) return launch_gemv_q8d<kPacked>(x, codes, grid, scale, y, N, K, stream);
     if (M == 1) return launch_gemv_q8c<kPacked>(x, codes, grid, scale, y, N, K, stream);
     const int64_t n_tiles = (N + 15) / 16;
     if (n_tiles > 2 * cu_count()) return launch_gemv_q8<1, 16, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);

@@ -296,11 +296,13 @@ def test_gemv_8bit_switch_and_kernel_name():
     ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)
     was = lib.dmm_set_gemv_8bit(1)
     try:
-        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_q8c_kernel"
-        assert lib.dmm_gemv_kernel_name(M, 8208, K) == b"dmm::gemv_q8c_kernel"        # more than two tiles per CU
+        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_q8d_kernel"
+        assert lib.dmm_gemv_kernel_name(M, 8208, K) == b"dmm::gemv_q8d_kernel"        # more than two tiles per CU
         assert lib.dmm_gemv_kernel_name(M, 8192, K) == b"dmm::gemv_stream_kernel"     # two, short x
-        assert lib.dmm_gemv_kernel_name(M, 8192, 12288) == b"dmm::gemv_q8c_kernel"    # two, long x
-        assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_q8c_kernel"       # x goes through in chunks
+        assert lib.dmm_gemv_kernel_name(M, 8192, 12288) == b"dmm::gemv_q8d_kernel"    # two, long x
+        assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_q8d_kernel"       # x goes through in chunks
+        assert lib.dmm_gemv_kernel_name(M, 32768, K) == b"dmm::gemv_q8d_kernel"       # eight tiles per CU
+        assert lib.dmm_gemv_kernel_name(M, 32784, K) == b"dmm::gemv_q8c_kernel"       # more: groups of three tiles
         assert lib.dmm_gemv_kernel_name(3, N, K) == b"dmm::gemv_q8_kernel"            # two to four rows of x
         assert lib.dmm_gemv_kernel_name(3, 12288, K) == b"dmm::gemv_stream_kernel"
         assert lib.dmm_gemv_kernel_name(3, N, 28672) == b"dmm::gemv_regx_kernel"      # their terms do not fit
@@ -374,7 +376,9 @@ def test_empty_problems():
 @pytest.mark.parametrize("path,M,N,K", [("gemv", 8, 16, 4096), ("gemm", 8, 16, 4096), ("generic", 8, 16, 4096),
                                          ("gemv", 1, 64, 8192), ("gemm", 64, 64, 8192),
                                          ("gemv8", 1, 64, 8192), ("gemv8", 1, 8192, 2048), ("gemv8", 3, 4100, 4096),
-                                         ("auto", 1, 16384, 4096)])
+                                         ("auto", 1, 16384, 4096),
+                                         ("gemv", 12, 4800, 5120), ("gemv", 16, 4112, 8192), ("gemv", 32, 1028, 8192),
+                                         ("auto", 64, 4096, 4096)])
 def test_integer_bridge_is_exact(path, M, N, K):
     """x integer-valued, grid = E8P bytes / 4, scale a power of two: every partial sum is a
     multiple of 1/4 below 2^24 quarters, so fp32 accumulation in any order is exact and the
@@ -387,9 +391,34 @@ def test_integer_bridge_is_exact(path, M, N, K):
     yi = orc.decode_matmul_i32(x, codes, cb)
     scale = 2.0 ** -8
     want = (yi.astype(np.float64) / 4 * scale).astype(np.float16)
+    if path == "gemv" and M >= 12:   # x too large for the LDS, or more than 16 rows of it: the small-batch kernel and its passes
+        assert capi.lib().dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_regx_kernel"
     y = c_matmul(dev(x.astype(np.float16)), dev(codes), dev(orc.grid_from_codebook(cb)), scale, path)
     torch.cuda.synchronize()
     assert np.array_equal(bits(y), bits(want))
+
+
+@pytest.mark.parametrize("N,K", [(4048, 1024), (8032, 4352), (12304, 12288), (16000, 768), (20000, 8192), (24592, 512),
+                                 (28000, 4096), (32768, 512), (33000, 768), (8192, 28672)])
+def test_gemv_8bit_every_share_of_tiles_is_exact(N, K):
+    """One row of x on the 8-bit kernels, exactly (the integer bridge): workgroups of one to eight row tiles
+    (every instantiation of the resident-accumulator kernel, with shares that differ by one between
+    workgroups), one to seven chunks of x with a last chunk that is not full, fewer k steps than waves, and
+    more than eight tiles per workgroup (the chunked kernel with its groups of three)."""
+    lib = capi.lib()
+    rng = np.random.default_rng(N + K)
+    cb = orc.build_codebook_abs()
+    x = rng.integers(-128, 128, size=(1, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    yi = orc.decode_matmul_i32(x, codes, cb)
+    scale = 2.0 ** -8
+    want = (yi.astype(np.float64) / 4 * scale).astype(np.float16)
+    y = c_matmul(dev(x.astype(np.float16)), dev(codes), dev(orc.grid_from_codebook(cb)), scale, "gemv8")
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), bits(want))
+    if (N + 15) // 16 > 2 * 256:
+        name = lib.dmm_gemv_kernel_name(1, N, K)
+        assert name == (b"dmm::gemv_q8d_kernel" if (N + 15) // 16 <= 8 * 256 else b"dmm::gemv_q8c_kernel")
 
 
 def test_reference_shape_golden_case():
