@@ -18,16 +18,23 @@
 //     dividing the U * NT items of the U-fold unrolled chunk loop, so slots and accumulators are
 //     static registers; an item is asked for D items ahead of its use.  Tiles past the workgroup's
 //     share and steps past K are out-of-range offsets: zeros, no memory access, no decode.
-//   * At the end every wave leaves columns 0 .. 3 of its accumulators in the LDS (in the tables'
-//     place), and wave t adds tile t up: four columns with their weights, then the 16 waves by DPP.
+//   * At the end every wave leaves columns 0 .. 3 of its accumulators in the LDS - in the x buffer that
+//     the last chunk does not use and the free space behind it, so nobody has to be waited for first -
+//     and after the launch's one closing barrier wave t adds tile t up: four columns with their weights,
+//     then the 16 waves by DPP.
 // The hand-over to the 16-bit kernel (a grid fp8 cannot hold, an x that is not finite) is the
 // chunked kernel's.
-// LDS map: tables [0, 96K), two x buffers (4 term rows, 2 rows of means, 64 zero bytes for the B
-// operands' idle columns), 16 vote words, 2 words for what the stagers find.
+// LDS map: tables [0, 96K), 16 vote words and 2 words for what the stagers find, two x buffers (4 term
+// rows, 2 rows of means, 64 zero bytes for the B operands' idle columns; chunk c sits in buffer
+// (n_chunks - 1 - c) % 2, the last one in buffer 0), and from buffer 1 on the partial sums of the end.
 constexpr int kQdXBuf = kQcXBuf + 64;
 constexpr int kQdRedWave = 4 * 4 * 16 + 16;        // 4 quarters x 4 columns of float4, padded: lane w of a reader hits bank group w
 constexpr int kQdRedTile = 16 * kQdRedWave;
-__host__ __device__ constexpr int qd_lds_bytes() { return kSTablesBytes + 2 * kQdXBuf + 128; }
+constexpr int kQdMaxTiles = 8;
+__host__ __device__ constexpr int qd_lds_bytes()
+{
+    return kSTablesBytes + 128 + kQdXBuf + (kQdXBuf > kQdMaxTiles * kQdRedTile ? kQdXBuf : kQdMaxTiles * kQdRedTile);
+}
 
 // qc_split_piece with the low half of the mean times 8 (exact: it lies 11 bits below the high half)
 __device__ __forceinline__ bool qd_split_piece(const u4_t &v, u2_t (&t)[4], uint32_t &mean_hi_lo8)
@@ -85,8 +92,9 @@ __global__ __launch_bounds__(1024) void gemv_q8d_kernel(const uint16_t *__restri
     constexpr int W = 16;
     static_assert((U * NT) % D == 0, "the ring has to divide the unrolled loop");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
-    unsigned char *xbuf = smem_raw + kSTablesBytes;
-    uint32_t *flags = reinterpret_cast<uint32_t *>(xbuf + 2 * kQdXBuf);   // [0 .. 15]: one vote per wave; [16], [17]: the stagers' finds
+    static_assert(NT <= kQdMaxTiles, "the partial sums of the end are sized for kQdMaxTiles tiles");
+    uint32_t *flags = reinterpret_cast<uint32_t *>(smem_raw + kSTablesBytes);   // [0 .. 15]: one vote per wave; [16], [17]: the stagers' finds
+    unsigned char *xbuf = smem_raw + kSTablesBytes + 128;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -168,7 +176,7 @@ __global__ __launch_bounds__(1024) void gemv_q8d_kernel(const uint16_t *__restri
 #pragma unroll
         for (int i = 0; i < 16; i++) lds_write16(gg ^ (uint32_t)(i * 16), u4_t{g8[0], g8[1], g8[0], g8[1]});
     } else {
-        fits = stage_piece(xpiece, 0, sp);   // pieces past the end of x are zeros
+        fits = stage_piece(xpiece, (n_chunks - 1) & 1, sp);   // pieces past the end of x are zeros
     }
     {
         const bool wave_bad = __builtin_amdgcn_ballot_w64(!fits) != 0;
@@ -201,7 +209,7 @@ __global__ __launch_bounds__(1024) void gemv_q8d_kernel(const uint16_t *__restri
             i8_t xb0 = i8_t{0, 0, 0, 0, 0, 0, 0, 0}, xb1 = xb0;
             h8_t xm = __builtin_bit_cast(h8_t, u4_t{0u, 0u, 0u, 0u});
             if (step_ok) {
-                const uint32_t bo = (uint32_t)((c & 1) * kQdXBuf);
+                const uint32_t bo = (uint32_t)(((n_chunks - 1 - c) & 1) * kQdXBuf);
                 const u4_t r0 = lds_read16(xt_off + bo), r1 = lds_read16(xt_off + bo + 16);
                 const u4_t r2 = lds_read16(xt_off + bo + 32), r3 = lds_read16(xt_off + bo + 48);
                 xm = __builtin_bit_cast(h8_t, lds_read16(xm_off + bo));
@@ -214,25 +222,27 @@ __global__ __launch_bounds__(1024) void gemv_q8d_kernel(const uint16_t *__restri
                 if (step_ok && t < nt) qd_tile_step(cw[slot], lane_base, xb0, xb1, xm, acc[t]);
                 issue(cw[slot], c + (t + D) / NT, (t + D) % NT);   // the item D further on
             }
-            if (stage_next && wave < 8 && !stage_piece(xpiece, (c + 1) & 1, sp)) flags[16 + (c & 1)] = 1u;
+            if (stage_next && wave < 8 && !stage_piece(xpiece, (n_chunks - 2 - c) & 1, sp)) flags[16 + (c & 1)] = 1u;
             if (stage_next) {
                 __syncthreads();   // hands the x buffer over
                 if (__builtin_amdgcn_ballot_w64(flags[16 + (c & 1)] != 0) != 0) hand_over = true;
             }
         }
     }
-    __syncthreads();   // everybody is through with the tables and x (or has read the flags)
+    // columns 0 .. 3 of every accumulator into the LDS, [tile][wave][quarter][column], from x buffer 1 on: the
+    // chunk that sat there has been read by everybody before the barrier that handed the last chunk over
+    const uint32_t red = lds_addr(xbuf) + (uint32_t)kQdXBuf;
+    if (!hand_over) {
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+            if (t < nt && c16 < 4)
+                lds_write16(red + (uint32_t)(t * kQdRedTile + wave * kQdRedWave + (q * 4 + c16) * 16), __builtin_bit_cast(u4_t, acc[t]));
+    }
+    __syncthreads();   // the launch's closing barrier: every partial sum is there (or everybody has read the flags)
     if (hand_over) {
         gemv_stream_body<1, W, 2, kPacked, 4>(x, codes, grid, scale, y, 1, N, K, tiles_q, tiles_r);
         return;
     }
-    // columns 0 .. 3 of every accumulator into the LDS, [tile][wave][quarter][column]
-    const uint32_t red = lds_addr(smem_raw);
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-        if (t < nt && c16 < 4)
-            lds_write16(red + (uint32_t)(t * kQdRedTile + wave * kQdRedWave + (q * 4 + c16) * 16), __builtin_bit_cast(u4_t, acc[t]));
-    __syncthreads();
     if (wave < nt) {
         // wave t adds up tile t: lane (w, quarter) takes wave w's 4 columns with their weights 8^-c, then
         // the 16 lanes of a row are added with DPP shifts
