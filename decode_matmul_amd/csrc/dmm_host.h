@@ -67,9 +67,9 @@ const std::vector<KernelInfo> &kernel_table()
 #define DMM_K_Q8(P) kinfo(gemv_q8_kernel<1, 16, 2, P>, kLdsMax, true), kinfo(gemv_q8_kernel<1, 16, 3, P>, kLdsMax, true), kinfo(gemv_q8c_kernel<3, 1, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_Q8),
 #define DMM_K_Q8D(P)                                                                                             \
-    kinfo(gemv_q8d_kernel<1, 2, 2, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<2, 2, 4, P>, kLdsMax, true),         \
-        kinfo(gemv_q8d_kernel<3, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<4, 1, 4, P>, kLdsMax, true),     \
-        kinfo(gemv_q8d_kernel<6, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<8, 1, 4, P>, kLdsMax, true)
+    kinfo(gemv_q8d_kernel<1, 2, 2, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<2, 1, 2, P>, kLdsMax, true),         \
+        kinfo(gemv_q8d_kernel<3, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<4, 1, 2, P>, kLdsMax, true),     \
+        kinfo(gemv_q8d_kernel<6, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<8, 1, 2, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_Q8D),
 #define DMM_K_REGX_XI(P, XI)                                                                                      \
     kinfo(gemv_regx_kernel<1, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, P, XI>, kLdsMax, true),     \
@@ -256,7 +256,11 @@ int launch_gemv_q8c(const void *x, const void *codes, const void *grid, float sc
                   (int)(n_tiles % wgs));
 }
 
-// the resident-accumulator form: up to 8 tiles per workgroup, instantiated for 1, 2, 3, 4, 6 and 8
+// the resident-accumulator form: up to 8 tiles per workgroup, instantiated for 1, 2, 3, 4, 6 and 8.  The ring
+// is two loads deep wherever two divides the tiles (measured as graph launches, two against four deep, us:
+// 8192 -> 28672 13.72 / 13.90, 28672 -> 8192 13.60 / 14.21, 8192 -> 8192 6.20 / 6.58, 8192 -> 16384 8.49 / 8.84,
+// 4096 -> 16384 5.88 / 6.23; eight deep 15.90 at 8192 -> 28672), three for three and six tiles (six tiles, two /
+// three / six deep: 8192 -> 24576 12.55 / 12.16 / 14.23, 4096 -> 22016 8.06 / 7.60 / 8.64)
 inline bool gemv_q8d_ok(int64_t N) { return (N + 15) / 16 <= 8 * (int64_t)cu_count(); }
 
 template <int NT, int U, int D, bool kPacked>
@@ -280,12 +284,12 @@ int launch_gemv_q8d(const void *x, const void *codes, const void *grid, float sc
     const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
     switch (share) {
         case 1: return launch_gemv_q8d_inst<1, 2, 2, kPacked>(x, codes, grid, scale, y, N, K, stream);
-        case 2: return launch_gemv_q8d_inst<2, 2, 4, kPacked>(x, codes, grid, scale, y, N, K, stream);
+        case 2: return launch_gemv_q8d_inst<2, 1, 2, kPacked>(x, codes, grid, scale, y, N, K, stream);
         case 3: return launch_gemv_q8d_inst<3, 1, 3, kPacked>(x, codes, grid, scale, y, N, K, stream);
-        case 4: return launch_gemv_q8d_inst<4, 1, 4, kPacked>(x, codes, grid, scale, y, N, K, stream);
+        case 4: return launch_gemv_q8d_inst<4, 1, 2, kPacked>(x, codes, grid, scale, y, N, K, stream);
         case 5:
         case 6: return launch_gemv_q8d_inst<6, 1, 3, kPacked>(x, codes, grid, scale, y, N, K, stream);
-        default: return launch_gemv_q8d_inst<8, 1, 4, kPacked>(x, codes, grid, scale, y, N, K, stream);
+        default: return launch_gemv_q8d_inst<8, 1, 2, kPacked>(x, codes, grid, scale, y, N, K, stream);
     }
 }
 
@@ -342,22 +346,23 @@ int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale,
 // whether an 8-bit kernel can take the shape at all (grid and x permitting, which the kernel finds out)
 bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok(M, N, K) : gemv_q8_ok<1, 16>(M, N, K); }
 
-// The choice among the matrix-vector kernels.  The 8-bit kernels where they apply and pay: one row of x
-// from more than two row tiles per workgroup on, and at exactly two for long x (measured as launches of
-// one HIP graph on rotating code buffers, the two kernels taking turns, 8-bit against 16-bit kernel, us
-// per launch: 8192 -> 10240 7.9 / 8.7, 8192 -> 9216 7.9 / 8.7, 8192 -> 28672 15.3 / 16.6, 4096 -> 22016
-// 8.7 / 10.9; two tiles: 28672 -> 8192 15.5 / 16.2, 16384 -> 8192 10.4 / 10.6, 12288 -> 8192 8.5 / 8.6,
-// 8192 -> 8192 7.0 / 7.0, 4096 -> 8192 5.3 / 5.3, 5120 -> 8192 6.2 / 5.7; below two tiles the 16-bit
-// kernel wins, 5120 -> 5120 6.2 / 5.6, 11008 -> 4096 6.9 / 5.5, its prologue being the cheaper one), two
-// to four rows from more than three tiles on.  A grid that does not fit fp8 costs them a second table
-// build, and the 16-bit kernel's y is the correctly rounded one.  Otherwise the 16-bit streaming
-// kernel, one tile at a time; the register-x kernel when x does not fit the LDS.
+// The choice among the matrix-vector kernels.  The 8-bit kernels where they apply and pay.  One row of x:
+// from more than one row tile per workgroup on, except for an x of two to three chunks whose last chunk is
+// short (8192 < K < 12288), which needs more than two tiles (measured as launches of one HIP graph on
+// rotating code buffers, 8-bit against 16-bit kernel, us per launch: 8192 -> 28672 14.0 / 16.6, 8192 -> 10240
+// 7.0 / 8.7, 28672 -> 8192 14.9 / 16.2, 28672 -> 6144 13.6 / 15.4, 8192 -> 8192 6.55 / 6.78, 8192 -> 4352 5.98 /
+// 6.69, 4096 -> 8192 5.01 / 5.44, 4096 -> 6144 4.96 / 5.41, 5120 -> 5120 5.40 / 5.69, 4096 -> 4608 4.86 / 5.39;
+// but 11008 -> 5120 7.90 / 7.71, 11008 -> 8192 8.60 / 8.01, and with one tile per workgroup 4096 -> 4096 4.46 /
+// 4.49, 11008 -> 4096 6.18 / 5.55).  Two to four rows from more than three tiles on.  A grid that does not
+// fit fp8 costs them a second table build, and the 16-bit kernel's y is the correctly rounded one.
+// Otherwise the 16-bit streaming kernel, one tile at a time; the register-x kernel when x does not fit
+// the LDS.
 enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
 
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const bool long_launch = M == 1 ? n_tiles > 2 * cus || (n_tiles == 2 * cus && K >= 12288) : n_tiles > 3 * cus;
+    const bool long_launch = M == 1 ? n_tiles > 2 * cus || (n_tiles > cus && (K <= 8192 || K >= 12288)) : n_tiles > 3 * cus;
     if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
     if (gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
     return kGemvRegx;
