@@ -84,6 +84,7 @@ const char *dmm_status_string(int status)
         case DMM_ERR_SCRATCH_TOO_SMALL:
             return "the split-K partial sums of this shape exceed the library's 16 MiB scratch buffer: use "
                    "dmm_decode_matmul_ws_f16 with a workspace of dmm_workspace_bytes, or dmm_decode_matmul_f16";
+        case DMM_ERR_HOST_MEMORY: return "host memory for a decoded row could not be allocated";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -239,7 +240,7 @@ int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *
     if (!mm_ok && !rows_ok) return DMM_ERR_UNSUPPORTED;
     if ((st = ensure_ready(s))) return st;
     if (workspace && workspace_bytes > 0 && mm_ok && M >= kSplitKMinM && aligned(y, 8) &&
-        !(passes_beat_splitk(M, N, K) && mv_ok)) {
+        !(passes_beat_splitk(M, N, K, cu_count()) && mv_ok)) {
         const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
         if (splits >= 2) return launch_gemm_splitk<true>(x, packed, grid, scale, y, workspace, splits, M, N, K, s);
     }
@@ -295,7 +296,7 @@ int64_t dmm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 {
     if (M < 1 || N < 1 || K < kGrBK || (K & 63) || M < kSplitKMinM || M > 65535LL * 128 || !gemm_reg_ok(M, N, K))
         return 0;
-    if (passes_beat_splitk(M, N, K)) return 0;   // the small-batch kernel takes it, without a workspace
+    if (passes_beat_splitk(M, N, K, cu_count_or_default())) return 0;   // the small-batch kernel takes it, without a workspace
     const int splits = splitk_plan(M, N, K, INT64_MAX, cu_count_or_default());
     return splits >= 2 ? (int64_t)splits * M * N * 4 : 0;
 }
@@ -334,18 +335,25 @@ int dmm_decode_matmul_host_f16(const void *x, const void *codes, const void *gri
     const int64_t kc = K >> 3;
     const half_t *xh = (const half_t *)x;
     half_t *yh = (half_t *)y;
+    std::atomic<int> failed{0};
+    std::atomic<int> *failed_p = &failed;
     host_parallel_rows(N, K * (M + 1), [=](int64_t n0, int64_t n1) {
-        std::vector<half_t> w((size_t)K);
+        half_t *w = (half_t *)malloc((size_t)K * sizeof(half_t));   // one decoded row
+        if (!w) {
+            failed_p->store(1, std::memory_order_relaxed);
+            return;
+        }
         for (int64_t n = n0; n < n1; n++) {
-            host_decode_row((const uint16_t *)codes + n * kc, (const half_t *)grid, kc, w.data());
+            host_decode_row((const uint16_t *)codes + n * kc, (const half_t *)grid, kc, w);
             for (int64_t m = 0; m < M; m++) {
                 float acc = 0.f;
-                for (int64_t k = 0; k < K; k++) acc += (float)xh[m * K + k] * (float)w[(size_t)k];
+                for (int64_t k = 0; k < K; k++) acc += (float)xh[m * K + k] * (float)w[k];
                 yh[m * N + n] = (half_t)(acc * scale);
             }
         }
+        free(w);
     });
-    return DMM_OK;
+    return failed.load(std::memory_order_relaxed) ? DMM_ERR_HOST_MEMORY : DMM_OK;
 }
 
 int dmm_read_probe(const void *codes, void *sink, int64_t N, int64_t K, void *stream)

@@ -406,7 +406,7 @@ constexpr int kQcChunkK = 4096;
 constexpr int kQcTermPitch = kQcChunkK + 16, kQcMeanPitch = kQcChunkK / 4 + 16;
 constexpr int kQcXBuf = 4 * kQcTermPitch + 2 * kQcMeanPitch;
 __host__ __device__ constexpr int qc_red_bytes(int T) { return 16 * (T * 16 + 1) * 16; }
-__host__ __device__ constexpr int qc_lds_bytes(int T) { return kSTablesBytes + qc_red_bytes(T) + 2 * kQcXBuf + 64; }
+__host__ __device__ constexpr int qc_lds_bytes(int T) { return kSTablesBytes + qc_red_bytes(T) + 2 * kQcXBuf + 128; }
 
 // the four bf8 terms of a piece of x (8 halves) and the mean of the 8 as hi + lo halves; returns
 // whether all 8 are finite (their fp32 sum is finite exactly when they all are)
@@ -445,7 +445,11 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
     f4_t *red = reinterpret_cast<f4_t *>(smem_raw + kSTablesBytes);
     unsigned char *xbuf = smem_raw + kSTablesBytes + qc_red_bytes(T);
-    uint32_t *flags = reinterpret_cast<uint32_t *>(xbuf + 2 * kQcXBuf);   // [0 .. 15]: one vote per wave; [0] doubles as the running flag
+    // [0 .. 15]: one prologue vote per wave.  [16], [17]: "an x staged later is not finite", the word of chunk gc
+    // being 16 + gc % 2: the stagers of chunk gc + 1 write the word nobody reads before the next barrier,
+    // while slower waves may still be reading the word of chunk gc.  A word once set ends the loop for
+    // every wave at the barrier that follows, so neither is ever cleared.
+    uint32_t *flags = reinterpret_cast<uint32_t *>(xbuf + 2 * kQcXBuf);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -526,6 +530,7 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
         // sign rows: 128 rows of 16 slots (16 bytes = two copies each); thread t of these 256 writes
         // 8 slots of row t / 2 (16 neighbouring lanes hit 16 different slot positions)
         const int t = tid - 768, row = t >> 1;
+        if (t < 2) flags[16 + t] = 0u;
         const u2_t sb = sign_bytes((uint32_t)row);
         // slot i ^ (row % 8) of the thread's eight: one exclusive or per address
         const uint32_t sg = lds_addr(smem_raw) + (uint32_t)((row * 16 + (t & 1) * 8 + (row & 7)) * 16);
@@ -625,7 +630,7 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
             }
             issue(cw[kSlot][t], p_base, p_gn, t);                  // the slot's next code word
         }
-        if (stager && !stage_piece(xpiece, resident ? nc : (gc + 1) & 1, sp)) flags[0] = 1u;
+        if (stager && !stage_piece(xpiece, resident ? nc : (gc + 1) & 1, sp)) flags[16 + ((gc + 1) & 1)] = 1u;
         if (!exists) return;
         const bool group_end = last_c;
         if (group_end) {
@@ -649,7 +654,7 @@ __global__ __launch_bounds__(1024) void gemv_q8c_kernel(const uint16_t *__restri
         barrier_in_group = !group_end && (barrier_in_group || stage_next);
         if (stage_next || group_end) {
             __syncthreads();   // hands the x buffers over and / or gathers the group's partial sums
-            if (stage_next && __builtin_amdgcn_ballot_w64(flags[0] != 0) != 0) hand_over = true;
+            if (stage_next && __builtin_amdgcn_ballot_w64(flags[16 + ((gc + 1) & 1)] != 0) != 0) hand_over = true;
         }
         if (group_end && !hand_over && wave < ntg) {
             // wave t adds up tile t: lane (w, quarter) takes wave w's 4 columns with their weights 8^-c,

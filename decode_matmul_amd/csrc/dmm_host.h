@@ -487,13 +487,14 @@ bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
 // matrix-vector kernels are as fast or faster).
 constexpr int kSplitKMinM = 17;
 
-// 17 .. 32 rows of x on a code matrix of up to 17 MB: two passes of the small-batch kernel beat the split
+// 17 .. 32 rows of x on a code matrix of up to 68 KB per compute unit (17 MB on the 256 units the
+// figures below were measured on): two passes of the small-batch kernel beat the split
 // and its second launch, so such a shape asks for no workspace and ignores one (graph launches, us, split /
 // passes, M = 32: 4096 -> 11008 15.8 / 13.8, 11008 -> 4096 18.3 / 15.8, 8192 -> 8192 18.2 / 16.8; but
 // 8192 -> 10240 20.4 / 20.6, 8192 -> 28672 31.7 / 42.0; M = 48 at 4096 -> 11008 19.0 / 18.0, 64 20.2 / 22.3)
-inline bool passes_beat_splitk(int64_t M, int64_t N, int64_t K)
+inline bool passes_beat_splitk(int64_t M, int64_t N, int64_t K, int cus)
 {
-    return M <= 32 && K >= 256 && (K & 255) == 0 && (N & 3) == 0 && N * (K >> 2) <= (17LL << 20);
+    return M <= 32 && K >= 256 && (K & 255) == 0 && (N & 3) == 0 && N * (K >> 2) <= (int64_t)cus * (68 << 10);
 }
 
 bool splitk_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
@@ -584,7 +585,7 @@ Int8Kind pick_int8(int64_t M, int64_t N, int64_t K, int cus)
         int64_t blocks = 1;
         const int r = small_batch_row_block((N + 15) / 16, cus, &blocks);
         const double t_pass = (double)(blocks * (((K >> 8) + 7) / 8)) * (0.35 + 0.27 * r);
-        const double t_gemv = 3.0 + (double)N * (double)(K >> 2) / 7.0e6 + (double)((M + 15) / 16) * t_pass;
+        const double t_gemv = 3.0 + (double)N * (double)(K >> 2) / (27344.0 * cus) /* 7 TB/s on 256 units */ + (double)((M + 15) / 16) * t_pass;
         if (t_gemm < t_gemv) return kInt8Gemm;
     }
     return kInt8Gemv;
@@ -632,7 +633,7 @@ bool passes_beat_gemm(int64_t M, int64_t N, int64_t K, int cus)
     const int tm = gemm_reg_tm(M);
     const int64_t tiles = ((M + 32 * tm - 1) / (32 * tm)) * ((N + kGrBN - 1) / kGrBN);
     const double t_gemm = 3.0 + (double)((tiles + cus - 1) / cus) * (double)K * (tm == 4 ? 0.0104 : 0.0069);
-    const double t_pass = 2.0 + (double)((M + 15) / 16) * (1.5 + (double)N * (double)(K >> 2) / 3.0e6);
+    const double t_pass = 2.0 + (double)((M + 15) / 16) * (1.5 + (double)N * (double)(K >> 2) / (11719.0 * cus));   // 3 TB/s on 256 units
     return t_pass < t_gemm;
 }
 
@@ -641,7 +642,7 @@ int dispatch_f16(const void *x, const void *codes, const void *grid, float scale
                  int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
     if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K) &&
-        !(passes_beat_splitk(M, N, K) && gemv_ok(x, codes, grid, y, M, N, K))) {
+        !(passes_beat_splitk(M, N, K, cu_count()) && gemv_ok(x, codes, grid, y, M, N, K))) {
         const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
         if (splits >= 2) return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, s);
     }
@@ -672,20 +673,34 @@ inline void host_decode_row(const uint16_t *codes, const half_t *grid, int64_t k
     }
 }
 
+// Rows [0, n_rows) split over host threads; body(n0, n1) must not throw.  Threads cost about 50 us
+// each to start, so only work of 2^24 multiply-adds or more (several milliseconds on one core) gets
+// any, and never more than one per 2^22.  If a thread cannot be started the rows it was to
+// take run on the calling thread.
 template <typename F>
-void host_parallel_rows(int64_t n_rows, int64_t work_per_row, F body)
+void host_parallel_rows(int64_t n_rows, int64_t work_per_row, F body) noexcept
 {
+    const int64_t work = n_rows * work_per_row;
     unsigned threads = std::thread::hardware_concurrency();
     if (threads == 0) threads = 1;
     if (threads > 16) threads = 16;
-    if (n_rows * work_per_row < (1 << 20) || n_rows < 2) threads = 1;
+    if ((int64_t)threads > (work >> 22)) threads = (unsigned)(work >> 22);
     if ((int64_t)threads > n_rows) threads = (unsigned)n_rows;
-    if (threads == 1) {
+    if (work < (1 << 24) || threads < 2) {
         body(0, n_rows);
         return;
     }
-    std::vector<std::thread> pool;
-    for (unsigned t = 0; t < threads; t++)
-        pool.emplace_back([=] { body(n_rows * t / threads, n_rows * (t + 1) / threads); });
-    for (auto &th : pool) th.join();
+    std::thread pool[16];
+    unsigned started = 0;
+    for (unsigned t = 1; t < threads; t++) {
+        try {
+            pool[started] = std::thread([=] { body(n_rows * t / threads, n_rows * (t + 1) / threads); });
+        } catch (...) {   // std::system_error: no more threads to be had
+            body(n_rows * t / threads, n_rows);
+            break;
+        }
+        started++;
+    }
+    body(0, n_rows / threads);
+    for (unsigned t = 0; t < started; t++) pool[t].join();
 }

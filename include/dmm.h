@@ -15,6 +15,12 @@
  * eager call) before capturing.  After that every entry point only enqueues kernels and
  * can be captured.
  *
+ * The choice between kernels depends on the device's compute-unit count.  The queries that
+ * predict it without touching a device (dmm_workspace_bytes, dmm_gemv_kernel_name,
+ * dmm_integer_kernel_name) assume 256 compute units until dmm_init (or a first call) has read
+ * the real count on the calling thread's device: on any other part they are exact only after
+ * that.  The choice itself was fitted on the 256-unit MI355X.
+ *
  * Code format (one 16-bit code per 8 consecutive weights along K), as defined by
  * /root/reference/test_decode_matmul.py:29-55 and
  * /root/reference/decode_matmul_cuda/decode_matmul_cuda.cu:45-65:
@@ -45,8 +51,9 @@ enum {
     DMM_ERR_NOT_INITIALIZED = -6, /* first call on a device made under stream capture     */
     DMM_ERR_INTERNAL = -7,      /* the library was built wrongly (a table kernel has
                                    static LDS); no kernel was launched                  */
-    DMM_ERR_SCRATCH_TOO_SMALL = -8 /* dmm_decode_matmul_noalloc_f16: the shape's partial
+    DMM_ERR_SCRATCH_TOO_SMALL = -8, /* dmm_decode_matmul_noalloc_f16: the shape's partial
                                    sums exceed the library's scratch buffer             */
+    DMM_ERR_HOST_MEMORY = -9    /* dmm_decode_matmul_host_f16: malloc of a row failed   */
 };
 
 /* Library version, (major << 16) | minor. */
@@ -111,8 +118,14 @@ int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid,
  * static device array (dmm_noalloc_scratch_bytes), one copy per GPU the library runs on,
  * held until the process ends.  The call allocates nothing and frees nothing.  A shape whose
  * preferred workspace exceeds the buffer is rejected with DMM_ERR_SCRATCH_TOO_SMALL (nothing is
- * launched); shapes that use no workspace (M <= 16, or too few k tiles to split) run exactly
- * as dmm_decode_matmul_f16.  Every partial sum is written before it is read, so the buffer
+ * launched): this is a hard limit - serving such a shape with fewer splits would break the
+ * bit-identity with the full workspace.  It concerns a band of middle-sized M only (M <= 64 is
+ * always accepted, and so is every M large enough to fill the chip without a split): on 256
+ * compute units the rejected M are 65 .. 1024 for N x K = 4096 x 4096 and 4096 x 11008,
+ * 77 .. 256 for 11008 x 4096, 65 .. 512 for 8192 x 8192 and 8192 x 28672, 69 .. 384 for
+ * 10240 x 8192, 74 .. 128 for 28672 x 8192 (not every M inside a band: ask
+ * dmm_workspace_bytes(M, N, K) <= dmm_noalloc_scratch_bytes()).  Shapes that use no
+ * workspace (M <= 16, or too few k tiles to split) run exactly as dmm_decode_matmul_f16.  Every partial sum is written before it is read, so the buffer
  * needs no clearing between calls; but all calls on one GPU share it: two such calls that
  * may overlap (different streams, or graphs replayed concurrently) race. */
 int64_t dmm_noalloc_scratch_bytes(void);
