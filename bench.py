@@ -68,6 +68,8 @@ def parse():
                     help="run only the integer-operator leg and print its object (for profiling that kernel)")
     ap.add_argument("--small-batch-only", action="store_true",
                     help="run only the two small-batch legs and print their objects (for profiling the small-batch kernel)")
+    ap.add_argument("--dispatch-check-only", action="store_true",
+                    help="run only the check of the operator's kernel choices against the alternatives and print its object")
     ap.add_argument("--rotate-mb", type=int, default=400, help="distinct code bytes to rotate through, at least")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch 8 plain device copies of 256 MiB first (a known-size reference for scaling "
@@ -123,6 +125,10 @@ def main():
 
     if args.integer_only:
         print(json.dumps({"integer_operator": integer_operator(torch, lib, capi, workload, dev, stream, rand_codes)}))
+        return
+
+    if args.dispatch_check_only:
+        print(json.dumps({"dispatch_check": dispatch_check(torch, lib, capi, workload, dev)}))
         return
 
     if args.small_batch_only:
@@ -196,7 +202,17 @@ def main():
                 print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
         return run_steps, mode
 
-    def dominant_kernel_timing():
+    def dominant_kernel_timing(f16_only=False):
+        """dominant_kernel_timing_now with the 8-bit kernels allowed (the headline) or switched off."""
+        if not f16_only:
+            return dominant_kernel_timing_now()
+        was8 = lib.dmm_set_gemv_8bit(0)
+        try:
+            return dominant_kernel_timing_now()
+        finally:
+            lib.dmm_set_gemv_8bit(was8)
+
+    def dominant_kernel_timing_now():
         """The kernel that carries most of the step's bytes (by the operator's choice per shape), and its
         launch duration in the regime the headline runs in: its launches of the step alone (its shapes
         taking turns over the rotating buffers) as a HIP graph, HIP events on the stream around each
@@ -284,6 +300,7 @@ def main():
             regions16 = [timed_region(run_auto) for _ in range(max(1, args.repeats))]
         finally:
             lib.dmm_set_gemv_8bit(was)
+    dom16, dom16_probs, dom16_launch_s, dom16_mode = dominant_kernel_timing(f16_only=True)
     wall = sorted(regions)[len(regions) // 2]
     wall16 = sorted(regions16)[len(regions16) // 2]
     ms_per_step = wall * 1e3 / args.steps
@@ -332,6 +349,16 @@ def main():
     if dom_launch_s is None:
         dom_launch_s = kd["seconds"] / kd["launches"]
     achieved = dom_bytes_per_launch / dom_launch_s / 1e9
+    # the same object for the 16-bit-only step's dominant kernel (its launches of the step as a graph)
+    f16_roofline = None
+    if dom16_launch_s is not None:
+        b16 = sum(workload.code_bytes(p["N"], p["K"]) for p in dom16_probs) / len(dom16_probs)
+        f16_roofline = {"kernel": dom16, "avg_launch_us": round(dom16_launch_s * 1e6, 3),
+                        "achieved": round(b16 / dom16_launch_s / 1e9, 2), "unit": "GB/s",
+                        "frac": round(b16 / dom16_launch_s / 1e9 / HBM_PEAK_GBS, 4),
+                        "algorithmic_bytes_per_launch": b16,
+                        "shapes": [{"K": p["K"], "N": p["N"]} for p in dom16_probs],
+                        "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH.get(dom16), "timing": dom16_mode}
 
     out = {
         "metric": "batch-1 effective weight GB/s (code bytes N*K/4 per second, Llama-2-70B projection shapes)",
@@ -344,11 +371,11 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16",
-        "dtype_note": "x, grid, y and the decoded weights are halves, sums fp32; launches of more than two row tiles "
+        "dtype": "f16 in/out; fp8 x bf8 MFMA operands (exact), fp32 sums",
+        "dtype_note": "x, grid, y and the decoded weights are halves, sums fp32; launches of more than one row tile "
                       "per compute unit multiply fp8 weights (exact for this grid) by x split into four bf8 terms "
-                      "(exact) on the 8-bit matrix unit; value_f16_only is the same step with every launch on "
-                      "half x half products",
+                      "(exact) on the 8-bit matrix unit; config.value_f16_only is the same step with every launch on "
+                      "half x half products, roofline.f16_only that step's dominant kernel",
         "value_f16_only": round(value_f16_only, 2),
         "ms_per_step_f16_only": round(wall16 * 1e3 / args.steps, 5),
         "kernels_f16_only": names16,
@@ -357,7 +384,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": "configs[2]: batch-1 decode-GEMV, 8192->10240, 8192->8192, 8192->28672, 28672->8192",
                    "M": 1, "code_buffers_rotated": copies, "distinct_code_MB": round(copies * step_bytes / 1e6, 1),
-                   "step": "4 GEMVs, one per shape", "launch": launch_mode, "preheat_ms": args.preheat_ms},
+                   "step": "4 GEMVs, one per shape", "launch": launch_mode, "preheat_ms": args.preheat_ms,
+                   "value_f16_only": round(value_f16_only, 2), "ms_per_step_f16_only": round(wall16 * 1e3 / args.steps, 5),
+                   "kernels": sorted({lib.dmm_gemv_kernel_name(1, N, K).decode() for K, N in shapes}),
+                   "kernels_f16_only": names16},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
@@ -366,7 +396,8 @@ def main():
                      "avg_launch_us": round(dom_launch_s * 1e6, 3),
                      "timing": dom_mode,
                      "avg_launch_us_eager_events": round(eager_launch_us, 3),
-                     "algorithmic_bytes_per_launch": dom_bytes_per_launch},
+                     "algorithmic_bytes_per_launch": dom_bytes_per_launch,
+                     "f16_only": f16_roofline},
         "all_gemv_launches": {"launches": n_launch, "avg_launch_us": round(kern_s / n_launch * 1e6, 3),
                               "GBps": round(all_gbs, 2), "frac_hbm": round(all_gbs / HBM_PEAK_GBS, 4),
                               "kernels": {n: {"launches": k["launches"],
@@ -386,6 +417,7 @@ def main():
                                              shapes=workload.LLAMA2_70B, batches=(2, 4, 8, 16))
         out["integer_operator"] = integer_operator(torch, lib, capi, workload, dev, stream, rand_codes)
         out["prefill"] = prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes)
+        out["dispatch_check"] = dispatch_check(torch, lib, capi, workload, dev)
         out["cpu_baseline"] = cpu_baseline(torch, workload)
     else:
         out["cpu_baseline"] = None
@@ -481,6 +513,58 @@ def hbm_read_probe(torch, lib, probs, copies, stream, steps):
         out["launch"] = "hip graph, %d steps (%d launches) per replay" % (graph_steps, graph_steps * len(probs))
     except Exception as e:
         print("bench.py: read-probe graph failed (%s)" % e, file=sys.stderr)
+    out["library_independent"] = torch_read_figures(torch, probs, copies)
+    return out
+
+
+def torch_read_figures(torch, probs, copies):
+    """What the box gives a reader of the same rotating code buffers without any kernel of this library: torch's
+    device-to-device copy (reads and writes the bytes) and torch's row sums (reads them, writes next to nothing:
+    the buffer as 4096 rows of int32, one sum per row), the four shapes taking turns, each as replays of one
+    HIP graph like the headline.  Per step of four launches; `GBps_read` counts the code bytes once."""
+    step_bytes = sum(p["N"] * p["K"] // 4 for p in probs)
+    graph_steps = max(copies, 12 // copies * copies)
+    dst = [torch.empty_like(p["codes"][0]) for p in probs]
+    views = [[c.view(torch.int32).view(4096, -1) for c in p["codes"]] for p in probs]
+    sums = [torch.empty(4096, dtype=torch.int32, device=dst[0].device) for _ in probs]
+
+    def enqueue_copy(i):
+        for k, p in enumerate(probs):
+            dst[k].copy_(p["codes"][i % copies])
+
+    def enqueue_sum(i):
+        for k in range(len(probs)):
+            torch.sum(views[k][i % copies], dim=1, dtype=torch.int32, out=sums[k])
+
+    def graph_step_us(enqueue):
+        enqueue(0)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(graph_steps):
+                enqueue(i)
+        for _ in range(10):
+            g.replay()
+        torch.cuda.synchronize()
+        t = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for _ in range(8):
+                g.replay()
+            torch.cuda.synchronize()
+            t.append((time.perf_counter() - t0) / (8 * graph_steps))
+        return sorted(t)[2] * 1e6
+    out = {"launch": "hip graph, %d steps (%d launches) per replay" % (graph_steps, graph_steps * len(probs))}
+    for name, enqueue, moved in (("torch_copy", enqueue_copy, 2), ("torch_row_sums", enqueue_sum, 1)):
+        try:
+            us = graph_step_us(enqueue)
+            out[name] = {"step_us": round(us, 3), "GBps_read": round(step_bytes / us / 1e3, 1),
+                         "frac_hbm_read": round(step_bytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                         "GBps_moved": round(moved * step_bytes / us / 1e3, 1),
+                         "frac_hbm_moved": round(moved * step_bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        except Exception as e:
+            print("bench.py: %s graph failed (%s)" % (name, e), file=sys.stderr)
+            out[name] = None
     return out
 
 
@@ -757,6 +841,156 @@ def prefill(torch, dmm, lib, capi, workload, dev, stream, rand_codes):
             "roofline": {"bound": "mfma", "achieved": round(tot_f / tot_t / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": round(tot_f / tot_t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": None, "kernel": "dmm::gemm_reg_kernel"}}
+
+
+def dispatch_check(torch, lib, capi, workload, dev):
+    """The operator's choice of kernel against the alternatives, around every threshold of the choice: each
+    candidate as launches of one HIP graph over the same rotating code buffers (300 MB or more per graph, so the
+    codes come from HBM), HIP events around a replay, median of 7.  A row lists the operator's own time
+    (`chosen_us`), the alternatives', and `slower_by` = chosen / best - 1; `flagged` are the rows where the
+    choice is more than 10 % slower than an alternative."""
+    from decode_matmul_amd import codebook
+    pool_bytes = 420 * 1000 * 1000
+    g = torch.Generator(device=dev)
+    g.manual_seed(77)
+    pool = torch.randint(-32768, 32768, (pool_bytes // 2,), generator=g, dtype=torch.int16, device=dev)
+    cb = codebook.build_codebook_abs().to(dev)
+
+    def graph_us(launch, nbytes):
+        """launch(code_ptr, stream) -> status; us per launch"""
+        stride = (nbytes + 255) // 256 * 256
+        n_buf = max(2, pool_bytes // stride)
+        L = min(max(6, -(-300 * 1000 * 1000 // stride)), 72, n_buf)
+        cur = torch.cuda.current_stream().cuda_stream
+        for i in range(2):
+            st = launch(pool.data_ptr() + i * stride, cur)
+            if st != 0:
+                return None
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            cap = torch.cuda.current_stream().cuda_stream
+            for i in range(L):
+                st = launch(pool.data_ptr() + i * stride, cap)
+                assert st == 0, st
+        t_warm = time.perf_counter()          # 25 ms of replays: the clocks a candidate is timed at must not
+        while True:                           # depend on how long the host took to set it up
+            for _ in range(4):
+                gr.replay()
+            torch.cuda.synchronize()
+            if time.perf_counter() - t_warm > 0.025:
+                break
+        t = []
+        for _ in range(7):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            gr.replay()
+            b.record()
+            torch.cuda.synchronize()
+            t.append(a.elapsed_time(b) * 1e3 / L)
+        return sorted(t)[3]
+
+    rows = []
+
+    def add(check, M, K, N, times, extra=None):
+        chosen = times.pop("operator")
+        alts = {k: round(v, 3) for k, v in times.items() if v is not None}
+        best = min(alts.values()) if alts else chosen
+        row = {"check": check, "M": M, "K": K, "N": N, "chosen_us": round(chosen, 3), "alternatives_us": alts,
+               "slower_by": round(chosen / best - 1.0, 4)}
+        if extra:
+            row.update(extra)
+        rows.append(row)
+
+    def half_inputs(M, K):
+        x, _, grid, scale = workload.make_inputs(M, 8, K, seed=0)
+        return x.to(dev), grid.to(dev), scale
+
+    # ---- one to four rows of x: 8-bit against 16-bit kernels (pick_gemv)
+    mv_shapes = {1: ((4096, 4096), (4096, 4352), (4096, 8192), (8192, 4096), (8192, 4352), (8192, 8192), (8192, 8448),
+                     (11008, 4096), (11008, 4352), (11008, 8192), (11008, 8448), (12288, 4352), (28672, 4096),
+                     (28672, 4352)),
+                 2: ((4096, 8192), (4096, 12288), (4096, 12544), (4096, 16384)),
+                 4: ((3072, 12288), (3072, 12544), (3072, 16384))}
+    for M, shapes in mv_shapes.items():
+        for K, N in shapes:
+            x, grid, scale = half_inputs(M, K)
+            y = torch.empty(M, N, dtype=torch.float16, device=dev)
+            nbytes = workload.code_bytes(N, K)
+
+            def op(fn):
+                return lambda c, s: fn(x.data_ptr(), c, grid.data_ptr(), scale, y.data_ptr(), M, N, K, s)
+            times = {"operator": graph_us(op(lib.dmm_decode_matmul_f16), nbytes),
+                     "8-bit": graph_us(op(lib.dmm_gemv_8bit_f16), nbytes)}
+            was = lib.dmm_set_gemv_8bit(0)
+            try:
+                times["16-bit"] = graph_us(op(lib.dmm_gemv_f16), nbytes)
+            finally:
+                lib.dmm_set_gemv_8bit(was)
+            add("pick_gemv", M, K, N, times, {"kernel": lib.dmm_gemv_kernel_name(M, N, K).decode()})
+
+    # ---- 17 .. 32 rows with a workspace (passes against split K), more rows (passes against the matrix-matrix
+    # kernel, with and without a workspace)
+    ws = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+    mm_cases = [("passes_beat_splitk", M, K, N) for M in (17, 32)
+                for K, N in ((4096, 11008), (8192, 8192), (8192, 8448), (4096, 17408), (8192, 10240))]
+    mm_cases += [("passes_beat_gemm", M, K, N) for M in (48, 64, 128, 256)
+                 for K, N in ((4096, 4096), (4096, 11008), (11008, 4096), (8192, 8192))]
+    for check, M, K, N in mm_cases:
+        x, grid, scale = half_inputs(M, K)
+        y = torch.empty(M, N, dtype=torch.float16, device=dev)
+        nbytes = workload.code_bytes(N, K)
+
+        def ws_op(c, s):
+            nb = min(lib.dmm_workspace_bytes(M, N, K), ws.numel())
+            return lib.dmm_decode_matmul_ws_f16(x.data_ptr(), c, grid.data_ptr(), scale, y.data_ptr(), M, N, K,
+                                                ws.data_ptr(), nb, s)
+
+        def plain_op(c, s):
+            return lib.dmm_decode_matmul_f16(x.data_ptr(), c, grid.data_ptr(), scale, y.data_ptr(), M, N, K, s)
+        times = {"operator": graph_us(ws_op, nbytes)}
+        if check == "passes_beat_gemm":
+            times["operator, no workspace"] = graph_us(plain_op, nbytes)
+        for name, value in (("passes", 0), ("matrix-matrix", 1), ("split K", 2)):
+            was = lib.dmm_set_choice(0, value)
+            try:
+                if value != 2 or lib.dmm_workspace_bytes(M, N, K) > 0:
+                    times[name] = graph_us(ws_op, nbytes)
+            finally:
+                lib.dmm_set_choice(0, was)
+        extra = None
+        if check == "passes_beat_gemm":      # the choice without a workspace: passes or matrix-matrix only
+            t0 = times.pop("operator, no workspace")
+            best2 = min(times["passes"], times["matrix-matrix"])
+            extra = {"chosen_no_workspace_us": round(t0, 3), "slower_by_no_workspace": round(t0 / best2 - 1.0, 4)}
+        add(check, M, K, N, times, extra)
+
+    # ---- the integer operator on more than 16 rows: passes against the matrix-matrix kernel (pick_int8)
+    for M in (32, 64, 128, 192, 256, 384):
+        for K, N in ((4096, 4096), (11008, 4096), (8192, 28672), (28672, 8192)):
+            gi = torch.Generator(device=dev)
+            gi.manual_seed(5)
+            x = torch.randint(-128, 128, (M, K), generator=gi, dtype=torch.int8, device=dev)
+            out = torch.empty(M, N, dtype=torch.int32, device=dev)
+
+            def i8_op(c, s):
+                return lib.dmm_decode_matmul_i8(x.data_ptr(), c, cb.data_ptr(), out.data_ptr(), M, N, K, 1, s)
+            times = {"operator": graph_us(i8_op, workload.code_bytes(N, K))}
+            for name, value in (("passes", 1), ("matrix-matrix", 2)):
+                was = lib.dmm_set_choice(1, value)
+                try:
+                    times[name] = graph_us(i8_op, workload.code_bytes(N, K))
+                finally:
+                    lib.dmm_set_choice(1, was)
+            add("pick_int8", M, K, N, times, {"kernel": lib.dmm_integer_kernel_name(M, N, K).decode()})
+
+    def worst(r):
+        return max(r["slower_by"], r.get("slower_by_no_workspace", 0.0))
+    flagged = [r for r in rows if worst(r) > 0.10]
+    return {"rows": rows, "n_rows": len(rows), "flagged": flagged,
+            "worst_slower_by": round(max(worst(r) for r in rows), 4),
+            "timing": "launches of one HIP graph per candidate over rotating code buffers, HIP events around a replay, "
+                      "median of 7; slower_by = operator's time / best candidate's - 1"}
 
 
 def cpu_baseline(torch, workload):

@@ -24,6 +24,7 @@ SYMBOLS = {
     "dmm_gemv_kernel_name": (ctypes.c_char_p, [_I64, _I64, _I64]),
     "dmm_integer_kernel_name": (ctypes.c_char_p, [_I64, _I64, _I64]),
     "dmm_set_gemv_8bit": (ctypes.c_int, [ctypes.c_int]),
+    "dmm_set_choice": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     "dmm_gemm_f16": (ctypes.c_int, _OP),
     "dmm_generic_f16": (ctypes.c_int, _OP),
     "dmm_workspace_bytes": (ctypes.c_int64, [_I64, _I64, _I64]),

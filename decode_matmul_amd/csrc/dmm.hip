@@ -160,6 +160,12 @@ int dmm_set_gemv_8bit(int enabled)
     return before;
 }
 
+int dmm_set_choice(int which, int value)
+{
+    if (which < 0 || which > 1 || value < -1 || value > 2) return DMM_ERR_BAD_SHAPE;
+    return g_choice[which].exchange(value, std::memory_order_relaxed);
+}
+
 const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K)
 {
     switch (pick_int8(M, N, K, cu_count_or_default())) {
@@ -240,7 +246,7 @@ int dmm_decode_matmul_packed_f16(const void *x, const void *packed, const void *
     if (!mm_ok && !rows_ok) return DMM_ERR_UNSUPPORTED;
     if ((st = ensure_ready(s))) return st;
     if (workspace && workspace_bytes > 0 && mm_ok && M >= kSplitKMinM && aligned(y, 8) &&
-        !(passes_beat_splitk(M, N, K, cu_count()) && mv_ok)) {
+        !(passes_beat_splitk(M, N, K, cu_count()) && rows_ok)) {
         const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
         if (splits >= 2) return launch_gemm_splitk<true>(x, packed, grid, scale, y, workspace, splits, M, N, K, s);
     }
@@ -277,8 +283,13 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
     }
     // the matrix-unit kernels (K <= 2^17: their weights are odd, so |w| <= 127 and no sum of K
     // products leaves int32 - nothing depends on what the matrix unit does on overflow)
-    const Int8Kind kind =
+    Int8Kind kind =
         aligned(x, 16) && aligned(codes, 16) && aligned(out, 16) ? pick_int8(M, N, K, cu_count()) : kInt8Scalar;
+    if (kind != kInt8Scalar && M > 16) {   // both matrix-unit kernels can take it: a benchmark may force one
+        const int force = g_choice[1].load(std::memory_order_relaxed);
+        if (force == 1) kind = kInt8Gemv;
+        if (force == 2) kind = kInt8Gemm;
+    }
     if (kind == kInt8Gemm)
         return tiled ? launch_int8g<true>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream)
                      : launch_int8g<false>(x, codes, codebook_abs, out, M, N, K, (hipStream_t)stream);
@@ -296,7 +307,8 @@ int64_t dmm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 {
     if (M < 1 || N < 1 || K < kGrBK || (K & 63) || M < kSplitKMinM || M > 65535LL * 128 || !gemm_reg_ok(M, N, K))
         return 0;
-    if (passes_beat_splitk(M, N, K, cu_count_or_default())) return 0;   // the small-batch kernel takes it, without a workspace
+    // the small-batch kernel takes it, without a workspace (unless a benchmark forces the split)
+    if (passes_beat_splitk(M, N, K, cu_count_or_default()) && g_choice[0].load(std::memory_order_relaxed) != 2) return 0;
     const int splits = splitk_plan(M, N, K, INT64_MAX, cu_count_or_default());
     return splits >= 2 ? (int64_t)splits * M * N * 4 : 0;
 }

@@ -313,6 +313,12 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
 
+// dmm_set_choice: what a benchmark that checks the operator's choices forces instead (-1: nothing).
+// [0]: more than 16 rows of x (0 passes of the small-batch kernel, 1 matrix-matrix kernel, 2 split K);
+// [1]: the integer operator on more than 16 rows (1 passes of the matrix-vector kernel, 2 matrix-matrix).
+// A forced kernel that cannot take the call leaves the choice to the library.
+std::atomic<int> g_choice[2] = {{-1}, {-1}};
+
 // Whether the operator may pick the 8-bit kernel: dmm_set_gemv_8bit, or DMM_GEMV_8BIT=0 in the
 // environment (read once, at the first call that needs it) for hosts that cannot call it.
 std::atomic<int> g_gemv_q8{-1};
@@ -487,14 +493,36 @@ bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
 // matrix-vector kernels are as fast or faster).
 constexpr int kSplitKMinM = 17;
 
-// 17 .. 32 rows of x on a code matrix of up to 68 KB per compute unit (17 MB on the 256 units the
-// figures below were measured on): two passes of the small-batch kernel beat the split
-// and its second launch, so such a shape asks for no workspace and ignores one (graph launches, us, split /
-// passes, M = 32: 4096 -> 11008 15.8 / 13.8, 11008 -> 4096 18.3 / 15.8, 8192 -> 8192 18.2 / 16.8; but
-// 8192 -> 10240 20.4 / 20.6, 8192 -> 28672 31.7 / 42.0; M = 48 at 4096 -> 11008 19.0 / 18.0, 64 20.2 / 22.3)
+// What passes of the small-batch kernel cost, us: per 16 rows of x about 1 us, the code bytes at 3.6 TB/s on
+// 256 compute units (they come from the caches after the first pass) and K / 6000 (every workgroup streams its
+// rows of x whole).  Graph launches, us per pass: 4096 -> 4096 2.6 - 3.3, 4096 -> 11008 4.5 - 5.5, 11008 -> 4096
+// 6.0 - 7.0, 8192 -> 8192 6.6 - 7.4.
+inline double passes_cost_us(int64_t M, int64_t N, int64_t K, int cus)
+{
+    return 2.0 + (double)((M + 15) / 16) * (1.0 + (double)N * (double)(K >> 2) / (14063.0 * cus) + (double)K / 6000.0);
+}
+
+bool passes_beat_gemm(int64_t M, int64_t N, int64_t K, int cus);
+
+// A workspace is there, and so the choice of splitting K.  17 .. 32 rows of x: two passes of the small-batch
+// kernel beat the split and its second launch while the busiest workgroup has no more than 68 KB of codes
+// (graph launches, us, split / passes, M = 32: 4096 -> 11008 16.8 / 14.9, 8192 -> 8192 19.7 / 18.3, but 8192 ->
+// 8448 18.9 / 22.0, 4096 -> 17408 19.1 / 22.3, 8192 -> 10240 22.4 / 22.0, 8192 -> 28672 31.7 / 42.0).  More rows:
+// the split costs about 14 us + 0.085 per row + 0.3 per MB of codes, and the passes have to beat that by a
+// twentieth, and the matrix-matrix kernel too (M = 48: 4096 -> 4096 18.0 / 11.9, 4096 -> 11008 20.0 / 18.6, 8192 -> 8192
+// 23.6 / 24.3; M = 64: 20.6 / 14.5, 21.3 / 22.8, 23.5 / 30.9; M = 128: 26.5 / 24.4, 28.1 / 39.7, 33.7 / 55.1) -
+// only where that was measured, up to 128 rows on 2 MB of codes or more.  Such a shape asks for no
+// workspace and ignores one.
 inline bool passes_beat_splitk(int64_t M, int64_t N, int64_t K, int cus)
 {
-    return M <= 32 && K >= 256 && (K & 255) == 0 && (N & 3) == 0 && N * (K >> 2) <= (int64_t)cus * (68 << 10);
+    if (K < 256 || (K & 255) || (N & 3)) return false;
+    if (M <= 32) {
+        const int64_t share = ((N + 15) / 16 + cus - 1) / cus;   // row tiles of the busiest workgroup
+        return share * 4 * K <= (68 << 10);
+    }
+    if (M > 128 || N * (K >> 2) < (2 << 20)) return false;
+    const double t_split = 14.0 + 0.085 * (double)M + 0.3e-6 * (double)N * (double)(K >> 2) * (256.0 / cus);
+    return passes_cost_us(M, N, K, cus) * 1.05 < t_split && passes_beat_gemm(M, N, K, cus);
 }
 
 bool splitk_ok(const void *x, const void *codes, const void *grid, const void *y, int64_t M, int64_t N,
@@ -586,7 +614,7 @@ Int8Kind pick_int8(int64_t M, int64_t N, int64_t K, int cus)
         const int r = small_batch_row_block((N + 15) / 16, cus, &blocks);
         const double t_pass = (double)(blocks * (((K >> 8) + 7) / 8)) * (0.35 + 0.27 * r);
         const double t_gemv = 3.0 + (double)N * (double)(K >> 2) / (27344.0 * cus) /* 7 TB/s on 256 units */ + (double)((M + 15) / 16) * t_pass;
-        if (t_gemm < t_gemv) return kInt8Gemm;
+        if (t_gemm < 0.95 * t_gemv) return kInt8Gemm;   // the estimate of the passes runs high for long K
     }
     return kInt8Gemv;
 }
@@ -622,27 +650,31 @@ int cu_count_or_default()
     return g_dev[dev].ready.load(std::memory_order_acquire) ? g_dev[dev].cus : 256;
 }
 
-// More than 32 rows of x and no workspace.  The matrix-matrix kernel costs about K * 6.9 ns (x tiles
-// of up to 64 rows) or K * 10.4 ns (128 rows) per round of one 256-row tile per CU, however few of its
-// tiles exist; the small-batch kernel about 1.5 us plus the code bytes at 3 TB/s (they come from the
-// caches after the first pass) per 16 rows of x.  The cheaper estimate wins.  Graph launches, us,
-// matrix-matrix / passes: M = 64 11008 -> 4096 74.7 / 30.2, 28672 -> 8192 186.7 / 95.6, 8192 -> 28672
-// 57.7 / 79.6; M = 128 4096 -> 11008 47.6 / 41.7, 8192 -> 10240 86.1 / 71.5, 8192 -> 28672 88.2 / 150.2.
+// More than 32 rows of x, passes of the small-batch kernel or the matrix-matrix kernel: the latter costs about
+// K * 6.9 ns (x tiles of up to 64 rows) or K * 10.4 ns (128 rows) per round of one 256-row tile per CU, however
+// few of its tiles exist.  The cheaper estimate wins.  Graph launches, us, matrix-matrix / passes: M = 64 11008 ->
+// 4096 75.7 / 28.4, 28672 -> 8192 186.7 / 95.6, 8192 -> 28672 57.7 / 79.6; M = 128 4096 -> 11008 49.1 / 39.7, 8192 ->
+// 8192 87.9 / 55.1; M = 256 4096 -> 4096 47.9 / 44.2, 4096 -> 11008 49.5 / 73.8, 11008 -> 4096 125.2 / 97.7,
+// 8192 -> 8192 88.7 / 107.5.
 bool passes_beat_gemm(int64_t M, int64_t N, int64_t K, int cus)
 {
     const int tm = gemm_reg_tm(M);
     const int64_t tiles = ((M + 32 * tm - 1) / (32 * tm)) * ((N + kGrBN - 1) / kGrBN);
     const double t_gemm = 3.0 + (double)((tiles + cus - 1) / cus) * (double)K * (tm == 4 ? 0.0104 : 0.0069);
-    const double t_pass = 2.0 + (double)((M + 15) / 16) * (1.5 + (double)N * (double)(K >> 2) / (11719.0 * cus));   // 3 TB/s on 256 units
-    return t_pass < t_gemm;
+    return passes_cost_us(M, N, K, cus) < t_gemm;
 }
 
 // the operator's dispatch once the arguments are checked and the device is ready
 int dispatch_f16(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M, int64_t N,
                  int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
+    const int force = M > 16 ? g_choice[0].load(std::memory_order_relaxed) : -1;
+    if (force == 0 && gemv_rows_ok(x, codes, grid, y, M, N, K))
+        return M <= 32 ? run_gemv<false>(x, codes, grid, scale, y, M, N, K, s)
+                       : run_gemv_regx<false>(x, codes, grid, scale, y, M, N, K, s);
+    if (force == 1 && gemm_ok(x, codes, grid, y, M, N, K)) return run_gemm(x, codes, grid, scale, y, M, N, K, s);
     if (workspace && workspace_bytes > 0 && splitk_ok(x, codes, grid, y, M, N, K) &&
-        !(passes_beat_splitk(M, N, K, cu_count()) && gemv_ok(x, codes, grid, y, M, N, K))) {
+        (force == 2 || !(passes_beat_splitk(M, N, K, cu_count()) && gemv_rows_ok(x, codes, grid, y, M, N, K)))) {
         const int splits = splitk_plan(M, N, K, workspace_bytes, cu_count());
         if (splits >= 2) return launch_gemm_splitk(x, codes, grid, scale, y, workspace, splits, M, N, K, s);
     }

@@ -121,7 +121,7 @@ int dmm_decode_matmul_ws_f16(const void *x, const void *codes, const void *grid,
  * launched): this is a hard limit - serving such a shape with fewer splits would break the
  * bit-identity with the full workspace.  It concerns a band of middle-sized M only (M <= 64 is
  * always accepted, and so is every M large enough to fill the chip without a split): on 256
- * compute units the rejected M are 65 .. 1024 for N x K = 4096 x 4096 and 4096 x 11008,
+ * compute units the rejected M are 113 .. 1024 for N x K = 4096 x 4096, 65 .. 1024 for 4096 x 11008,
  * 77 .. 256 for 11008 x 4096, 65 .. 512 for 8192 x 8192 and 8192 x 28672, 69 .. 384 for
  * 10240 x 8192, 74 .. 128 for 28672 x 8192 (not every M inside a band: ask
  * dmm_workspace_bytes(M, N, K) <= dmm_noalloc_scratch_bytes()).  Shapes that use no
@@ -240,6 +240,19 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
  * (matrix-vector, 16 rows of x per launch) or "dmm::int8_kernel" (scalar).  For tests and
  * benchmarks; no counterpart in the reference. */
 const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K);
+
+/* For benchmarks that check the operator's choices against the alternatives, as launches of one
+ * HIP graph: forces a kernel where the library would choose, process-wide, for calls made after it
+ * returns.  which = 0: the half-precision operator on more than 16 rows of x (value 0: passes of the
+ * small-batch kernel, 16 rows each; 1: the matrix-matrix kernel; 2: split K, where a workspace is
+ * given - dmm_workspace_bytes then answers for the split as well).  which = 1: the integer
+ * operator on more than 16 rows (1: passes of the matrix-vector kernel, 2: the matrix-matrix
+ * kernel).  value -1: the library's own choice (the default).  A forced kernel that cannot take a
+ * call (shape, alignment) leaves that call to the library's choice; results do not depend on
+ * the setting beyond what the kernels' own summation orders differ by (the integer operator:
+ * not at all).  Returns the previous value (>= -1), or DMM_ERR_BAD_SHAPE for arguments out of
+ * range.  No counterpart in the reference. */
+int dmm_set_choice(int which, int value);
 
 /* Kernel timing hook for benchmarks.  While a (start, stop) pair of hipEvent_t handles is
  * set on the calling thread, the dominant kernel of each operator call records `start`

@@ -89,8 +89,8 @@ def test_argument_errors_are_status_codes_not_crashes():
     # the workspace variant: size query, misaligned or negative workspace, NULL workspace = plain call
     assert lib.dmm_workspace_bytes(1, 4096, 4096) == 0            # batch 1 never splits
     assert lib.dmm_workspace_bytes(2048, 4096, 4096) == 0         # enough tiles already
-    assert lib.dmm_workspace_bytes(48, 11008, 4096) % (48 * 11008 * 4) == 0
-    assert lib.dmm_workspace_bytes(48, 11008, 4096) >= 2 * 48 * 11008 * 4
+    assert lib.dmm_workspace_bytes(48, 8192, 8192) % (48 * 8192 * 4) == 0
+    assert lib.dmm_workspace_bytes(48, 8192, 8192) >= 2 * 48 * 8192 * 4
     assert lib.dmm_workspace_bytes(32, 11008, 4096) == 0          # up to 32 rows, 11 MB of codes: passes, no split
     assert lib.dmm_workspace_bytes(32, 28672, 8192) >= 2 * 32 * 28672 * 4   # 59 MB of codes: the split pays
     assert lib.dmm_workspace_bytes(32, 11008, 4160) > 0           # K % 256 != 0: no small-batch kernel

@@ -40,9 +40,9 @@ def test_noalloc_matches_workspace_entry_two_calls_in_a_row():
     limit = lib.dmm_noalloc_scratch_bytes()
     assert limit == 16 << 20
     # a large call, then smaller ones: the second finds the first's partial sums in the buffer.
-    # (48, 11008, 4096) and (40, 1024, 2048) split K; (8, 512, 1024) uses no scratch at all.
+    # (48, 8192, 8192) and (40, 1024, 2048) split K; (8, 512, 1024) uses no scratch at all.
     used = []
-    for seed, (M, N, K) in enumerate(((48, 11008, 4096), (40, 1024, 2048), (64, 4096, 11008), (8, 512, 1024))):
+    for seed, (M, N, K) in enumerate(((48, 8192, 8192), (40, 1024, 2048), (64, 4096, 11008), (8, 512, 1024))):
         x, codes, grid, scale = workload.make_inputs(M, N, K, seed=seed, device=DEV)
         want, nbytes = _ws_call(x, codes, grid, scale)
         assert nbytes <= limit
