@@ -493,13 +493,15 @@ bool gemm_reg_ok(int64_t M, int64_t N, int64_t K)
 // matrix-vector kernels are as fast or faster).
 constexpr int kSplitKMinM = 17;
 
-// What passes of the small-batch kernel cost, us: per 16 rows of x about 1 us, the code bytes at 3.6 TB/s on
-// 256 compute units (they come from the caches after the first pass) and K / 6000 (every workgroup streams its
-// rows of x whole).  Graph launches, us per pass: 4096 -> 4096 2.6 - 3.3, 4096 -> 11008 4.5 - 5.5, 11008 -> 4096
-// 6.0 - 7.0, 8192 -> 8192 6.6 - 7.4.
+// What passes of the small-batch kernel cost, us: 2 for the launch, the code bytes once at 5.5 TB/s on 256
+// compute units (the first pass reads them from HBM), and per 16 rows of x about 0.9, the code bytes at
+// 3.8 TB/s (from the caches) and K / 6000 (every workgroup streams its rows of x whole).  Graph launches, us,
+// M = 64 / 128 / 256: 4096 -> 4096 14.5 / 24.4 / 44.2, 4096 -> 11008 22.8 / 39.7 / 73.8, 11008 -> 4096 28.4 / 51.4 /
+// 97.7, 8192 -> 8192 30.9 / 55.1 / 107.5.
 inline double passes_cost_us(int64_t M, int64_t N, int64_t K, int cus)
 {
-    return 2.0 + (double)((M + 15) / 16) * (1.0 + (double)N * (double)(K >> 2) / (14063.0 * cus) + (double)K / 6000.0);
+    const double mb = 1e-6 * (double)N * (double)(K >> 2) * (256.0 / cus);
+    return 2.0 + mb / 5.5 + (double)((M + 15) / 16) * (0.9 + mb / 3.8 + (double)K / 6000.0);
 }
 
 bool passes_beat_gemm(int64_t M, int64_t N, int64_t K, int cus);
