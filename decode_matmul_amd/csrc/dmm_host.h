@@ -370,7 +370,13 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
     const bool long_launch = M == 1 ? n_tiles > 2 * cus || (n_tiles > cus && (K <= 8192 || K >= 12288)) : n_tiles > 3 * cus;
     if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
-    if (gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
+    // Two to four rows: the small-batch kernel's eight waves start sooner than the streaming kernel's sixteen
+    // with their x in the LDS, which decides a launch of one tile per workgroup on a short x, and four rows
+    // (graph launches, us, streaming / small-batch: M = 2 4096 -> 4096 4.77 / 4.47, 11008 -> 4096 6.27 / 6.51,
+    // 4096 -> 11008 7.28 / 7.26; M = 4 4096 -> 4096 5.13 / 4.47, 4096 -> 11008 7.63 / 7.45, 4096 -> 12288 7.74 / 7.59;
+    // but M = 2 8192 -> 28672 17.7 / 21.2, M = 3 18.6 / 21.4)
+    const bool small_first = M == 4 || (M >= 2 && M <= 4 && n_tiles <= cus && K <= 4096);
+    if (!small_first && gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
     return kGemvRegx;
 }
 

@@ -309,6 +309,9 @@ def test_gemv_8bit_switch_and_kernel_name():
         assert lib.dmm_gemv_kernel_name(M, 32784, K) == b"dmm::gemv_q8c_kernel"       # more: groups of three tiles
         assert lib.dmm_gemv_kernel_name(3, N, K) == b"dmm::gemv_q8_kernel"            # two to four rows of x
         assert lib.dmm_gemv_kernel_name(3, 12288, K) == b"dmm::gemv_stream_kernel"
+        assert lib.dmm_gemv_kernel_name(4, 12288, K) == b"dmm::gemv_regx_kernel"      # four rows: the small-batch kernel
+        assert lib.dmm_gemv_kernel_name(2, 4096, K) == b"dmm::gemv_regx_kernel"       # one tile per CU, short x
+        assert lib.dmm_gemv_kernel_name(2, 4096, 8192) == b"dmm::gemv_stream_kernel"
         assert lib.dmm_gemv_kernel_name(3, N, 28672) == b"dmm::gemv_regx_kernel"      # their terms do not fit
         assert lib.dmm_gemv_kernel_name(32, N, K) == b"dmm::gemv_regx_kernel"
         assert lib.dmm_gemv_kernel_name(M, N, 264) == b""
