@@ -134,11 +134,13 @@ __global__ __launch_bounds__(1024) void gemv_q8d_kernel(const uint16_t *__restri
         cwd = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, ok ? tile0_off + t * tile_stride + step * step_stride : kOut, 0);
     };
     u4_t cw[D];
-    // The first items of the code stream.  A compute unit's memory pipeline holds about 32 KB of
-    // outstanding loads; a wave that asks for more blocks at the issue until earlier loads have come
-    // back, and a blocked wave writes no tables.  So only kFirst items per wave (32 KB per workgroup)
-    // go out ahead of the prologue's work and the rest of the ring after its barrier.
-    constexpr int kFirst = D < 2 ? D : 2;
+    // The first items of the code stream.  The memory pipeline of a compute unit takes a row-major code
+    // load apart in about 64 clocks (16 rows, 16 pages) and serves loads in the order they were issued,
+    // so every code load that goes out ahead of the prologue's own loads (grid rows, x) delays the tables
+    // by that much, and a wave that asks for more than the pipeline holds blocks at the issue and writes
+    // no tables meanwhile.  One item per wave goes out here, the rest of the ring after the wave's share
+    // of the prologue's work, ahead of the barrier: they are back when the barrier opens.
+    constexpr int kFirst = 1;
 #pragma unroll
     for (int d = 0; d < kFirst; d++) issue(cw[d], d / NT, d % NT);
 
@@ -178,13 +180,13 @@ __global__ __launch_bounds__(1024) void gemv_q8d_kernel(const uint16_t *__restri
     } else {
         fits = stage_piece(xpiece, (n_chunks - 1) & 1, sp);   // pieces past the end of x are zeros
     }
+#pragma unroll
+    for (int d = kFirst; d < D; d++) issue(cw[d], d / NT, d % NT);
     {
         const bool wave_bad = __builtin_amdgcn_ballot_w64(!fits) != 0;
         if (lane == 0) flags[wave] = wave_bad ? 1u : 0u;
     }
     __syncthreads();
-#pragma unroll
-    for (int d = kFirst; d < D; d++) issue(cw[d], d / NT, d % NT);
     bool hand_over = __builtin_amdgcn_ballot_w64(flags[lane & (W - 1)] != 0) != 0;
 
     // B operands of this lane (offsets inside an x buffer): columns 0 .. 3 read term c16 of the wave's k step
