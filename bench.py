@@ -6,21 +6,27 @@ shapes.  One step = the four GEMVs (8192->10240, 8192->8192, 8192->28672, 28672-
 on the next of several distinct code buffers so that the 256 MB Infinity Cache cannot serve
 the weights; `value` is code bytes (N*K/4 per GEMV) per second over the timed region, inputs
 resident in HBM.  The region of exactly --steps steps is timed --repeats times (one HIP graph
-replay of up to 60 steps, bracketed by synchronisation) and the median region counts;
-`value_f16_only` is the same with the 8-bit kernels switched off, timed after the headline.
-Before the --warmup steps the step is replayed for --preheat-ms (200 ms): the device needs some
-15 ms of work to leave its idle clocks.
+replay of up to 60 steps, bracketed by synchronisation) and the median region counts.
+`dtype` says what the arithmetic is: halves in and out, fp8 x bf8 operands on the matrix unit
+(exact for the grid and every finite x), fp32 sums; `config.value_f16_only` is the same step with
+the 8-bit kernels switched off, timed after the headline.  Before the --warmup steps the step is
+replayed for --preheat-ms (200 ms): the device needs some 15 ms of work to leave its idle clocks.
 
 `roofline` is the GEMV kernel that carries most of the step's bytes, alone: code bytes per
 launch over the kernel's launch duration - HIP events on the stream around replays of a graph of
-that kernel's launches of the step, region / launches - against 8 TB/s; `gemv_shapes` and
+that kernel's launches of the step, region / launches - against 8 TB/s; `roofline.f16_only` is the
+same for the 16-bit-only step's kernel, and `roofline.read_only_step` what a reader of the same
+rotating buffers gets per step: this library's read probe (same launch shape and access pattern
+as the batch-1 kernels, no decode) and, owing nothing to this library, torch's row sums and
+torch's device copy (from `hbm_read_probe`, which also has the probe per shape and per launch with
+nothing to read: the memory system's and the launch path's share of the step).  `gemv_shapes` and
 `all_gemv_launches` hold every launch of the step, per shape and per kernel, from HIP events
-placed around each eager launch by the library's timing hook.  `hbm_read_probe` is what a kernel that only
-reads the same code buffers reaches (per shape, as a graph step, and per launch with nothing
-to read): the memory system's and the launch path's share of the step.  `gemv_7b_step` is a
+placed around each eager launch by the library's timing hook.  `gemv_7b_step` is a
 Llama-2-7B layer's four projections as one graph, gate and up as one call on concatenated code
 rows.  `prefill`, `small_batch` and `integer_operator` carry the M=2048, M=4..32 and int8
-figures; `cpu_baseline` is the torch CPU path on the host cores on one 8192x8192 GEMV.
+figures; `dispatch_check` times the operator's choice of kernel against the alternatives around
+every threshold of the choice and lists the rows where it is more than 10 % slower;
+`cpu_baseline` is the torch CPU path on the host cores on the four calls of one step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
 """
@@ -42,7 +48,7 @@ MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 # WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain 256 MiB device copy
 # (x2.000 and x1.000).  39.19 MB per launch against 38,855,680 algorithmic bytes (codes, x, grid, y): 1.009.
 # The many-tile 8-bit kernel (more than eight row tiles per compute unit) runs in no leg of this file.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8d_kernel": 39191365, "dmm::gemv_stream_kernel": 39190001}
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8d_kernel": 39191335, "dmm::gemv_stream_kernel": 39189916}
 GEMV_TRAFFIC_SOURCE = {k: "constant from an earlier rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command, summarised in "
                           "profiles/gemv_kernels_llama70b_batch1.md; not measured by this run (a counter run cannot share a "
                           "process with the timed one)" for k in GEMV_TRAFFIC_BYTES_PER_LAUNCH}
@@ -409,6 +415,16 @@ def main():
 
     if not args.quick:
         out["hbm_read_probe"] = hbm_read_probe(torch, lib, probs, copies, stream, args.steps)
+        # what a reader of the same rotating buffers gets, per step of four launches, beside the operator's step:
+        # this library's read-only probe and two that owe nothing to it (torch's row sums and device copy)
+        hp, li = out["hbm_read_probe"], out["hbm_read_probe"].get("library_independent") or {}
+        out["roofline"]["read_only_step"] = {
+            "operator_step_us": round(ms_per_step * 1e3, 3),
+            "own_probe_step_us": hp.get("step_us"), "own_probe_GBps": hp.get("step_GBps"),
+            "torch_row_sums_step_us": (li.get("torch_row_sums") or {}).get("step_us"),
+            "torch_row_sums_GBps_read": (li.get("torch_row_sums") or {}).get("GBps_read"),
+            "torch_copy_step_us": (li.get("torch_copy") or {}).get("step_us"),
+            "torch_copy_GBps_moved": (li.get("torch_copy") or {}).get("GBps_moved")}
         out["gemv_packed"] = gemv_packed(torch, lib, capi, workload, probs, copies, stream, args.steps)
         out["gemv_7b_step"] = gemv_7b_step(torch, lib, capi, workload, dev, rand_codes)
         out["gemv_7b_shapes"] = gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes)

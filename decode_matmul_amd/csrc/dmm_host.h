@@ -353,22 +353,20 @@ int run_gemv_q8(const void *x, const void *codes, const void *grid, float scale,
 bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok(M, N, K) : gemv_q8_ok<1, 16>(M, N, K); }
 
 // The choice among the matrix-vector kernels.  The 8-bit kernels where they apply and pay.  One row of x:
-// from more than one row tile per workgroup on, except for an x of two to three chunks whose last chunk is
-// short (8192 < K < 12288), which needs more than two tiles (measured as launches of one HIP graph on
-// rotating code buffers, 8-bit against 16-bit kernel, us per launch: 8192 -> 28672 14.0 / 16.6, 8192 -> 10240
-// 7.0 / 8.7, 28672 -> 8192 14.9 / 16.2, 28672 -> 6144 13.6 / 15.4, 8192 -> 8192 6.55 / 6.78, 8192 -> 4352 5.98 /
-// 6.69, 4096 -> 8192 5.01 / 5.44, 4096 -> 6144 4.96 / 5.41, 5120 -> 5120 5.40 / 5.69, 4096 -> 4608 4.86 / 5.39;
-// but 11008 -> 5120 7.90 / 7.71, 11008 -> 8192 8.60 / 8.01, and with one tile per workgroup 4096 -> 4096 4.46 /
-// 4.49, 11008 -> 4096 6.18 / 5.55).  Two to four rows from more than three tiles on.  A grid that does not
-// fit fp8 costs them a second table build, and the 16-bit kernel's y is the correctly rounded one.
-// Otherwise the 16-bit streaming kernel, one tile at a time; the register-x kernel when x does not fit
-// the LDS.
+// from more than one row tile per workgroup on, and with one tile on a long x (measured as launches of one
+// HIP graph on rotating code buffers, 8-bit against 16-bit kernel, us per launch: 8192 -> 28672 13.7 / 16.6,
+// 28672 -> 8192 14.0 / 16.2, 8192 -> 10240 6.9 / 8.7, 8192 -> 8192 6.2 / 7.2, 8192 -> 4352 5.9 / 6.8, 4096 -> 8192
+// 4.7 / 5.3, 4096 -> 4352 4.4 / 5.2, 11008 -> 8192 7.6 / 8.2, 11008 -> 4352 7.0 / 7.7, 28672 -> 4096 10.4 / 11.0;
+// but with one tile per workgroup 4096 -> 4096 4.22 / 4.21, 8192 -> 4096 4.97 / 4.89, 11008 -> 4096 5.98 / 5.48).
+// Two to four rows from more than three tiles on.  A grid that does not fit fp8 costs them a second table
+// build, and the 16-bit kernel's y is the correctly rounded one.  Otherwise the 16-bit streaming kernel,
+// one tile at a time; the small-batch kernel when x does not fit the LDS.
 enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
 
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const bool long_launch = M == 1 ? n_tiles > 2 * cus || (n_tiles > cus && (K <= 8192 || K >= 12288)) : n_tiles > 3 * cus;
+    const bool long_launch = M == 1 ? n_tiles > cus || K >= 16384 : n_tiles > 3 * cus;
     if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
     // Two to four rows: the small-batch kernel's eight waves start sooner than the streaming kernel's sixteen
     // with their x in the LDS, which decides a launch of one tile per workgroup on a short x, and four rows

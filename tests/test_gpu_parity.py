@@ -301,7 +301,9 @@ def test_gemv_8bit_switch_and_kernel_name():
         assert lib.dmm_gemv_kernel_name(M, 8192, K) == b"dmm::gemv_q8d_kernel"        # two tiles per CU
         assert lib.dmm_gemv_kernel_name(M, 4112, K) == b"dmm::gemv_q8d_kernel"        # more than one
         assert lib.dmm_gemv_kernel_name(M, 4096, K) == b"dmm::gemv_stream_kernel"     # one
-        assert lib.dmm_gemv_kernel_name(M, 8192, 11008) == b"dmm::gemv_stream_kernel" # two, x of two and a bit chunks
+        assert lib.dmm_gemv_kernel_name(M, 8192, 11008) == b"dmm::gemv_q8d_kernel"    # two, x of two and a bit chunks
+        assert lib.dmm_gemv_kernel_name(M, 4096, 11008) == b"dmm::gemv_stream_kernel" # one tile per CU
+        assert lib.dmm_gemv_kernel_name(M, 4096, 28672) == b"dmm::gemv_q8d_kernel"    # one, long x
         assert lib.dmm_gemv_kernel_name(M, 8208, 11008) == b"dmm::gemv_q8d_kernel"
         assert lib.dmm_gemv_kernel_name(M, 8192, 12288) == b"dmm::gemv_q8d_kernel"    # two, long x
         assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_q8d_kernel"       # x goes through in chunks
