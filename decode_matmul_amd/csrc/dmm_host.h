@@ -358,7 +358,9 @@ bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok
 // 28672 -> 8192 14.0 / 16.2, 8192 -> 10240 6.9 / 8.7, 8192 -> 8192 6.2 / 7.2, 8192 -> 4352 5.9 / 6.8, 4096 -> 8192
 // 4.7 / 5.3, 4096 -> 4352 4.4 / 5.2, 11008 -> 8192 7.6 / 8.2, 11008 -> 4352 7.0 / 7.7, 28672 -> 4096 10.4 / 11.0;
 // but with one tile per workgroup 4096 -> 4096 4.22 / 4.21, 8192 -> 4096 4.97 / 4.89, 11008 -> 4096 5.98 / 5.48).
-// Two to four rows from more than three tiles on.  A grid that does not fit fp8 costs them a second table
+// Two to four rows from more than four tiles on (M = 2, 8-bit / 16-bit: 4096 -> 22016 10.1 / 11.0, 4096 -> 32000
+// 12.4 / 14.1, but 4096 -> 16384 8.7 / 8.7, 4096 -> 12544 8.5 / 8.3; M = 4: 3072 -> 16384 8.6 / 8.2, 3072 -> 12544 8.4 / 7.8).
+// A grid that does not fit fp8 costs them a second table
 // build, and the 16-bit kernel's y is the correctly rounded one.  Otherwise the 16-bit streaming kernel,
 // one tile at a time; the small-batch kernel when x does not fit the LDS.
 enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
@@ -366,7 +368,7 @@ enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const bool long_launch = M == 1 ? n_tiles > cus || K >= 16384 : n_tiles > 3 * cus;
+    const bool long_launch = M == 1 ? n_tiles > cus || K >= 16384 : n_tiles > 4 * cus;
     if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
     // Two to four rows: the small-batch kernel's eight waves start sooner than the streaming kernel's sixteen
     // with their x in the LDS, which decides a launch of one tile per workgroup on a short x, and four rows

@@ -148,7 +148,7 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
 /*   dmm_gemv_8bit_f16  the matrix-vector kernels on 8-bit MFMA operands, which dmm_gemv_f16 and
  *                    the operator pick for M = 1 on launches of more than one 16-row tile per
  *                    compute unit (from one on when K >= 16384) and for M = 2 .. 4 on launches of
- *                    more than three (shorter ones gain nothing from them).  Weights as fp8 (e4m3) bytes - exact when
+ *                    more than four (shorter ones gain nothing from them).  Weights as fp8 (e4m3) bytes - exact when
  *                    every grid value has at most 4 significant bits in fp8's range, as the E8P
  *                    grid does - and x as four bf8 (e5m2) terms that add up to it exactly; the
  *                    +-1/4 shift of a code is added through the per-code means of x (two halves,

@@ -309,7 +309,8 @@ def test_gemv_8bit_switch_and_kernel_name():
         assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_q8d_kernel"       # x goes through in chunks
         assert lib.dmm_gemv_kernel_name(M, 32768, K) == b"dmm::gemv_q8d_kernel"       # eight tiles per CU
         assert lib.dmm_gemv_kernel_name(M, 32784, K) == b"dmm::gemv_q8c_kernel"       # more: groups of three tiles
-        assert lib.dmm_gemv_kernel_name(3, N, K) == b"dmm::gemv_q8_kernel"            # two to four rows of x
+        assert lib.dmm_gemv_kernel_name(3, 32768, K) == b"dmm::gemv_q8_kernel"        # two to four rows of x, many tiles
+        assert lib.dmm_gemv_kernel_name(3, N, K) == b"dmm::gemv_stream_kernel"        # four tiles per CU: not yet
         assert lib.dmm_gemv_kernel_name(3, 12288, K) == b"dmm::gemv_stream_kernel"
         assert lib.dmm_gemv_kernel_name(4, 12288, K) == b"dmm::gemv_regx_kernel"      # four rows: the small-batch kernel
         assert lib.dmm_gemv_kernel_name(2, 4096, K) == b"dmm::gemv_regx_kernel"       # one tile per CU, short x
@@ -905,6 +906,39 @@ def test_split_k_integer_bridge_is_exact():
     y, wsb = c_matmul_ws(dev(x.astype(np.float16)), dev(codes), dev(orc.grid_from_codebook(cb)), scale)
     torch.cuda.synchronize()
     assert wsb > 0 and np.array_equal(bits(y), bits(want))
+
+
+def test_forced_kernel_choices_give_the_same_results():
+    """dmm_set_choice (the benchmark's check of the dispatch) forces a kernel, never a result: the integer
+    operator is exact either way, the half-precision operator on the integer bridge too (every route's
+    sums are exact there), and a forced kernel that cannot take a call leaves it to the library."""
+    lib = capi.lib()
+    rng = np.random.default_rng(77)
+    cb = orc.build_codebook_abs()
+    M, N, K = 40, 272, 1024
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    yi = orc.decode_matmul_i32(x, codes, cb)
+    try:
+        for value in (-1, 1, 2):
+            assert lib.dmm_set_choice(1, value) >= -1
+            out = c_matmul_i8(dev(x), dev(codes), dev(cb), False)
+            torch.cuda.synchronize()
+            assert np.array_equal(out.cpu().numpy(), yi), value
+        scale = 2.0 ** -8
+        want = (yi.astype(np.float64) / 4 * scale).astype(np.float16)
+        xd, cd, gd = dev(x.astype(np.float16)), dev(codes), dev(orc.grid_from_codebook(cb))
+        for value in (-1, 0, 1, 2):
+            assert lib.dmm_set_choice(0, value) >= -1
+            y, _ = c_matmul_ws(xd, cd, gd, scale)
+            torch.cuda.synchronize()
+            assert np.array_equal(bits(y), bits(want)), value
+            y1 = c_matmul(xd[:1].contiguous(), cd, gd, scale, "auto")     # one row: the override does not apply
+            torch.cuda.synchronize()
+            assert np.array_equal(bits(y1), bits(want[:1])), value
+    finally:
+        lib.dmm_set_choice(0, -1)
+        lib.dmm_set_choice(1, -1)
 
 
 # ----------------------------------------------------------------- maximum sizes

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_status_strings():
     lib = capi.lib()
-    for st in (0, -1, -2, -3, -4, -5):
+    for st in (0, -1, -2, -3, -4, -5, -6, -7, -8, -9):
         assert len(lib.dmm_status_string(st)) > 0
     assert b"shape" in lib.dmm_status_string(-2)
 
@@ -119,6 +119,17 @@ def test_argument_errors_are_status_codes_not_crashes():
     # the timing hook wants both events or neither
     assert lib.dmm_set_kernel_events(p, None) == -1
     assert lib.dmm_set_kernel_events(None, None) == 0
+    # the benchmark's override of a kernel choice: returns the previous value, refuses what it does not know
+    assert lib.dmm_set_choice(0, -1) == -1 and lib.dmm_set_choice(1, -1) == -1
+    assert lib.dmm_set_choice(2, 0) == -2 and lib.dmm_set_choice(-1, 0) == -2
+    assert lib.dmm_set_choice(0, 3) == -2 and lib.dmm_set_choice(0, -2) == -2
+    try:
+        assert lib.dmm_workspace_bytes(32, 4096, 4096) == 0        # two passes of the small-batch kernel ...
+        assert lib.dmm_set_choice(0, 2) == -1
+        assert lib.dmm_workspace_bytes(32, 4096, 4096) > 0         # ... unless the split is forced
+        assert lib.dmm_set_choice(0, -1) == 2
+    finally:
+        lib.dmm_set_choice(0, -1)
 
 
 def test_operator_rejects_bad_inputs_with_runtime_error():
