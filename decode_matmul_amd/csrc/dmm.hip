@@ -55,6 +55,7 @@ constexpr int kWave = 64;
 #include "dmm_gemv_f16.h"
 #include "dmm_gemv_q8.h"
 #include "dmm_gemv_q8d.h"
+#include "dmm_gemv_f16d.h"
 #include "dmm_gemv_small.h"
 #include "dmm_gemm.h"
 #include "dmm_int8.h"
@@ -181,6 +182,7 @@ const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K)
     if (M > 16) return "dmm::gemv_regx_kernel";
     switch (pick_gemv(M, N, K)) {
         case kGemvStream: return "dmm::gemv_stream_kernel";
+        case kGemvF16d: return "dmm::gemv_f16d_kernel";
         case kGemvQ8: return M > 1 ? "dmm::gemv_q8_kernel" : gemv_q8d_ok(N) ? "dmm::gemv_q8d_kernel" : "dmm::gemv_q8c_kernel";
         default: return "dmm::gemv_regx_kernel";
     }

@@ -71,6 +71,11 @@ const std::vector<KernelInfo> &kernel_table()
         kinfo(gemv_q8d_kernel<3, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<4, 1, 2, P>, kLdsMax, true),     \
         kinfo(gemv_q8d_kernel<6, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<8, 1, 2, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_Q8D),
+#define DMM_K_F16D(P)                                                                                            \
+    kinfo(gemv_f16d_kernel<2, 1, 2, P>, kLdsMax, true),                                                           \
+        kinfo(gemv_f16d_kernel<3, 1, 3, P>, kLdsMax, true), kinfo(gemv_f16d_kernel<4, 1, 2, P>, kLdsMax, true),   \
+        kinfo(gemv_f16d_kernel<6, 1, 3, P>, kLdsMax, true), kinfo(gemv_f16d_kernel<8, 1, 2, P>, kLdsMax, true)
+        DMM_BOTH_LAYOUTS(DMM_K_F16D),
 #define DMM_K_REGX_XI(P, XI)                                                                                      \
     kinfo(gemv_regx_kernel<1, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, P, XI>, kLdsMax, true),     \
         kinfo(gemv_regx_kernel<3, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<4, 8, 2, P, XI>, kLdsMax, true)
@@ -92,6 +97,7 @@ const std::vector<KernelInfo> &kernel_table()
 #undef DMM_K_GREG
 #undef DMM_K_REGX
 #undef DMM_K_REGX_XI
+#undef DMM_K_F16D
 #undef DMM_K_Q8D
 #undef DMM_K_Q8
 #undef DMM_K_STREAM
@@ -293,6 +299,41 @@ int launch_gemv_q8d(const void *x, const void *codes, const void *grid, float sc
     }
 }
 
+// the same loop order on 16-bit operands, for one to four rows of x of any length (x goes through the LDS in
+// chunks): up to 8 tiles per workgroup
+inline bool gemv_f16d_ok(int64_t M, int64_t N, int64_t K)
+{
+    return M >= 1 && M <= 4 && (N + 15) / 16 <= 8 * (int64_t)cu_count() && N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31);
+}
+
+template <int NT, int U, int D, bool kPacked>
+int launch_gemv_f16d_inst(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M, int64_t N,
+                          int64_t K, hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
+    return launch(gemv_f16d_kernel<NT, U, D, kPacked>, dim3((unsigned)wgs), dim3(1024), (size_t)fd_lds_bytes(), stream,
+                  (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+template <bool kPacked>
+int launch_gemv_f16d(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M, int64_t N,
+                     int64_t K, hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
+    switch (share) {
+        case 1:
+        case 2: return launch_gemv_f16d_inst<2, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case 3: return launch_gemv_f16d_inst<3, 1, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case 4: return launch_gemv_f16d_inst<4, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case 5:
+        case 6: return launch_gemv_f16d_inst<6, 1, 3, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        default: return launch_gemv_f16d_inst<8, 1, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+    }
+}
+
 template <int R, int W>
 bool gemv_stream_ok(int64_t M, int64_t N, int64_t K)
 {
@@ -363,20 +404,29 @@ bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok
 // A grid that does not fit fp8 costs them a second table
 // build, and the 16-bit kernel's y is the correctly rounded one.  Otherwise the 16-bit streaming kernel,
 // one tile at a time; the small-batch kernel when x does not fit the LDS.
-enum GemvKind { kGemvQ8, kGemvStream, kGemvRegx };
+enum GemvKind { kGemvQ8, kGemvStream, kGemvF16d, kGemvRegx };
 
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
     const bool long_launch = M == 1 ? n_tiles > cus || K >= 16384 : n_tiles > 4 * cus;
     if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
-    // Two to four rows: the small-batch kernel's eight waves start sooner than the streaming kernel's sixteen
-    // with their x in the LDS, which decides a launch of one tile per workgroup on a short x, and four rows
-    // (graph launches, us, streaming / small-batch: M = 2 4096 -> 4096 4.77 / 4.47, 11008 -> 4096 6.27 / 6.51,
-    // 4096 -> 11008 7.28 / 7.26; M = 4 4096 -> 4096 5.13 / 4.47, 4096 -> 11008 7.63 / 7.45, 4096 -> 12288 7.74 / 7.59;
-    // but M = 2 8192 -> 28672 17.7 / 21.2, M = 3 18.6 / 21.4)
+    // Two to four rows on launches of more than one tile per workgroup: the 16-bit kernel that takes x in chunks
+    // and keeps every tile's sums in registers - up to four tiles per workgroup always (K >= 4096: every wave
+    // has a k step of the chunk), up to eight for four rows or where x does not fit the LDS beside the tables (graph launches,
+    // us, chunked against the kernel that ran before: M = 2 4096 -> 11008 6.4 / 7.2, 4096 -> 12288 6.6 / 7.5,
+    // 8192 -> 8192 7.05 / 7.40, 8192 -> 10240 8.9 / 9.6, 28672 -> 8192 17.8 / 20.3, but 8192 -> 28672 20.1 / 18.8;
+    // M = 4 4096 -> 11008 6.7 / 7.4, 4096 -> 22016 11.4 / 12.5, 8192 -> 10240 8.5 / 9.8, 8192 -> 28672 18.9 / 22.7,
+    // 28672 -> 8192 18.7 / 20.9; with one tile per workgroup 11008 -> 4096 7.5 / 6.6, 28672 -> 4096 12.6 / 11.8).
+    const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
+    const bool x_fits = gemv_stream_ok<1, 16>(M, N, K);
+    if (M >= 2 && M <= 4 && share >= 2 && gemv_f16d_ok(M, N, K) && (x_fits ? (share <= 4 || M == 4) && K >= 4096 : true))
+        return kGemvF16d;
+    // Otherwise the small-batch kernel's eight waves start sooner than the streaming kernel's sixteen with
+    // their x in the LDS, which decides a launch of one tile per workgroup on a short x, and four rows (M = 2
+    // 4096 -> 4096 4.77 / 4.47, 11008 -> 4096 6.27 / 6.51; M = 4 4096 -> 4096 5.13 / 4.47)
     const bool small_first = M == 4 || (M >= 2 && M <= 4 && n_tiles <= cus && K <= 4096);
-    if (!small_first && gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
+    if (!small_first && x_fits) return kGemvStream;
     return kGemvRegx;
 }
 
@@ -426,6 +476,7 @@ int run_gemv(const void *x, const void *codes, const void *grid, float scale, vo
     if (M > 16) return run_gemv_regx<kPacked>(x, codes, grid, scale, y, M, N, K, stream);   // 16 rows per pass
     switch (pick_gemv(M, N, K)) {
         case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
+        case kGemvF16d: return launch_gemv_f16d<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         case kGemvStream: return launch_gemv_stream<1, 16, 2, kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         default: return run_gemv_regx<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
     }

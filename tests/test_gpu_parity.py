@@ -315,7 +315,12 @@ def test_gemv_8bit_switch_and_kernel_name():
         assert lib.dmm_gemv_kernel_name(4, 12288, K) == b"dmm::gemv_regx_kernel"      # four rows: the small-batch kernel
         assert lib.dmm_gemv_kernel_name(2, 4096, K) == b"dmm::gemv_regx_kernel"       # one tile per CU, short x
         assert lib.dmm_gemv_kernel_name(2, 4096, 8192) == b"dmm::gemv_stream_kernel"
-        assert lib.dmm_gemv_kernel_name(3, N, 28672) == b"dmm::gemv_regx_kernel"      # their terms do not fit
+        assert lib.dmm_gemv_kernel_name(3, N, 28672) == b"dmm::gemv_f16d_kernel"      # x does not fit the LDS: in chunks
+        assert lib.dmm_gemv_kernel_name(3, 4096, 28672) == b"dmm::gemv_regx_kernel"   # ... but not for one tile per CU
+        assert lib.dmm_gemv_kernel_name(2, 12288, 4096) == b"dmm::gemv_f16d_kernel"   # up to four tiles, K >= 4096
+        assert lib.dmm_gemv_kernel_name(2, 28672, 8192) == b"dmm::gemv_stream_kernel" # more tiles, x fits
+        assert lib.dmm_gemv_kernel_name(4, 28672, 4096) == b"dmm::gemv_f16d_kernel"   # four rows: up to eight tiles
+        assert lib.dmm_gemv_kernel_name(2, 28672, 4096) == b"dmm::gemv_q8_kernel"     # short x, many tiles: 8-bit
         assert lib.dmm_gemv_kernel_name(32, N, K) == b"dmm::gemv_regx_kernel"
         assert lib.dmm_gemv_kernel_name(M, N, 264) == b""
         y8 = c_matmul(dev(x), dev(codes), dev(grid), scale, "auto")
@@ -429,6 +434,37 @@ def test_gemv_8bit_every_share_of_tiles_is_exact(N, K):
     if (N + 15) // 16 > 2 * 256:
         name = lib.dmm_gemv_kernel_name(1, N, K)
         assert name == (b"dmm::gemv_q8d_kernel" if (N + 15) // 16 <= 8 * 256 else b"dmm::gemv_q8c_kernel")
+
+
+@pytest.mark.parametrize("M,N,K", [(2, 6000, 16384), (4, 4112, 8448), (4, 12272, 7168), (3, 16400, 11008), (4, 20000, 8192),
+                                   (2, 24592, 16384), (4, 28672, 8192), (4, 32768, 7168), (2, 8192, 28672), (3, 4100, 28672)])
+def test_chunked_16bit_kernel_is_exact(M, N, K):
+    """Two to four rows of an x that does not fit the LDS beside the tables, on the 16-bit kernel that takes x
+    in chunks, exactly (the integer bridge): workgroups of one to eight row tiles (launches of two to eight per
+    workgroup at most), two to seven chunks with a
+    last chunk that is not full, rows of x to spare in the buffer.  Reference: the library's own decode
+    (pinned bit for bit against the oracle above) times x in fp64 on the GPU, which is exact for these
+    integers, plus the oracle's integer product on the first and last rows of W."""
+    assert capi.lib().dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_f16d_kernel"
+    rng = np.random.default_rng(M + N + K)
+    cb = orc.build_codebook_abs()
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(M * N + K)
+    codes = torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=DEV)
+    scale = 2.0 ** -8
+    xd, gd = dev(x.astype(np.float16)), dev(orc.grid_from_codebook(cb))
+    buf = torch.full((64 + M * N + 64,), -7.0, dtype=torch.float16, device=DEV)
+    y = buf[64:64 + M * N].view(M, N)
+    c_matmul(xd, codes, gd, scale, "gemv", out=y)
+    W = c_decode(codes, gd)
+    torch.cuda.synchronize()
+    want = ((xd.double() @ W.double().T) * scale).to(torch.float16)
+    assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+    assert torch.all(buf[:64] == -7.0) and torch.all(buf[64 + M * N:] == -7.0)
+    rows = np.concatenate([np.arange(min(24, N)), np.arange(max(N - 24, 0), N)])
+    yi = orc.decode_matmul_i32(x, codes[torch.from_numpy(rows).to(DEV)].cpu().numpy(), cb)
+    assert np.array_equal(bits(y[:, torch.from_numpy(rows).to(DEV)].contiguous()), bits((yi.astype(np.float64) / 4 * scale).astype(np.float16)))
 
 
 def test_reference_shape_golden_case():
@@ -655,7 +691,8 @@ def test_matrix_matrix_with_y_only_2_byte_aligned(M, N, K):
 
 
 # ----------------------------------------------------------------- small-batch kernel, row blocks
-@pytest.mark.parametrize("M,K", [(8, 4096), (16, 4096), (3, 28672), (12, 1024 * 5), (2, 28672), (5, 16384), (9, 8192)])
+@pytest.mark.parametrize("M,K", [(8, 4096), (16, 4096), (3, 28672), (12, 1024 * 5), (2, 28672), (5, 16384), (9, 8192),
+                                 (4, 4096), (4, 3328)])
 @pytest.mark.parametrize("share", [1, 2, 3, 4, 5, 7, 8])
 def test_small_batch_row_block_sizes(M, K, share):
     """The register-x kernel takes one to four row tiles per block, chosen from the most tiles
@@ -666,7 +703,11 @@ def test_small_batch_row_block_sizes(M, K, share):
     in fp32 on the GPU, plus the oracle itself on the first and last rows."""
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     N = 16 * (cus * share - 37) - 4
-    assert capi.lib().dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_regx_kernel"
+    # up to four rows of x on more than one tile per workgroup go to the chunked 16-bit kernel from K = 4096 on
+    # (every share of tiles it is instantiated for comes by here as well); everything else in this list to the
+    # register-x kernel
+    chunked = M <= 4 and share >= 2 and K >= 4096
+    assert capi.lib().dmm_gemv_kernel_name(M, N, K) == (b"dmm::gemv_f16d_kernel" if chunked else b"dmm::gemv_regx_kernel")
     x, _, grid, scale = workload.make_inputs(M, 8, K, seed=share)
     g = torch.Generator(device=DEV)
     g.manual_seed(1000 * M + share)
