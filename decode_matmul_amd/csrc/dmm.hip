@@ -163,7 +163,7 @@ int dmm_set_gemv_8bit(int enabled)
 
 int dmm_set_choice(int which, int value)
 {
-    if (which < 0 || which > 1 || value < -1 || value > 2) return DMM_ERR_BAD_SHAPE;
+    if (which < 0 || which > 2 || value < -1 || value > 2) return DMM_ERR_BAD_SHAPE;
     return g_choice[which].exchange(value, std::memory_order_relaxed);
 }
 

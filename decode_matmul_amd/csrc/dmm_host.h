@@ -356,9 +356,10 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
 
 // dmm_set_choice: what a benchmark that checks the operator's choices forces instead (-1: nothing).
 // [0]: more than 16 rows of x (0 passes of the small-batch kernel, 1 matrix-matrix kernel, 2 split K);
-// [1]: the integer operator on more than 16 rows (1 passes of the matrix-vector kernel, 2 matrix-matrix).
+// [1]: the integer operator on more than 16 rows (1 passes of the matrix-vector kernel, 2 matrix-matrix);
+// [2]: two to four rows of x (0 never the 16-bit kernel that takes x in chunks, 1 wherever it can run).
 // A forced kernel that cannot take the call leaves the choice to the library.
-std::atomic<int> g_choice[2] = {{-1}, {-1}};
+std::atomic<int> g_choice[3] = {{-1}, {-1}, {-1}};
 
 // Whether the operator may pick the 8-bit kernel: dmm_set_gemv_8bit, or DMM_GEMV_8BIT=0 in the
 // environment (read once, at the first call that needs it) for hosts that cannot call it.
@@ -420,7 +421,10 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
     // 28672 -> 8192 18.7 / 20.9; with one tile per workgroup 11008 -> 4096 7.5 / 6.6, 28672 -> 4096 12.6 / 11.8).
     const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
     const bool x_fits = gemv_stream_ok<1, 16>(M, N, K);
-    if (M >= 2 && M <= 4 && share >= 2 && gemv_f16d_ok(M, N, K) && (x_fits ? (share <= 4 || M == 4) && K >= 4096 : true))
+    const int force = M >= 2 && M <= 4 ? g_choice[2].load(std::memory_order_relaxed) : -1;
+    if (force == 1 && gemv_f16d_ok(M, N, K)) return kGemvF16d;
+    if (force != 0 && M >= 2 && M <= 4 && share >= 2 && gemv_f16d_ok(M, N, K) &&
+        (x_fits ? (share <= 4 || M == 4) && K >= 4096 : true))
         return kGemvF16d;
     // Otherwise the small-batch kernel's eight waves start sooner than the streaming kernel's sixteen with
     // their x in the LDS, which decides a launch of one tile per workgroup on a short x, and four rows (M = 2

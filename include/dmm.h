@@ -247,7 +247,8 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K);
  * small-batch kernel, 16 rows each; 1: the matrix-matrix kernel; 2: split K, where a workspace is
  * given - dmm_workspace_bytes then answers for the split as well).  which = 1: the integer
  * operator on more than 16 rows (1: passes of the matrix-vector kernel, 2: the matrix-matrix
- * kernel).  value -1: the library's own choice (the default).  A forced kernel that cannot take a
+ * kernel).  which = 2: two to four rows of x (0: never the 16-bit kernel that takes x in chunks,
+ * 1: wherever it can run).  value -1: the library's own choice (the default).  A forced kernel that cannot take a
  * call (shape, alignment) leaves that call to the library's choice; results do not depend on
  * the setting beyond what the kernels' own summation orders differ by (the integer operator:
  * not at all).  Returns the previous value (>= -1), or DMM_ERR_BAD_SHAPE for arguments out of

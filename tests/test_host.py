@@ -121,7 +121,8 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert lib.dmm_set_kernel_events(None, None) == 0
     # the benchmark's override of a kernel choice: returns the previous value, refuses what it does not know
     assert lib.dmm_set_choice(0, -1) == -1 and lib.dmm_set_choice(1, -1) == -1
-    assert lib.dmm_set_choice(2, 0) == -2 and lib.dmm_set_choice(-1, 0) == -2
+    assert lib.dmm_set_choice(3, 0) == -2 and lib.dmm_set_choice(-1, 0) == -2
+    assert lib.dmm_set_choice(2, -1) == -1
     assert lib.dmm_set_choice(0, 3) == -2 and lib.dmm_set_choice(0, -2) == -2
     try:
         assert lib.dmm_workspace_bytes(32, 4096, 4096) == 0        # two passes of the small-batch kernel ...
