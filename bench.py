@@ -945,23 +945,23 @@ def dispatch_check(torch, lib, capi, workload, dev):
                 lib.dmm_set_gemv_8bit(was)
             add("pick_gemv", M, K, N, times, {"kernel": lib.dmm_gemv_kernel_name(M, N, K).decode()})
 
-    # ---- two to four rows: the 16-bit kernel that takes x in chunks against the kernels that served before it
-    for M in (2, 4):
-        for K, N in ((4096, 11008), (4096, 12288), (4096, 22016), (11008, 4096), (8192, 8192), (8192, 10240),
-                     (8192, 28672), (28672, 8192)):
+    # ---- up to eight rows: the 16-bit kernel with resident sums against the kernels that served before it
+    for M in (2, 4, 8):
+        for K, N in ((4096, 11008), (4096, 22016), (11008, 4096), (8192, 8192), (8192, 10240), (8192, 28672),
+                     (28672, 8192), (1024, 16384)):
             x, grid, scale = half_inputs(M, K)
             y = torch.empty(M, N, dtype=torch.float16, device=dev)
 
             def op2(c, s):
                 return lib.dmm_decode_matmul_f16(x.data_ptr(), c, grid.data_ptr(), scale, y.data_ptr(), M, N, K, s)
             times = {"operator": graph_us(op2, workload.code_bytes(N, K))}
-            for name, value in (("streaming or small-batch", 0), ("chunked", 1)):
+            for name, value in (("streaming, small-batch or 8-bit", 0), ("resident sums", 1)):
                 was = lib.dmm_set_choice(2, value)
                 try:
                     times[name] = graph_us(op2, workload.code_bytes(N, K))
                 finally:
                     lib.dmm_set_choice(2, was)
-            add("pick_gemv, chunked x", M, K, N, times, {"kernel": lib.dmm_gemv_kernel_name(M, N, K).decode()})
+            add("pick_gemv, resident sums", M, K, N, times, {"kernel": lib.dmm_gemv_kernel_name(M, N, K).decode()})
 
     # ---- 17 .. 32 rows with a workspace (passes against split K), more rows (passes against the matrix-matrix
     # kernel, with and without a workspace)

@@ -71,10 +71,11 @@ const std::vector<KernelInfo> &kernel_table()
         kinfo(gemv_q8d_kernel<3, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<4, 1, 2, P>, kLdsMax, true),     \
         kinfo(gemv_q8d_kernel<6, 1, 3, P>, kLdsMax, true), kinfo(gemv_q8d_kernel<8, 1, 2, P>, kLdsMax, true)
         DMM_BOTH_LAYOUTS(DMM_K_Q8D),
-#define DMM_K_F16D(P)                                                                                            \
-    kinfo(gemv_f16d_kernel<2, 1, 2, P>, kLdsMax, true),                                                           \
-        kinfo(gemv_f16d_kernel<3, 1, 3, P>, kLdsMax, true), kinfo(gemv_f16d_kernel<4, 1, 2, P>, kLdsMax, true),   \
-        kinfo(gemv_f16d_kernel<6, 1, 3, P>, kLdsMax, true), kinfo(gemv_f16d_kernel<8, 1, 2, P>, kLdsMax, true)
+#define DMM_K_F16D_XI(P, XI)                                                                                      \
+    kinfo(gemv_f16d_kernel<2, 1, 2, P, XI>, kLdsMax, true), kinfo(gemv_f16d_kernel<3, 1, 3, P, XI>, kLdsMax, true),     \
+        kinfo(gemv_f16d_kernel<4, 1, 2, P, XI>, kLdsMax, true), kinfo(gemv_f16d_kernel<6, 1, 3, P, XI>, kLdsMax, true), \
+        kinfo(gemv_f16d_kernel<8, 1, 2, P, XI>, kLdsMax, true)
+#define DMM_K_F16D(P) DMM_K_F16D_XI(P, 2), DMM_K_F16D_XI(P, 4)
         DMM_BOTH_LAYOUTS(DMM_K_F16D),
 #define DMM_K_REGX_XI(P, XI)                                                                                      \
     kinfo(gemv_regx_kernel<1, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, P, XI>, kLdsMax, true),     \
@@ -98,6 +99,7 @@ const std::vector<KernelInfo> &kernel_table()
 #undef DMM_K_REGX
 #undef DMM_K_REGX_XI
 #undef DMM_K_F16D
+#undef DMM_K_F16D_XI
 #undef DMM_K_Q8D
 #undef DMM_K_Q8
 #undef DMM_K_STREAM
@@ -299,11 +301,11 @@ int launch_gemv_q8d(const void *x, const void *codes, const void *grid, float sc
     }
 }
 
-// the same loop order on 16-bit operands, for one to four rows of x of any length (x goes through the LDS in
-// chunks): up to 8 tiles per workgroup
+// the same loop order on 16-bit operands, for up to eight rows of x of any length (a wave fetches the x of its
+// k steps itself): up to 8 tiles per workgroup
 inline bool gemv_f16d_ok(int64_t M, int64_t N, int64_t K)
 {
-    return M >= 1 && M <= 4 && (N + 15) / 16 <= 8 * (int64_t)cu_count() && N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31);
+    return M >= 1 && M <= 8 && (N + 15) / 16 <= 8 * (int64_t)cu_count() && N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31);
 }
 
 template <int NT, int U, int D, bool kPacked>
@@ -312,7 +314,11 @@ int launch_gemv_f16d_inst(const void *x, const void *codes, const void *grid, fl
 {
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
-    return launch(gemv_f16d_kernel<NT, U, D, kPacked>, dim3((unsigned)wgs), dim3(1024), (size_t)fd_lds_bytes(), stream,
+    if (M <= 4)
+        return launch(gemv_f16d_kernel<NT, U, D, kPacked, 2>, dim3((unsigned)wgs), dim3(1024), (size_t)fd_lds_bytes(2), stream,
+                      (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                      (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    return launch(gemv_f16d_kernel<NT, U, D, kPacked, 4>, dim3((unsigned)wgs), dim3(1024), (size_t)fd_lds_bytes(4), stream,
                   (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }
@@ -400,8 +406,7 @@ bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok
 // 28672 -> 8192 14.0 / 16.2, 8192 -> 10240 6.9 / 8.7, 8192 -> 8192 6.2 / 7.2, 8192 -> 4352 5.9 / 6.8, 4096 -> 8192
 // 4.7 / 5.3, 4096 -> 4352 4.4 / 5.2, 11008 -> 8192 7.6 / 8.2, 11008 -> 4352 7.0 / 7.7, 28672 -> 4096 10.4 / 11.0;
 // but with one tile per workgroup 4096 -> 4096 4.22 / 4.21, 8192 -> 4096 4.97 / 4.89, 11008 -> 4096 5.98 / 5.48).
-// Two to four rows from more than four tiles on (M = 2, 8-bit / 16-bit: 4096 -> 22016 10.1 / 11.0, 4096 -> 32000
-// 12.4 / 14.1, but 4096 -> 16384 8.7 / 8.7, 4096 -> 12544 8.5 / 8.3; M = 4: 3072 -> 16384 8.6 / 8.2, 3072 -> 12544 8.4 / 7.8).
+// Two to four rows only beyond eight tiles per workgroup (below, the 16-bit kernel with resident sums is faster).
 // A grid that does not fit fp8 costs them a second table
 // build, and the 16-bit kernel's y is the correctly rounded one.  Otherwise the 16-bit streaming kernel,
 // one tile at a time; the small-batch kernel when x does not fit the LDS.
@@ -410,27 +415,28 @@ enum GemvKind { kGemvQ8, kGemvStream, kGemvF16d, kGemvRegx };
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
-    const bool long_launch = M == 1 ? n_tiles > cus || K >= 16384 : n_tiles > 4 * cus;
-    if (long_launch && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
-    // Two to four rows on launches of more than one tile per workgroup: the 16-bit kernel that takes x in chunks
-    // and keeps every tile's sums in registers - up to four tiles per workgroup always (K >= 4096: every wave
-    // has a k step of the chunk), up to eight for four rows or where x does not fit the LDS beside the tables (graph launches,
-    // us, chunked against the kernel that ran before: M = 2 4096 -> 11008 6.4 / 7.2, 4096 -> 12288 6.6 / 7.5,
-    // 8192 -> 8192 7.05 / 7.40, 8192 -> 10240 8.9 / 9.6, 28672 -> 8192 17.8 / 20.3, but 8192 -> 28672 20.1 / 18.8;
-    // M = 4 4096 -> 11008 6.7 / 7.4, 4096 -> 22016 11.4 / 12.5, 8192 -> 10240 8.5 / 9.8, 8192 -> 28672 18.9 / 22.7,
-    // 28672 -> 8192 18.7 / 20.9; with one tile per workgroup 11008 -> 4096 7.5 / 6.6, 28672 -> 4096 12.6 / 11.8).
     const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
-    const bool x_fits = gemv_stream_ok<1, 16>(M, N, K);
-    const int force = M >= 2 && M <= 4 ? g_choice[2].load(std::memory_order_relaxed) : -1;
+    if (M == 1 && (n_tiles > cus || K >= 16384) && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
+    // Up to eight rows on launches of more than one and up to eight tiles per workgroup: the 16-bit kernel that keeps
+    // every tile's sums in registers and has each wave fetch the x of its own k steps.  It beats what served
+    // before it at every such shape measured (graph launches, us, this kernel / before: M = 2 4096 -> 11008
+    // 6.2 / 7.2, 8192 -> 8192 6.45 / 7.40, 8192 -> 10240 8.0 / 9.6, 8192 -> 28672 17.3 / 18.6, 28672 -> 8192 16.6 / 20.3,
+    // 2048 -> 16384 5.25 / 7.02, 256 -> 32768 6.45 / 13.66; M = 4 8192 -> 28672 16.9 / 22.7, 28672 -> 8192 17.7 / 20.9;
+    // M = 8 8192 -> 10240 9.6 / 10.7, 8192 -> 28672 18.4 / 24.2, 4096 -> 22016 10.6 / 12.8; one row with the 8-bit
+    // kernels off: 8192 -> 28672 16.6 / 18.0, 4096 -> 22016 9.3 / 11.3), the 8-bit kernel for two to four rows
+    // included (M = 2 4096 -> 22016 9.5 / 10.4, 4096 -> 32000 10.1 / 11.75; M = 4 3072 -> 32768 9.7 / 11.8).  With
+    // one tile per workgroup it is level with them or behind (M = 1 11008 -> 4096 6.03 / 5.63, M = 4 6.31 / 6.71).
+    const int force = M <= 8 ? g_choice[2].load(std::memory_order_relaxed) : -1;
     if (force == 1 && gemv_f16d_ok(M, N, K)) return kGemvF16d;
-    if (force != 0 && M >= 2 && M <= 4 && share >= 2 && gemv_f16d_ok(M, N, K) &&
-        (x_fits ? (share <= 4 || M == 4) && K >= 4096 : true))
-        return kGemvF16d;
-    // Otherwise the small-batch kernel's eight waves start sooner than the streaming kernel's sixteen with
-    // their x in the LDS, which decides a launch of one tile per workgroup on a short x, and four rows (M = 2
+    if (force != 0 && share >= 2 && gemv_f16d_ok(M, N, K)) return kGemvF16d;
+    // Beyond eight tiles per workgroup: two to four rows on 8-bit operands where their x fits the LDS
+    if (M >= 2 && n_tiles > 4 * cus && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
+    // Otherwise the 16-bit streaming kernel, one tile at a time, or the small-batch kernel when x does not fit the
+    // LDS - and for two to four rows on a launch of one tile per workgroup with a short x, and for four rows,
+    // where its eight waves start sooner than the streaming kernel's sixteen with their x in the LDS (M = 2
     // 4096 -> 4096 4.77 / 4.47, 11008 -> 4096 6.27 / 6.51; M = 4 4096 -> 4096 5.13 / 4.47)
     const bool small_first = M == 4 || (M >= 2 && M <= 4 && n_tiles <= cus && K <= 4096);
-    if (!small_first && x_fits) return kGemvStream;
+    if (!small_first && gemv_stream_ok<1, 16>(M, N, K)) return kGemvStream;
     return kGemvRegx;
 }
 

@@ -208,12 +208,15 @@ def test_gemv_8bit_one_row_of_x_in_chunks(N, K, grid_kind):
     assert torch.equal(ya, yp)                   # packed codes: same kernel choice, same arithmetic, same order
     if (N + 15) // 16 > 2 * 256:
         assert torch.equal(y, ya)                # launches this long take the 8-bit kernel by themselves
-    if grid_kind == "half_any":                  # handed over: exactly the 16-bit kernel's result
+    if grid_kind == "half_any":                  # handed over: exactly the 16-bit streaming kernel's result
         was = capi.lib().dmm_set_gemv_8bit(0)
+        was2 = capi.lib().dmm_set_choice(2, 0)   # (with the 8-bit kernels off the operator would take the other 16-bit one)
         try:
+            assert capi.lib().dmm_gemv_kernel_name(1, N, K) == b"dmm::gemv_stream_kernel"
             y16 = c_matmul(dev(x), dev(codes), dev(grid), scale, "gemv")
         finally:
             capi.lib().dmm_set_gemv_8bit(was)
+            capi.lib().dmm_set_choice(2, was2)
         assert torch.equal(y, y16)
 
 
@@ -309,24 +312,24 @@ def test_gemv_8bit_switch_and_kernel_name():
         assert lib.dmm_gemv_kernel_name(M, N, 28672) == b"dmm::gemv_q8d_kernel"       # x goes through in chunks
         assert lib.dmm_gemv_kernel_name(M, 32768, K) == b"dmm::gemv_q8d_kernel"       # eight tiles per CU
         assert lib.dmm_gemv_kernel_name(M, 32784, K) == b"dmm::gemv_q8c_kernel"       # more: groups of three tiles
-        assert lib.dmm_gemv_kernel_name(3, 32768, K) == b"dmm::gemv_q8_kernel"        # two to four rows of x, many tiles
-        assert lib.dmm_gemv_kernel_name(3, N, K) == b"dmm::gemv_stream_kernel"        # four tiles per CU: not yet
-        assert lib.dmm_gemv_kernel_name(3, 12288, K) == b"dmm::gemv_stream_kernel"
-        assert lib.dmm_gemv_kernel_name(4, 12288, K) == b"dmm::gemv_regx_kernel"      # four rows: the small-batch kernel
+        # up to eight rows on two to eight tiles per CU: the 16-bit kernel with resident sums, whatever K
+        for m in (2, 3, 4, 5, 8):
+            for n, k in ((N, K), (12288, K), (8192, 256), (32768, K), (N, 28672), (28672, 8192), (4112, 4096)):
+                assert lib.dmm_gemv_kernel_name(m, n, k) == b"dmm::gemv_f16d_kernel", (m, n, k)
+        assert lib.dmm_gemv_kernel_name(3, 32784, K) == b"dmm::gemv_q8_kernel"        # more tiles, two to four rows: 8-bit
+        assert lib.dmm_gemv_kernel_name(5, 32784, K) == b"dmm::gemv_stream_kernel"
+        assert lib.dmm_gemv_kernel_name(9, N, K) == b"dmm::gemv_stream_kernel"        # more rows
+        assert lib.dmm_gemv_kernel_name(9, N, 8192) == b"dmm::gemv_regx_kernel"       # ... whose x does not fit the LDS
         assert lib.dmm_gemv_kernel_name(2, 4096, K) == b"dmm::gemv_regx_kernel"       # one tile per CU, short x
         assert lib.dmm_gemv_kernel_name(2, 4096, 8192) == b"dmm::gemv_stream_kernel"
-        assert lib.dmm_gemv_kernel_name(3, N, 28672) == b"dmm::gemv_f16d_kernel"      # x does not fit the LDS: in chunks
-        assert lib.dmm_gemv_kernel_name(3, 4096, 28672) == b"dmm::gemv_regx_kernel"   # ... but not for one tile per CU
-        assert lib.dmm_gemv_kernel_name(2, 12288, 4096) == b"dmm::gemv_f16d_kernel"   # up to four tiles, K >= 4096
-        assert lib.dmm_gemv_kernel_name(2, 28672, 8192) == b"dmm::gemv_stream_kernel" # more tiles, x fits
-        assert lib.dmm_gemv_kernel_name(4, 28672, 4096) == b"dmm::gemv_f16d_kernel"   # four rows: up to eight tiles
-        assert lib.dmm_gemv_kernel_name(2, 28672, 4096) == b"dmm::gemv_q8_kernel"     # short x, many tiles: 8-bit
+        assert lib.dmm_gemv_kernel_name(3, 4096, 28672) == b"dmm::gemv_regx_kernel"
         assert lib.dmm_gemv_kernel_name(32, N, K) == b"dmm::gemv_regx_kernel"
         assert lib.dmm_gemv_kernel_name(M, N, 264) == b""
         y8 = c_matmul(dev(x), dev(codes), dev(grid), scale, "auto")
         assert torch.equal(y8, c_matmul(dev(x), dev(codes), dev(grid), scale, "gemv8"))
         assert lib.dmm_set_gemv_8bit(0) == 1
-        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_stream_kernel"
+        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_f16d_kernel"
+        assert lib.dmm_gemv_kernel_name(M, 4096, K) == b"dmm::gemv_stream_kernel"
         y16 = c_matmul(dev(x), dev(codes), dev(grid), scale, "auto")
         torch.cuda.synchronize()
         assert_close_to_oracle(y8, ref, "8-bit")
@@ -437,26 +440,33 @@ def test_gemv_8bit_every_share_of_tiles_is_exact(N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(2, 6000, 16384), (4, 4112, 8448), (4, 12272, 7168), (3, 16400, 11008), (4, 20000, 8192),
-                                   (2, 24592, 16384), (4, 28672, 8192), (4, 32768, 7168), (2, 8192, 28672), (3, 4100, 28672)])
+                                   (2, 24592, 16384), (4, 28672, 8192), (4, 32768, 7168), (2, 8192, 28672), (3, 4100, 28672),
+                                   (8, 4112, 8192), (6, 20000, 4096), (8, 28672, 4096), (5, 8192, 28672), (8, 12272, 256),
+                                   (7, 32768, 512), (1, 16400, 4352), (5, 24592, 1280)])
 def test_chunked_16bit_kernel_is_exact(M, N, K):
-    """Two to four rows of an x that does not fit the LDS beside the tables, on the 16-bit kernel that takes x
-    in chunks, exactly (the integer bridge): workgroups of one to eight row tiles (launches of two to eight per
-    workgroup at most), two to seven chunks with a
-    last chunk that is not full, rows of x to spare in the buffer.  Reference: the library's own decode
+    """Up to eight rows of x on the 16-bit kernel with resident sums, exactly (the integer bridge): both widths
+    of the x slice (up to four and up to eight rows, full and with rows to spare), workgroups of one to eight row
+    tiles (launches of two to eight per workgroup at most), one to seven chunks with a last chunk that is not
+    full, fewer k steps than waves, one row of x with the 8-bit kernels switched off.  Reference: the library's own decode
     (pinned bit for bit against the oracle above) times x in fp64 on the GPU, which is exact for these
     integers, plus the oracle's integer product on the first and last rows of W."""
-    assert capi.lib().dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_f16d_kernel"
-    rng = np.random.default_rng(M + N + K)
-    cb = orc.build_codebook_abs()
-    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
-    g = torch.Generator(device=DEV)
-    g.manual_seed(M * N + K)
-    codes = torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=DEV)
-    scale = 2.0 ** -8
-    xd, gd = dev(x.astype(np.float16)), dev(orc.grid_from_codebook(cb))
-    buf = torch.full((64 + M * N + 64,), -7.0, dtype=torch.float16, device=DEV)
-    y = buf[64:64 + M * N].view(M, N)
-    c_matmul(xd, codes, gd, scale, "gemv", out=y)
+    lib = capi.lib()
+    was = lib.dmm_set_gemv_8bit(0 if M == 1 else 1)
+    try:
+        assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_f16d_kernel"
+        rng = np.random.default_rng(M + N + K)
+        cb = orc.build_codebook_abs()
+        x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+        g = torch.Generator(device=DEV)
+        g.manual_seed(M * N + K)
+        codes = torch.randint(-32768, 32768, (N, K // 8), generator=g, dtype=torch.int16, device=DEV)
+        scale = 2.0 ** -8
+        xd, gd = dev(x.astype(np.float16)), dev(orc.grid_from_codebook(cb))
+        buf = torch.full((64 + M * N + 64,), -7.0, dtype=torch.float16, device=DEV)
+        y = buf[64:64 + M * N].view(M, N)
+        c_matmul(xd, codes, gd, scale, "gemv", out=y)
+    finally:
+        lib.dmm_set_gemv_8bit(was)
     W = c_decode(codes, gd)
     torch.cuda.synchronize()
     want = ((xd.double() @ W.double().T) * scale).to(torch.float16)
@@ -693,7 +703,7 @@ def test_matrix_matrix_with_y_only_2_byte_aligned(M, N, K):
 # ----------------------------------------------------------------- small-batch kernel, row blocks
 @pytest.mark.parametrize("M,K", [(8, 4096), (16, 4096), (3, 28672), (12, 1024 * 5), (2, 28672), (5, 16384), (9, 8192),
                                  (4, 4096), (4, 3328)])
-@pytest.mark.parametrize("share", [1, 2, 3, 4, 5, 7, 8])
+@pytest.mark.parametrize("share", [1, 2, 3, 4, 5, 7, 8, 9, 11])
 def test_small_batch_row_block_sizes(M, K, share):
     """The register-x kernel takes one to four row tiles per block, chosen from the most tiles
     a workgroup gets (`share`): every choice, with workgroups whose last block is partial and
@@ -703,11 +713,11 @@ def test_small_batch_row_block_sizes(M, K, share):
     in fp32 on the GPU, plus the oracle itself on the first and last rows."""
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     N = 16 * (cus * share - 37) - 4
-    # up to four rows of x on more than one tile per workgroup go to the chunked 16-bit kernel from K = 4096 on
-    # (every share of tiles it is instantiated for comes by here as well); everything else in this list to the
+    # up to eight rows of x on two to eight tiles per workgroup go to the 16-bit kernel with resident sums (every
+    # share of tiles it is instantiated for comes by here as well); everything else in this list to the
     # register-x kernel
-    chunked = M <= 4 and share >= 2 and K >= 4096
-    assert capi.lib().dmm_gemv_kernel_name(M, N, K) == (b"dmm::gemv_f16d_kernel" if chunked else b"dmm::gemv_regx_kernel")
+    resident = M <= 8 and 2 <= share <= 8
+    assert capi.lib().dmm_gemv_kernel_name(M, N, K) == (b"dmm::gemv_f16d_kernel" if resident else b"dmm::gemv_regx_kernel")
     x, _, grid, scale = workload.make_inputs(M, 8, K, seed=share)
     g = torch.Generator(device=DEV)
     g.manual_seed(1000 * M + share)
@@ -1051,7 +1061,7 @@ def test_graph_capture_and_replay():
     with eager work and synchronisations between the replays, after x has been changed in
     place (a replay must read the current contents of its buffers)."""
     shapes = [(1, 1024, 4096), (1, 4096, 1024), (8, 512, 2048), (160, 384, 512),
-              (1, 16384, 512), (3, 16400, 768),      # the 8-bit kernel, batch 1 and batch 3
+              (1, 16384, 512), (3, 16400, 768),      # the 8-bit kernel, and three rows on the 16-bit kernel with resident sums
               (12, 4800, 5120)]                      # the register-x kernel
     probs = []
     for i, (M, N, K) in enumerate(shapes):
