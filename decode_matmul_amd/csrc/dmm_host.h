@@ -363,7 +363,7 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
 // dmm_set_choice: what a benchmark that checks the operator's choices forces instead (-1: nothing).
 // [0]: more than 16 rows of x (0 passes of the small-batch kernel, 1 matrix-matrix kernel, 2 split K);
 // [1]: the integer operator on more than 16 rows (1 passes of the matrix-vector kernel, 2 matrix-matrix);
-// [2]: two to four rows of x (0 never the 16-bit kernel that takes x in chunks, 1 wherever it can run).
+// [2]: up to eight rows of x (0 never the 16-bit kernel with resident sums, 1 wherever it can run).
 // A forced kernel that cannot take the call leaves the choice to the library.
 std::atomic<int> g_choice[3] = {{-1}, {-1}, {-1}};
 

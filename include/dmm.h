@@ -148,7 +148,7 @@ int dmm_gemv_f16(const void *x, const void *codes, const void *grid, float scale
 /*   dmm_gemv_8bit_f16  the matrix-vector kernels on 8-bit MFMA operands, which dmm_gemv_f16 and
  *                    the operator pick for M = 1 on launches of more than one 16-row tile per
  *                    compute unit (from one on when K >= 16384) and for M = 2 .. 4 on launches of
- *                    more than four (shorter ones gain nothing from them).  Weights as fp8 (e4m3) bytes - exact when
+ *                    more than eight (below that a 16-bit kernel is faster).  Weights as fp8 (e4m3) bytes - exact when
  *                    every grid value has at most 4 significant bits in fp8's range, as the E8P
  *                    grid does - and x as four bf8 (e5m2) terms that add up to it exactly; the
  *                    +-1/4 shift of a code is added through the per-code means of x (two halves,
@@ -179,8 +179,8 @@ int dmm_set_gemv_8bit(int enabled);
 /* Which matrix-vector kernel the operator runs for a shape with aligned pointers, as a profiler's
  * kernel trace names it without the template arguments ("dmm::gemv_q8d_kernel" - one row of x on
  * 8-bit operands, up to eight row tiles per compute unit -, "dmm::gemv_q8c_kernel" - the same for
- * more tiles -, "dmm::gemv_q8_kernel", "dmm::gemv_stream_kernel", "dmm::gemv_f16d_kernel" - two to four
- * rows on 16-bit operands with x taken in chunks -, "dmm::gemv_regx_kernel"; ""
+ * more tiles -, "dmm::gemv_q8_kernel", "dmm::gemv_stream_kernel", "dmm::gemv_f16d_kernel" - up to eight
+ * rows on 16-bit operands, two to eight row tiles per compute unit -, "dmm::gemv_regx_kernel"; ""
  * outside dmm_gemv_f16's domain).  For
  * benchmarks that report per kernel.  Static storage.  No counterpart in the reference. */
 const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K);
@@ -247,8 +247,8 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K);
  * small-batch kernel, 16 rows each; 1: the matrix-matrix kernel; 2: split K, where a workspace is
  * given - dmm_workspace_bytes then answers for the split as well).  which = 1: the integer
  * operator on more than 16 rows (1: passes of the matrix-vector kernel, 2: the matrix-matrix
- * kernel).  which = 2: two to four rows of x (0: never the 16-bit kernel that takes x in chunks,
- * 1: wherever it can run).  value -1: the library's own choice (the default).  A forced kernel that cannot take a
+ * kernel).  which = 2: up to eight rows of x (0: never the 16-bit kernel that keeps every tile's
+ * sums in registers, 1: wherever it can run).  value -1: the library's own choice (the default).  A forced kernel that cannot take a
  * call (shape, alignment) leaves that call to the library's choice; results do not depend on
  * the setting beyond what the kernels' own summation orders differ by (the integer operator:
  * not at all).  Returns the previous value (>= -1), or DMM_ERR_BAD_SHAPE for arguments out of
