@@ -44,11 +44,13 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 # HBM bytes one GEMV launch moves, per kernel, averaged over the four shapes of the step (the 8-bit kernel
-# serves all of them in the headline, the 16-bit kernel in the 16-bit-only leg): rocprofv3 FETCH_SIZE and
+# serves all of them in the headline, the 16-bit kernel with resident sums in the 16-bit-only leg; the
+# streaming kernel's figure is from the build in which it served that leg): rocprofv3 FETCH_SIZE and
 # WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain 256 MiB device copy
 # (x2.000 and x1.000).  39.19 MB per launch against 38,855,680 algorithmic bytes (codes, x, grid, y): 1.009.
 # The many-tile 8-bit kernel (more than eight row tiles per compute unit) runs in no leg of this file.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8d_kernel": 39191335, "dmm::gemv_stream_kernel": 39189916}
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8d_kernel": 39192105, "dmm::gemv_f16d_kernel": 39175971,
+                                 "dmm::gemv_stream_kernel": 39189916}
 GEMV_TRAFFIC_SOURCE = {k: "constant from an earlier rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command, summarised in "
                           "profiles/gemv_kernels_llama70b_batch1.md; not measured by this run (a counter run cannot share a "
                           "process with the timed one)" for k in GEMV_TRAFFIC_BYTES_PER_LAUNCH}
