@@ -1001,6 +1001,27 @@ def dispatch_check(torch, lib, capi, workload, dev):
             extra = {"chosen_no_workspace_us": round(t0, 3), "slower_by_no_workspace": round(t0 / best2 - 1.0, 4)}
         add(check, M, K, N, times, extra)
 
+    # ---- the integer operator on up to 8 rows: the kernel with resident sums against the row-block kernel
+    for M in (1, 4, 8):
+        for K, N in ((4096, 11008), (8192, 8192), (8192, 10240), (8192, 28672), (28672, 8192)):
+            gi = torch.Generator(device=dev)
+            gi.manual_seed(5)
+            x = torch.randint(-128, 128, (M, K), generator=gi, dtype=torch.int8, device=dev)
+            out = torch.empty(M, N, dtype=torch.int32, device=dev)
+
+            def i8_small(c, s):
+                return lib.dmm_decode_matmul_i8(x.data_ptr(), c, cb.data_ptr(), out.data_ptr(), M, N, K, 1, s)
+            times = {"operator": graph_us(i8_small, workload.code_bytes(N, K))}
+            kernel = lib.dmm_integer_kernel_name(M, N, K).decode()
+            was = lib.dmm_set_choice(1, 1)
+            try:
+                times["row blocks"] = graph_us(i8_small, workload.code_bytes(N, K))
+            finally:
+                lib.dmm_set_choice(1, was)
+            if kernel == "dmm::int8d_kernel":
+                times["resident sums"] = times["operator"]
+            add("int8, up to 8 rows", M, K, N, times, {"kernel": kernel})
+
     # ---- the integer operator on more than 16 rows: passes against the matrix-matrix kernel (pick_int8)
     for M in (32, 64, 128, 192, 256, 384):
         for K, N in ((4096, 4096), (11008, 4096), (8192, 28672), (28672, 8192)):

@@ -171,7 +171,7 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K)
 {
     switch (pick_int8(M, N, K, cu_count_or_default())) {
         case kInt8Gemm: return "dmm::int8g_kernel";
-        case kInt8Gemv: return "dmm::int8x_kernel";
+        case kInt8Gemv: return int8_takes_resident(M, N, cu_count_or_default()) ? "dmm::int8d_kernel" : "dmm::int8x_kernel";
         default: return "dmm::int8_kernel";
     }
 }

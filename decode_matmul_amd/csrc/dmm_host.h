@@ -91,9 +91,14 @@ const std::vector<KernelInfo> &kernel_table()
 #define DMM_K_I8X_S(T, S)                                                                                    \
     kinfo(int8x_kernel<1, 8, 2, T, S>, kLdsMax, true), kinfo(int8x_kernel<2, 8, 2, T, S>, kLdsMax, true),              \
         kinfo(int8x_kernel<3, 8, 2, T, S>, kLdsMax, true), kinfo(int8x_kernel<4, 8, 2, T, S>, kLdsMax, true)
-#define DMM_K_I8X(T) DMM_K_I8X_S(T, false), DMM_K_I8X_S(T, true), kinfo(int8g_kernel<T>, kI8gSmem, true)
+#define DMM_K_I8D(T)                                                                                         \
+    kinfo(int8d_kernel<2, 1, 2, T>, kLdsMax, true), kinfo(int8d_kernel<3, 1, 3, T>, kLdsMax, true),                \
+        kinfo(int8d_kernel<4, 1, 2, T>, kLdsMax, true), kinfo(int8d_kernel<6, 1, 3, T>, kLdsMax, true),            \
+        kinfo(int8d_kernel<8, 1, 2, T>, kLdsMax, true)
+#define DMM_K_I8X(T) DMM_K_I8X_S(T, false), DMM_K_I8X_S(T, true), DMM_K_I8D(T), kinfo(int8g_kernel<T>, kI8gSmem, true)
         DMM_BOTH_LAYOUTS(DMM_K_I8X),
 #undef DMM_K_I8X
+#undef DMM_K_I8D
 #undef DMM_K_I8X_S
 #undef DMM_K_GREG
 #undef DMM_K_REGX
@@ -697,11 +702,55 @@ int launch_int8g(const void *x, const void *codes, const void *cb, void *out, in
                   (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
 }
 
+// Up to 8 rows of x with two to eight row tiles per compute unit: the kernel with resident sums (graph
+// launches, us, int8x / int8d, see the dispatch check of bench.py for the box's own figures)
+inline bool int8d_ok(int64_t M, int64_t N, int cus)
+{
+    const int64_t n_tiles = (N + 15) / 16;
+    return M >= 1 && M <= 8 && n_tiles > cus && n_tiles <= 8 * (int64_t)cus;
+}
+
+template <int NT, int U, int D, bool kTiled>
+int launch_int8d_inst(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+                      hipStream_t stream)
+{
+    const size_t shmem = (size_t)2 * kI8TableBytes + 16 * kI8dPiece;
+    const int64_t n_tiles = (N + 15) / 16;
+    const int64_t wgs = cu_count();   // int8d_ok: more tiles than that, and at most NT each
+    return launch(int8d_kernel<NT, U, D, kTiled>, dim3((unsigned)wgs), dim3(1024), shmem, stream, (const int8_t *)x,
+                  (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K,
+                  (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+}
+
+template <bool kTiled>
+int launch_int8d(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
+                 hipStream_t stream)
+{
+    const int64_t n_tiles = (N + 15) / 16;
+    const int cus = cu_count();
+    switch ((int)((n_tiles + cus - 1) / cus)) {
+        case 2: return launch_int8d_inst<2, 1, 2, kTiled>(x, codes, cb, out, M, N, K, stream);
+        case 3: return launch_int8d_inst<3, 1, 3, kTiled>(x, codes, cb, out, M, N, K, stream);
+        case 4: return launch_int8d_inst<4, 1, 2, kTiled>(x, codes, cb, out, M, N, K, stream);
+        case 5:
+        case 6: return launch_int8d_inst<6, 1, 3, kTiled>(x, codes, cb, out, M, N, K, stream);
+        default: return launch_int8d_inst<8, 1, 2, kTiled>(x, codes, cb, out, M, N, K, stream);
+    }
+}
+
+// does the matrix-vector route of the integer operator take the kernel with resident sums?  g_choice[1] = 1
+// keeps the row-block kernel
+inline bool int8_takes_resident(int64_t M, int64_t N, int cus)
+{
+    return int8d_ok(M, N, cus) && g_choice[1].load(std::memory_order_relaxed) != 1;
+}
+
 // any number of rows of x, 16 per pass
 template <bool kTiled>
 int run_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
               hipStream_t stream)
 {
+    if (int8_takes_resident(M, N, cu_count())) return launch_int8d<kTiled>(x, codes, cb, out, M, N, K, stream);
     switch (small_batch_row_block((N + 15) / 16, cu_count())) {
         case 1: return launch_int8x<1, kTiled>(x, codes, cb, out, M, N, K, stream);
         case 2: return launch_int8x<2, kTiled>(x, codes, cb, out, M, N, K, stream);

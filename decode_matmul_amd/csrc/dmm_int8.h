@@ -376,6 +376,219 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 }
 
 
+// ------------------------------------------------------------------ the integer operator, up to eight rows, resident sums
+// int8x_kernel's tables and byte decode in the loop order of the batch-1 half-precision kernels: sixteen
+// waves, chunk (16 k steps, one per wave) outside and tiles inside, the int32 sums of all NT <= 8 row tiles
+// of the workgroup's share in registers from start to end, a ring of D code loads per wave over the items
+// (chunk, tile), one of them ahead of the prologue's work.  A wave fetches the x of its own k step - up
+// to 8 rows of 256 bytes, two load instructions of four whole lines each - through a 2 KB piece of LDS
+// that is its own (pieces of row m exchanged by m: no bank conflicts) into the four B operands of a tile
+// step, and keeps them for every tile; the slice of the next chunk is asked for before the tile steps of
+// this one.  No barrier between the one after the tables and the end, where the sums go through the same
+// pieces, four tiles at a time (the 128 KB of tables leave 32 KB).  Exact like int8x_kernel; a table with
+// a byte that is not 2 mod 4 goes to the scalar decode.
+template <int kCtrl>
+__device__ __forceinline__ int dpp_shr_add_i(int v)
+{
+    return v + __builtin_amdgcn_update_dpp(0, v, kCtrl, 0xF, 0xF, true);
+}
+// sum over each row of 16 lanes, result in lane 15 of the row
+__device__ __forceinline__ int row_sum16_i(int v)
+{
+    v = dpp_shr_add_i<0x118>(v);
+    v = dpp_shr_add_i<0x114>(v);
+    v = dpp_shr_add_i<0x112>(v);
+    return dpp_shr_add_i<0x111>(v);
+}
+
+constexpr int kI8dPiece = 2048;   // LDS bytes of a wave's own piece: 8 rows x 256 bytes
+
+template <int NT, int U, int D, bool kTiled>
+__global__ __launch_bounds__(1024) void int8d_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+                                                     const int64_t *__restrict__ codebook_abs,
+                                                     int32_t *__restrict__ out, int M, int N, int K, int tiles_q,
+                                                     int tiles_r)
+{
+    constexpr int W = 16;
+    static_assert((U * NT) % D == 0, "the ring has to divide the unrolled loop");
+    static_assert(NT <= 8, "the sums of the end go through the pieces four tiles at a time, twice at most");
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c16 = lane & 15;
+    const int q = lane >> 4;
+    const int n_steps = K >> 8;
+    const int n_chunks = (n_steps + W - 1) / W;
+    const int row_bytes = K >> 2;
+    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u;          // grid rows: [0, 64K)
+    const uint32_t lane_base2 = lane_base | 0x10000u;               // mask rows: [64K, 128K)
+
+    uint64_t entry = 0;
+    if (tid < 256) entry = (uint64_t)codebook_abs[tid];
+
+    // the wave's slice of the first chunk: load i is piece lane % 16 (16 bytes) of row 4 i + lane / 16; rows
+    // past M lie past the end of the buffer (zeros, no memory access), and so does a k step that does not exist
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(x), 0, M * K, 0x00020000);
+    constexpr int kOut = (int)0x80000000;
+    const int xcoff = q * K + c16 * 16;
+    auto x_soff = [&](int c, int i) { return c * W + wave < n_steps ? (c * W + wave) * 256 + i * 4 * K : kOut; };
+    u4_t xv[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(0, i), 0);
+    // the wave's piece: row m at m * 256, its piece p in slot p ^ m.  Writes: row 4 i + h, piece lane % 16,
+    // h = lane / 16, i.e. (xs_w ^ 64 i) + 1024 i.  Reads: row c16 % 8, piece 4 q + t, i.e. xs_r ^ 16 t (columns
+    // 8 .. 15 of the product repeat 0 .. 7 and are not stored).
+    const uint32_t piece = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + wave * kI8dPiece);
+    const uint32_t xs_w = piece + (uint32_t)(q * 256 + ((c16 ^ q) << 4));
+    const int xr_row = c16 & 7;
+    const uint32_t xs_r = piece + (uint32_t)(xr_row * 256 + (((4 * q) ^ xr_row) << 4));
+
+    const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
+    const int nt = tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);   // <= NT (the host's business)
+
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(codes), 0, (int)((int64_t)(kTiled ? ((N + 15) >> 4) * 16 : N) * row_bytes), 0x00020000);
+    // row-major: row c16 of the tile, 16 bytes at quarter q.  Tiled: the tile row is 16 rows x K / 4 bytes as
+    // well, a tile (4 code columns) is 128 bytes, and lane (g = c16 % 8, quarter q) reads 16 bytes at g * 16 of
+    // tiles 2 q and 2 q + 1 of the step's 8.
+    const int voff = kTiled ? q * 256 + (c16 & 7) * 16 : c16 * row_bytes + q * 16;
+    const int tile_stride = 16 * row_bytes;
+    const int step_stride = kTiled ? 1024 : 64;
+    const int tile0_off = t0 * tile_stride;
+    const uint32_t half_sel = (c16 & 8) ? 0x07060302u : 0x05040100u;   // tiled: which row of the pair is ours
+    constexpr int kCw = kTiled ? 2 : 1;
+    auto issue = [&](u4_t (&cwd)[kCw], int c, int t) {
+        const int step = c * W + wave;
+        const bool ok = t < nt && step < n_steps;
+        const int so = ok ? tile0_off + t * tile_stride + step * step_stride : kOut;
+        cwd[0] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff, so, 0);
+        if (kTiled) cwd[kCw - 1] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, voff + 128, so, 0);
+    };
+    u4_t cw[D][kCw];
+    issue(cw[0], 0, 0);
+
+    // tables: threads 0 .. 255 write the 32 copies of table entry tid (16 slots of two copies),
+    // threads 256 .. 511 those of the mask of high byte tid - 256
+    bool bad = false;
+    if (tid < 512) {
+        uint64_t v = entry;
+        if (tid < 256) {
+            bad = (entry & 0x0303030303030303ull) != 0x0202020202020202ull;
+        } else {
+            const uint32_t t = (uint32_t)tid - 256u;
+            uint32_t s8 = t & 0x7Fu;
+            s8 |= (__builtin_popcount(s8) & 1u) << 7;
+            v = (t >> 7) ? 0x0303030303030303ull : 0x0101010101010101ull;
+#pragma unroll
+            for (int d = 0; d < 8; d++)
+                if ((s8 >> d) & 1u) v ^= 0xFCull << (8 * d);
+        }
+        const uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+        const uint32_t rowp = lds_addr(smem_raw) + (uint32_t)((tid * 16 + (tid & 15)) * 16);
+#pragma unroll
+        for (int i = 0; i < 16; i++) lds_write16(rowp ^ (uint32_t)(i * 16), u4_t{lo, hi, lo, hi});
+    }
+#pragma unroll
+    for (int d = 1; d < D; d++) issue(cw[d], d / NT, d % NT);
+    // the vote on the table: one word per wave in the area of the pieces, read by everybody after the barrier
+    uint32_t *votes = reinterpret_cast<uint32_t *>(smem_raw + 2 * kI8TableBytes);
+    const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
+    if (lane == 0) votes[wave] = wave_bad ? 1u : 0u;
+    __syncthreads();
+    const bool any_bad = __builtin_amdgcn_ballot_w64(votes[lane & (W - 1)] != 0) != 0;
+    __syncthreads();   // the votes are read before the first slice of x overwrites them
+    if (any_bad) {
+        // scalar decode for this workgroup's rows; the raw table goes where the pieces would
+        uint64_t *table = reinterpret_cast<uint64_t *>(smem_raw + 2 * kI8TableBytes);
+        if (tid < 256) table[tid] = entry;
+        __syncthreads();
+        const int64_t n_end = (int64_t)(t0 + nt) * 16 < N ? (int64_t)(t0 + nt) * 16 : N;
+        int8_rows<false>(x, codes, table, table, out, M, N, K, kTiled ? 1 : 0, false, (int64_t)t0 * 16 + wave, W, n_end);
+        return;
+    }
+
+    i4_t acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = i4_t{0, 0, 0, 0};
+
+    for (int c0 = 0; c0 < n_chunks; c0 += U) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int c = c0 + u;
+            const bool step_ok = (U == 1 || c < n_chunks) && c * W + wave < n_steps;
+            // the slice through the wave's piece: in as loaded, out as the B operands of the four MFMAs
+#pragma unroll
+            for (int i = 0; i < 2; i++) lds_write16((xs_w ^ (uint32_t)(64 * i)) + (uint32_t)(1024 * i), xv[i]);
+            u4_t xb[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) xb[t] = lds_read16(xs_r ^ (uint32_t)(16 * t));
+#pragma unroll
+            for (int i = 0; i < 2; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(c + 1, i), 0);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int slot = (u * NT + t) % D;
+                if (step_ok && t < nt) {
+                    u4_t w4;   // the lane's 8 codes of the step, two per word
+                    if (kTiled) {
+                        const u4_t &a = cw[slot][0], &b = cw[slot][kCw - 1];
+                        w4 = u4_t{__builtin_amdgcn_perm(a[1], a[0], half_sel), __builtin_amdgcn_perm(a[3], a[2], half_sel),
+                                  __builtin_amdgcn_perm(b[1], b[0], half_sel), __builtin_amdgcn_perm(b[3], b[2], half_sel)};
+                    } else {
+                        w4 = cw[slot][0];
+                    }
+                    u2_t g[8], m[8];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const uint32_t w = w4[i];
+                        g[2 * i] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0400u));
+                        m[2 * i] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020500u));
+                        g[2 * i + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base, 0x0C0C0600u));
+                        m[2 * i + 1] = lds_read8(__builtin_amdgcn_perm(w, lane_base2, 0x0C020700u));
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const i4_t a = i4_t{(int)(g[2 * i][0] ^ m[2 * i][0]), (int)(g[2 * i][1] ^ m[2 * i][1]),
+                                            (int)(g[2 * i + 1][0] ^ m[2 * i + 1][0]), (int)(g[2 * i + 1][1] ^ m[2 * i + 1][1])};
+                        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, __builtin_bit_cast(i4_t, xb[i]), acc[t], 0, 0, 0);
+                    }
+                }
+                issue(cw[slot], c + (t + D) / NT, (t + D) % NT);   // the item D further on
+            }
+        }
+    }
+    // the sums, four tiles at a time, through the wave's own piece: cell (tile % 4, quarter, column) at slot
+    // cell ^ wave, so that the 16 lanes of a reader, one per wave, meet no bank conflict; wave w adds up
+    // columns 2 (w / 4) and 2 (w / 4) + 1 of tile w % 4 of the four
+#pragma unroll
+    for (int r0 = 0; r0 < NT; r0 += 4) {
+        if (r0 > 0) {
+            if (r0 >= nt) break;        // uniform
+            __syncthreads();            // the readers of the round before are done with the pieces
+        }
+#pragma unroll
+        for (int t = r0; t < r0 + 4 && t < NT; t++)
+            if (t < nt && c16 < 8)
+                lds_write16(piece + (uint32_t)((((((t & 3) * 4 + q) * 8 + c16) ^ wave)) << 4), __builtin_bit_cast(u4_t, acc[t]));
+        __syncthreads();
+        const int tw = wave & 3;
+        if (r0 + tw < nt) {
+            const uint32_t src = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + c16 * kI8dPiece);
+            const int n = (t0 + r0 + tw) * 16 + 4 * q;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int m = 2 * (wave >> 2) + j;
+                i4_t v = __builtin_bit_cast(i4_t, lds_read16(src + (uint32_t)(((((tw * 4 + q) * 8 + m) ^ c16)) << 4)));
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = row_sum16_i(v[e]);
+                if (c16 == 15 && m < M && n < N)   // N % 4 == 0, so the four rows are in range together
+                    *reinterpret_cast<i4_t *>(out + (int64_t)m * N + n) = v;
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------ the integer operator, many rows of x
 // Block tile 256 (n) x 128 (m), eight waves in two groups of four.  A group is a complete
 // 256 x 128 x 64 pipeline - one wave per SIMD, each 64 rows of W (two 32-row tiles) x all 128 rows

@@ -567,7 +567,9 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     and a table with bytes that are not 2 mod 4, which every workgroup must notice and serve
     with the scalar decode.  Exact against the oracle's restatement of
     /root/reference/test_decode_matmul.py:58-71."""
-    assert capi.lib().dmm_integer_kernel_name(M, N, K) == b"dmm::int8x_kernel"
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    resident = M <= 8 and 2 <= -(-((N + 15) // 16) // cus) <= 8   # two to eight row tiles per compute unit
+    assert capi.lib().dmm_integer_kernel_name(M, N, K) == (b"dmm::int8d_kernel" if resident else b"dmm::int8x_kernel")
     rng = np.random.default_rng(M * 977 + N + K)
     if table == "e8p":
         cb = orc.build_codebook_abs()
@@ -582,6 +584,51 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     out = c_matmul_i8(dev(x), cd, dev(cb), tiled)
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M,N,K,tiled,table", [
+    # two to eight row tiles per compute unit (every instance of the kernel, shares that leave the last
+    # tiles of an instance unused, N no multiple of 16), one k step to 33 (waves without a step, a ragged
+    # last chunk), one to eight rows of x, both code layouts, every kind of table
+    (1, 4100, 256, False, "e8p"), (2, 8192, 8192, True, "e8p"), (3, 16 * (256 * 2 + 5), 768, True, "mod4"),
+    (4, 16 * (256 * 3 - 10), 4352, False, "e8p"), (5, 8192 + 16, 1024, True, "any"), (6, 16384, 2048, True, "e8p"),
+    (7, 16 * (256 * 5 - 1), 512, False, "mod4"), (8, 16 * (256 * 6 - 100), 1280, True, "e8p"),
+    (8, 28672, 256, True, "e8p"), (1, 28672, 8448, True, "e8p"), (8, 32768, 768, False, "mod4"),
+    (3, 16 * (256 * 7 + 1) - 12, 512, False, "any"), (8, 10240, 8192, True, "e8p"), (1, 16 * (256 * 4), 4096, False, "e8p")])
+def test_integer_operator_resident_sums(M, N, K, tiled, table):
+    """Up to eight rows of x with two to eight row tiles per compute unit run on the kernel that keeps the
+    sums of its whole share in registers.  Exact against the oracle's decode times x in float64 (every sum
+    is far below 2^53, so that product is the integer one) and, on the first and last rows of W, against
+    the integer oracle itself (/root/reference/test_decode_matmul.py:58-71 restated); the row-block kernel,
+    forced, gives the same tensor."""
+    assert capi.lib().dmm_integer_kernel_name(M, N, K) == b"dmm::int8d_kernel"
+    rng = np.random.default_rng(M * 613 + N + K)
+    if table == "e8p":
+        cb = orc.build_codebook_abs()
+    elif table == "mod4":
+        cb = ((rng.integers(0, 256, size=(256, 8)).astype(np.uint8) & 0xFC) | 2).view(np.int64).reshape(256).copy()
+    else:
+        cb = rng.integers(-2 ** 63, 2 ** 63, size=256, dtype=np.int64)
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
+    cd = dev(orc.transpose_tile(codes)) if tiled else dev(codes)
+    out = c_matmul_i8(dev(x), cd, dev(cb), tiled)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    rows = np.r_[0:40, N - 40:N]
+    assert np.array_equal(got[:, rows], orc.decode_matmul_i32(x, codes[rows], cb))
+    W = torch.from_numpy(orc.decode_i8(codes, cb)).to(DEV).double()
+    want = (dev(x).double() @ W.T).cpu().numpy().astype(np.int64).astype(np.int32)
+    del W
+    assert np.array_equal(got, want)
+    before = capi.lib().dmm_set_choice(1, 1)
+    try:
+        assert capi.lib().dmm_integer_kernel_name(M, N, K) == b"dmm::int8x_kernel"
+        out2 = c_matmul_i8(dev(x), cd, dev(cb), tiled)
+        torch.cuda.synchronize()
+    finally:
+        capi.lib().dmm_set_choice(1, before)
+    assert torch.equal(out, out2)
 
 
 @pytest.mark.parametrize("M,N,K,tiled,table", [
