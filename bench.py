@@ -947,10 +947,10 @@ def dispatch_check(torch, lib, capi, workload, dev):
                 lib.dmm_set_gemv_8bit(was)
             add("pick_gemv", M, K, N, times, {"kernel": lib.dmm_gemv_kernel_name(M, N, K).decode()})
 
-    # ---- up to eight rows: the 16-bit kernel with resident sums against the kernels that served before it
-    for M in (2, 4, 8):
+    # ---- up to 32 rows: the 16-bit kernel with resident sums against the kernels that served before it
+    for M in (2, 4, 8, 12, 16, 24, 32):
         for K, N in ((4096, 11008), (4096, 22016), (11008, 4096), (8192, 8192), (8192, 10240), (8192, 28672),
-                     (28672, 8192), (1024, 16384)):
+                     (28672, 8192), (1024, 16384), (4096, 4096), (8192, 4096)):
             x, grid, scale = half_inputs(M, K)
             y = torch.empty(M, N, dtype=torch.float16, device=dev)
 
@@ -969,7 +969,8 @@ def dispatch_check(torch, lib, capi, workload, dev):
     # kernel, with and without a workspace)
     ws = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
     mm_cases = [("passes_beat_splitk", M, K, N) for M in (17, 32)
-                for K, N in ((4096, 11008), (8192, 8192), (8192, 8448), (4096, 17408), (8192, 10240))]
+                for K, N in ((4096, 11008), (8192, 8192), (8192, 8448), (4096, 17408), (8192, 10240), (4096, 4096),
+                             (11008, 4096), (4096, 22016), (8192, 28672), (28672, 8192), (16384, 8192))]
     mm_cases += [("passes_beat_gemm", M, K, N) for M in (48, 64, 128, 256)
                  for K, N in ((4096, 4096), (4096, 11008), (11008, 4096), (8192, 8192))]
     for check, M, K, N in mm_cases:

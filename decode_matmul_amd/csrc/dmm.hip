@@ -179,7 +179,6 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K)
 const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K)
 {
     if (M < 1 || M > 32 || N < 1 || K < 256 || (K & 255) || (N & 3) || N * (K >> 2) >= (1LL << 31)) return "";
-    if (M > 16) return "dmm::gemv_regx_kernel";
     switch (pick_gemv(M, N, K)) {
         case kGemvStream: return "dmm::gemv_stream_kernel";
         case kGemvF16d: return "dmm::gemv_f16d_kernel";

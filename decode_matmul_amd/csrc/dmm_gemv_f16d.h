@@ -1,4 +1,4 @@
-// Two to eight rows of x on 16-bit operands with x taken a k step at a time and every tile of a workgroup in registers.
+// Up to 32 rows of x on 16-bit operands with x taken a k step at a time and every tile of a workgroup in registers.
 // Part of libdmm: included by dmm.hip inside namespace dmm, in this order; not a
 // translation unit of its own.
 
@@ -9,7 +9,7 @@
 // the streaming kernel's tables, decode and MFMA (one code = two 16-byte gathers, four packed FMAs, one
 // v_mfma_f32_16x16x32_f16 whose B column m is row m of x) and the loop order of the batch-1 kernel on 8-bit
 // operands:
-//   * a chunk of x is 16 k steps, one per wave, and a wave only ever needs its own: the slice of its k step (up
+//   * a chunk of x is W = 16 k steps (8 for nine to sixteen rows of x), one per wave, and a wave only ever needs its own: the slice of its k step (up
 //     to 2 XI rows of 512 bytes) is loaded in XI instructions whose 32 lanes per row take 512 consecutive bytes,
 //     written as loaded into a piece of LDS that belongs to the wave alone and read back as the eight B
 //     operands of a tile step (the 16-byte pieces of row m exchanged by m, so that writes and reads meet no
@@ -20,18 +20,18 @@
 //     with one the sums do not depend on how many tiles a workgroup has), and the code stream is a ring of D
 //     loads per wave over the items (chunk, tile).
 //   * at the end every wave leaves its accumulators' columns 0 .. 2 XI - 1 (the rows of x) in its own piece,
-//     and after the launch's one other barrier wave t adds tile t up over the 16 waves by DPP and stores y.
+//     and after the launch's one other barrier wave t adds tile t up over the W waves by DPP and stores y.
 // Any grid of finite halves, any x: the arithmetic is the streaming kernel's (fp32 sums of exact products),
 // only the order of the sums differs.
-// LDS map: tables [0, 96K), then 16 pieces of XI KB.
-__host__ __device__ constexpr int fd_lds_bytes(int XI) { return kSTablesBytes + 16 * XI * 1024; }
+// LDS map: tables [0, 96K), then W pieces of XI KB.
+__host__ __device__ constexpr int fd_lds_bytes(int XI, int W = 16) { return kSTablesBytes + W * XI * 1024; }
 
 // One tile's 256-wide k step: 8 codes of the lane -> 16 gathers, 32 packed FMAs, 8 MFMAs into acc.  kAhead: the
 // gathers of a code word are issued before the arithmetic of the word before it (17 more registers, which the
 // instances with many tiles do not have).
-template <bool kAhead>
+template <bool kAhead, int CG>
 __device__ __forceinline__ void fd_tile_step(const u4_t &cw, uint32_t lane_base, uint32_t quarter_bits,
-                                             const u4_t (&xb)[8], f4_t &acc)
+                                             const u4_t (&xb)[CG][8], f4_t (&acc)[CG])
 {
     StreamGather buf[kAhead ? 2 : 1];
     stream_gather(buf[0], cw[0], lane_base, quarter_bits);
@@ -40,28 +40,37 @@ __device__ __forceinline__ void fd_tile_step(const u4_t &cw, uint32_t lane_base,
         if (kAhead && t2 + 1 < 4) stream_gather(buf[(t2 + 1) & 1], cw[t2 + 1], lane_base, quarter_bits);
         const StreamGather &b = buf[kAhead ? t2 & 1 : 0];
         const h8_t a0 = stream_finish<false>(b.g0, b.s0, b.dd);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[2 * t2]), acc, 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < CG; g++)
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(h8_t, xb[g][2 * t2]), acc[g], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         const h8_t a1 = stream_finish<true>(b.g1, b.s1, b.dd);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[2 * t2 + 1]), acc, 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < CG; g++)
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(h8_t, xb[g][2 * t2 + 1]), acc[g], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (!kAhead && t2 + 1 < 4) stream_gather(buf[0], cw[t2 + 1], lane_base, quarter_bits);
     }
 }
 
-// XI: load instructions per slice of x, two rows each: 2 for up to four rows, 4 for up to eight
-template <int NT, int U, int D, bool kPacked, int XI>
-__global__ __launch_bounds__(1024) void gemv_f16d_kernel(const uint16_t *__restrict__ x,
+// XI: load instructions per slice of x, two rows each: 2 for up to four rows, 4 for up to eight, 8 for up to sixteen.
+// W: waves, i.e. k steps per chunk: 16, or 8 where sixteen pieces of 8 KB would not fit beside the tables.
+// CG: groups of sixteen rows of x (1, or 2 for 17 to 32 rows): one decode of a code feeds an MFMA per group, the
+// slices of the groups go through the wave's piece one after the other, and so do the sums at the end.
+template <int NT, int U, int D, bool kPacked, int XI, int W = 16, int CG = 1>
+__global__ __launch_bounds__(64 * W) void gemv_f16d_kernel(const uint16_t *__restrict__ x,
                                                          const uint16_t *__restrict__ codes,
                                                          const void *__restrict__ grid, float scale,
                                                          uint16_t *__restrict__ y, int M, int N, int K, int tiles_q,
                                                          int tiles_r)
 {
-    constexpr int W = 16;
     constexpr int CM = 2 * XI;          // columns of the product that can hold a row of x
     constexpr int kPiece = XI * 1024;   // bytes of a wave's own piece: CM rows x 512 bytes
-    static_assert(XI == 2 || XI == 4, "up to four or up to eight rows of x");
-    constexpr bool kAhead = NT < 8 && !(NT >= 6 && XI == 4);   // 8 tiles, or 6 with eight rows of x: no registers for it
+    static_assert((W == 16 && (XI == 2 || XI == 4)) || (W == 8 && XI == 8), "up to four, eight or sixteen rows of x");
+    static_assert(CG == 1 || (CG == 2 && XI == 8), "a second group of rows only beside a full first one");
+    static_assert(fd_lds_bytes(XI, W) <= 160 * 1024, "tables and pieces have to fit the LDS");
+    // sixteen waves: 8 tiles, or 6 with eight rows of x, leave no registers for it
+    constexpr bool kAhead = W == 8 || (NT < 8 && !(NT >= 6 && XI == 4));
     static_assert((U * NT) % D == 0, "the ring has to divide the unrolled loop");
     static_assert(NT * 4 * CM * 16 <= kPiece, "the partial sums of the end go through the wave's piece");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
@@ -85,10 +94,12 @@ __global__ __launch_bounds__(1024) void gemv_f16d_kernel(const uint16_t *__restr
     constexpr int kOut = (int)0x80000000;
     // load i: 4 i K bytes further on, in the scalar offset (recomputed where it is used: a register less to hold)
     auto x_voff = [&]() { return (((int)threadIdx.x >> 5 & 1) * K + ((int)threadIdx.x & 31) * 8) * 2; };
-    auto x_soff = [&](int c, int i) { return c * W + wave < n_steps ? (c * W + wave) * 512 + i * 4 * K : kOut; };
-    u4_t xv[XI];
+    auto x_soff = [&](int c, int i) { return c * W + wave < n_steps ? (c * W + wave) * 512 + i * 4 * K : kOut; };   // i: pair of rows
+    u4_t xv[CG][XI];
 #pragma unroll
-    for (int i = 0; i < XI; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_voff(), x_soff(0, i), 0);
+    for (int g = 0; g < CG; g++)
+#pragma unroll
+        for (int i = 0; i < XI; i++) xv[g][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_voff(), x_soff(0, g * 8 + i), 0);
     // the wave's piece: row m at m * 512, its piece p in slot p ^ m.  Writes: row 2 i + h, piece lane % 32,
     // h = lane / 32, i.e. (xs_w ^ 32 i) + 1024 i.  Reads: row c16, piece 8 q + t, i.e. xs_r ^ 16 t; lanes whose row
     // is never written (c16 >= CM) read row c16 % CM: their columns of the product are not stored.
@@ -125,9 +136,11 @@ __global__ __launch_bounds__(1024) void gemv_f16d_kernel(const uint16_t *__restr
     for (int d = 1; d < D; d++) issue(cw[d], d / NT, d % NT);
     __syncthreads();
 
-    f4_t acc[NT];
+    f4_t acc[NT][CG];
 #pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int g = 0; g < CG; g++) acc[t][g] = f4_t{0.f, 0.f, 0.f, 0.f};
 
     for (int c0 = 0; c0 < n_chunks; c0 += U) {
 #pragma unroll
@@ -135,43 +148,53 @@ __global__ __launch_bounds__(1024) void gemv_f16d_kernel(const uint16_t *__restr
             const int c = c0 + u;
             const bool step_ok = (U == 1 || c < n_chunks) && c * W + wave < n_steps;
             // the slice through the wave's piece: in as loaded, out as the B operands of the eight MFMAs
+            // (the LDS serves a wave's instructions in order: the second group's slice may follow the first one's reads)
+            u4_t xb[CG][8];
 #pragma unroll
-            for (int i = 0; i < XI; i++) lds_write16((xs_w() ^ (uint32_t)(32 * i)) + (uint32_t)(1024 * i), xv[i]);
-            u4_t xb[8];
+            for (int g = 0; g < CG; g++) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) xb[i] = lds_read16(xs_r ^ (uint32_t)(16 * i));
+                for (int i = 0; i < XI; i++) lds_write16((xs_w() ^ (uint32_t)(32 * i)) + (uint32_t)(1024 * i), xv[g][i]);
 #pragma unroll
-            for (int i = 0; i < XI; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_voff(), x_soff(c + 1, i), 0);
+                for (int i = 0; i < 8; i++) xb[g][i] = lds_read16(xs_r ^ (uint32_t)(16 * i));
+#pragma unroll
+                for (int i = 0; i < XI; i++)
+                    xv[g][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_voff(), x_soff(c + 1, g * 8 + i), 0);
+            }
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const int slot = (u * NT + t) % D;
-                if (step_ok && t < nt) fd_tile_step<kAhead>(cw[slot], lane_base, quarter_bits, xb, acc[t]);
+                if (step_ok && t < nt) fd_tile_step<kAhead, CG>(cw[slot], lane_base, quarter_bits, xb, acc[t]);
                 issue(cw[slot], c + (t + D) / NT, (t + D) % NT);   // the item D further on
             }
         }
     }
-    // the sums of every tile into the wave's own piece: cell (tile, quarter, column) at slot cell ^ wave, so that
-    // the 16 lanes of a reader, one per wave, meet no bank conflict
+    // the sums of every tile into the wave's own piece, a group of rows at a time: cell (tile, quarter, column) at
+    // slot cell ^ wave, so that the 16 lanes of a reader, one per wave, meet no bank conflict
 #pragma unroll
-    for (int t = 0; t < NT; t++)
-        if (t < nt && c16 < CM)
-            lds_write16(piece + (uint32_t)(((((t * 4 + q) * CM + c16) ^ wave)) << 4), __builtin_bit_cast(u4_t, acc[t]));
-    __syncthreads();
-    if (wave < nt) {
-        // wave t adds up tile t: lane (w, quarter) takes wave w's sums of the quarter's four rows for each
-        // row of x, then the 16 lanes of a row are added with DPP shifts
-        const uint32_t src = lds_addr(smem_raw) + (uint32_t)(kSTablesBytes + c16 * kPiece);
-        const int n = (t0 + wave) * 16 + 4 * q;
+    for (int g = 0; g < CG; g++) {
+        if (g > 0) __syncthreads();   // the readers of the group before are done with the pieces
 #pragma unroll
-        for (int m = 0; m < CM; m++) {
-            f4_t v = __builtin_bit_cast(f4_t, lds_read16(src + (uint32_t)(((((wave * 4 + q) * CM + m) ^ c16)) << 4)));
+        for (int t = 0; t < NT; t++)
+            if (t < nt && c16 < CM)
+                lds_write16(piece + (uint32_t)(((((t * 4 + q) * CM + c16) ^ wave)) << 4), __builtin_bit_cast(u4_t, acc[t][g]));
+        __syncthreads();
+        if (wave < nt) {
+            // wave t adds up tile t: lane (w, quarter) takes wave w's sums of the quarter's four rows for each
+            // row of x (nothing where there is no wave w), then the 16 lanes of a row are added with DPP shifts
+            const uint32_t src = lds_addr(smem_raw) + (uint32_t)(kSTablesBytes + (c16 & (W - 1)) * kPiece);
+            const int n = (t0 + wave) * 16 + 4 * q;
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
-            if (c16 == 15 && m < M && n < N) {   // N % 4 == 0, so the four rows are in range together
-                h4_t o;
+            for (int m = 0; m < CM; m++) {
+                f4_t v = __builtin_bit_cast(f4_t, lds_read16(src + (uint32_t)(((((wave * 4 + q) * CM + m) ^ (c16 & (W - 1)))) << 4)));
+                if (W < 16 && c16 >= W) v = f4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
-                *reinterpret_cast<h4_t *>(y + (int64_t)m * N + n) = o;
+                for (int e = 0; e < 4; e++) v[e] = row_sum16(v[e]);
+                if (c16 == 15 && g * 16 + m < M && n < N) {   // N % 4 == 0, so the four rows are in range together
+                    h4_t o;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = (half_t)(v[e] * scale);
+                    *reinterpret_cast<h4_t *>(y + (int64_t)(g * 16 + m) * N + n) = o;
+                }
             }
         }
     }

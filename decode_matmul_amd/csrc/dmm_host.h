@@ -75,7 +75,15 @@ const std::vector<KernelInfo> &kernel_table()
     kinfo(gemv_f16d_kernel<2, 1, 2, P, XI>, kLdsMax, true), kinfo(gemv_f16d_kernel<3, 1, 3, P, XI>, kLdsMax, true),     \
         kinfo(gemv_f16d_kernel<4, 1, 2, P, XI>, kLdsMax, true), kinfo(gemv_f16d_kernel<6, 1, 3, P, XI>, kLdsMax, true), \
         kinfo(gemv_f16d_kernel<8, 1, 2, P, XI>, kLdsMax, true)
-#define DMM_K_F16D(P) DMM_K_F16D_XI(P, 2), DMM_K_F16D_XI(P, 4)
+#define DMM_K_F16D_W8(P)                                                                                         \
+    kinfo(gemv_f16d_kernel<2, 1, 2, P, 8, 8>, kLdsMax, true), kinfo(gemv_f16d_kernel<3, 1, 3, P, 8, 8>, kLdsMax, true),   \
+        kinfo(gemv_f16d_kernel<4, 1, 2, P, 8, 8>, kLdsMax, true), kinfo(gemv_f16d_kernel<6, 1, 3, P, 8, 8>, kLdsMax, true), \
+        kinfo(gemv_f16d_kernel<8, 1, 2, P, 8, 8>, kLdsMax, true)
+#define DMM_K_F16D_W8G2(P)                                                                                       \
+    kinfo(gemv_f16d_kernel<2, 1, 2, P, 8, 8, 2>, kLdsMax, true), kinfo(gemv_f16d_kernel<3, 1, 3, P, 8, 8, 2>, kLdsMax, true),   \
+        kinfo(gemv_f16d_kernel<4, 1, 2, P, 8, 8, 2>, kLdsMax, true), kinfo(gemv_f16d_kernel<6, 1, 3, P, 8, 8, 2>, kLdsMax, true), \
+        kinfo(gemv_f16d_kernel<8, 1, 2, P, 8, 8, 2>, kLdsMax, true)
+#define DMM_K_F16D(P) DMM_K_F16D_XI(P, 2), DMM_K_F16D_XI(P, 4), DMM_K_F16D_W8(P), DMM_K_F16D_W8G2(P)
         DMM_BOTH_LAYOUTS(DMM_K_F16D),
 #define DMM_K_REGX_XI(P, XI)                                                                                      \
     kinfo(gemv_regx_kernel<1, 8, 2, P, XI>, kLdsMax, true), kinfo(gemv_regx_kernel<2, 8, 2, P, XI>, kLdsMax, true),     \
@@ -104,6 +112,8 @@ const std::vector<KernelInfo> &kernel_table()
 #undef DMM_K_REGX
 #undef DMM_K_REGX_XI
 #undef DMM_K_F16D
+#undef DMM_K_F16D_W8
+#undef DMM_K_F16D_W8G2
 #undef DMM_K_F16D_XI
 #undef DMM_K_Q8D
 #undef DMM_K_Q8
@@ -306,11 +316,12 @@ int launch_gemv_q8d(const void *x, const void *codes, const void *grid, float sc
     }
 }
 
-// the same loop order on 16-bit operands, for up to eight rows of x of any length (a wave fetches the x of its
-// k steps itself): up to 8 tiles per workgroup
+// the same loop order on 16-bit operands, for up to 32 rows of x of any length (a wave fetches the x of its
+// k steps itself; from nine rows on eight waves instead of sixteen, from seventeen on two MFMAs per code): up to
+// 8 tiles per workgroup
 inline bool gemv_f16d_ok(int64_t M, int64_t N, int64_t K)
 {
-    return M >= 1 && M <= 8 && (N + 15) / 16 <= 8 * (int64_t)cu_count() && N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31);
+    return M >= 1 && M <= 32 && (N + 15) / 16 <= 8 * (int64_t)cu_count() && N * (K >> 2) < (1LL << 31) && M * K * 2 < (1LL << 31);
 }
 
 template <int NT, int U, int D, bool kPacked>
@@ -321,6 +332,14 @@ int launch_gemv_f16d_inst(const void *x, const void *codes, const void *grid, fl
     const int64_t wgs = n_tiles < cu_count() ? n_tiles : cu_count();
     if (M <= 4)
         return launch(gemv_f16d_kernel<NT, U, D, kPacked, 2>, dim3((unsigned)wgs), dim3(1024), (size_t)fd_lds_bytes(2), stream,
+                      (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                      (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    if (M > 16)
+        return launch(gemv_f16d_kernel<NT, U, D, kPacked, 8, 8, 2>, dim3((unsigned)wgs), dim3(512), (size_t)fd_lds_bytes(8, 8), stream,
+                      (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
+                      (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    if (M > 8)
+        return launch(gemv_f16d_kernel<NT, U, D, kPacked, 8, 8>, dim3((unsigned)wgs), dim3(512), (size_t)fd_lds_bytes(8, 8), stream,
                       (const uint16_t *)x, (const uint16_t *)codes, grid, scale, (uint16_t *)y, (int)M, (int)N, (int)K,
                       (int)(n_tiles / wgs), (int)(n_tiles % wgs));
     return launch(gemv_f16d_kernel<NT, U, D, kPacked, 4>, dim3((unsigned)wgs), dim3(1024), (size_t)fd_lds_bytes(4), stream,
@@ -417,6 +436,14 @@ bool gemv_8bit_ok(int64_t M, int64_t N, int64_t K) { return M == 1 ? gemv_q8c_ok
 // one tile at a time; the small-batch kernel when x does not fit the LDS.
 enum GemvKind { kGemvQ8, kGemvStream, kGemvF16d, kGemvRegx };
 
+// 17 .. 32 rows of x: is this a shape for the 16-bit kernel with resident sums (two to eight tiles per workgroup,
+// K of 2048 or more)?
+inline bool rows32_resident(int64_t N, int64_t K, int64_t cus)
+{
+    const int64_t n_tiles = (N + 15) / 16;
+    return n_tiles > cus && n_tiles <= 8 * cus && K >= 2048;
+}
+
 GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
 {
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
@@ -431,9 +458,18 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
     // kernels off: 8192 -> 28672 16.6 / 18.0, 4096 -> 22016 9.3 / 11.3), the 8-bit kernel for two to four rows
     // included (M = 2 4096 -> 22016 9.5 / 10.4, 4096 -> 32000 10.1 / 11.75; M = 4 3072 -> 32768 9.7 / 11.8).  With
     // one tile per workgroup it is level with them or behind (M = 1 11008 -> 4096 6.03 / 5.63, M = 4 6.31 / 6.71).
-    const int force = M <= 8 ? g_choice[2].load(std::memory_order_relaxed) : -1;
+    const int force = g_choice[2].load(std::memory_order_relaxed);
+    // Seventeen to 32 rows: the same kernel with two MFMAs per code where a workgroup has two to eight tiles and
+    // K is not short, else two passes of the small-batch kernel (graph launches, us, this kernel / passes, M = 32:
+    // 4096 -> 11008 13.1 / 14.4, 4096 -> 22016 18.0 / 23.6, 8192 -> 10240 18.4 / 21.6, 8192 -> 28672 30.0 / 45.0,
+    // 28672 -> 8192 41.4 / 48.1; but 4096 -> 4096 10.7 / 9.4, 1024 -> 16384 10.3 / 9.1, and level at 8192 -> 4096 and
+    // 11008 -> 4096)
+    if (M > 16) {
+        if (force == 1 && gemv_f16d_ok(M, N, K)) return kGemvF16d;
+        return force != 0 && rows32_resident(N, K, cus) && gemv_f16d_ok(M, N, K) ? kGemvF16d : kGemvRegx;
+    }
     if (force == 1 && gemv_f16d_ok(M, N, K)) return kGemvF16d;
-    if (force != 0 && share >= 2 && gemv_f16d_ok(M, N, K)) return kGemvF16d;
+    if (force != 0 && (share >= 2 || M > 8) && gemv_f16d_ok(M, N, K)) return kGemvF16d;
     // Beyond eight tiles per workgroup: two to four rows on 8-bit operands where their x fits the LDS
     if (M >= 2 && n_tiles > 4 * cus && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
     // Otherwise the 16-bit streaming kernel, one tile at a time, or the small-batch kernel when x does not fit the
@@ -488,7 +524,6 @@ template <bool kPacked>
 int run_gemv(const void *x, const void *codes, const void *grid, float scale, void *y, int64_t M,
              int64_t N, int64_t K, hipStream_t stream)
 {
-    if (M > 16) return run_gemv_regx<kPacked>(x, codes, grid, scale, y, M, N, K, stream);   // 16 rows per pass
     switch (pick_gemv(M, N, K)) {
         case kGemvQ8: return run_gemv_q8<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
         case kGemvF16d: return launch_gemv_f16d<kPacked>(x, codes, grid, scale, y, M, N, K, stream);
@@ -578,8 +613,8 @@ inline double passes_cost_us(int64_t M, int64_t N, int64_t K, int cus)
 
 bool passes_beat_gemm(int64_t M, int64_t N, int64_t K, int cus);
 
-// A workspace is there, and so the choice of splitting K.  17 .. 32 rows of x: two passes of the small-batch
-// kernel beat the split and its second launch while the busiest workgroup has no more than 68 KB of codes
+// A workspace is there, and so the choice of splitting K.  17 .. 32 rows of x where the small-batch kernel
+// serves: its two passes beat the split and its second launch while the busiest workgroup has no more than 68 KB of codes
 // (graph launches, us, split / passes, M = 32: 4096 -> 11008 16.8 / 14.9, 8192 -> 8192 19.7 / 18.3, but 8192 ->
 // 8448 18.9 / 22.0, 4096 -> 17408 19.1 / 22.3, 8192 -> 10240 22.4 / 22.0, 8192 -> 28672 31.7 / 42.0).  More rows:
 // the split costs about 14 us + 0.085 per row + 0.3 per MB of codes, and the passes have to beat that by a
@@ -591,6 +626,10 @@ inline bool passes_beat_splitk(int64_t M, int64_t N, int64_t K, int cus)
 {
     if (K < 256 || (K & 255) || (N & 3)) return false;
     if (M <= 32) {
+        // the kernel with resident sums serves (one launch, every code decoded once): it wins up to K = 12288 or so
+        // (graph launches, us, split / that kernel, M = 32: 4096 -> 22016 22.1 / 18.4, 8192 -> 10240 21.9 / 18.7,
+        // 8192 -> 28672 34.6 / 30.9, but 16384 -> 8192 24.0 / 27.2, 28672 -> 8192 34.1 / 41.8)
+        if (g_choice[2].load(std::memory_order_relaxed) != 0 && rows32_resident(N, K, cus)) return K <= 12288;
         const int64_t share = ((N + 15) / 16 + cus - 1) / cus;   // row tiles of the busiest workgroup
         return share * 4 * K <= (68 << 10);
     }

@@ -250,7 +250,7 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K);
  * given - dmm_workspace_bytes then answers for the split as well).  which = 1: the integer
  * operator on more than 16 rows (1: passes of the matrix-vector kernel, 2: the matrix-matrix
  * kernel) and on up to 8 rows (1: the row-block kernel where the library would take the one that
- * keeps every tile's sums in registers).  which = 2: up to eight rows of x (0: never the 16-bit kernel that keeps every tile's
+ * keeps every tile's sums in registers).  which = 2: up to 32 rows of x (0: never the 16-bit kernel that keeps every tile's
  * sums in registers, 1: wherever it can run).  value -1: the library's own choice (the default).
  * A forced kernel that cannot take a call (shape, alignment) leaves that call to the library's choice; results do not depend on
  * the setting beyond what the kernels' own summation orders differ by (the integer operator:

@@ -318,12 +318,20 @@ def test_gemv_8bit_switch_and_kernel_name():
                 assert lib.dmm_gemv_kernel_name(m, n, k) == b"dmm::gemv_f16d_kernel", (m, n, k)
         assert lib.dmm_gemv_kernel_name(3, 32784, K) == b"dmm::gemv_q8_kernel"        # more tiles, two to four rows: 8-bit
         assert lib.dmm_gemv_kernel_name(5, 32784, K) == b"dmm::gemv_stream_kernel"
-        assert lib.dmm_gemv_kernel_name(9, N, K) == b"dmm::gemv_stream_kernel"        # more rows
-        assert lib.dmm_gemv_kernel_name(9, N, 8192) == b"dmm::gemv_regx_kernel"       # ... whose x does not fit the LDS
+        # nine to sixteen rows: the same kernel on eight waves, whatever the share (up to eight tiles per CU)
+        for m, n, k in ((9, N, K), (9, N, 8192), (16, 4096, 4096), (12, 32768, 256), (16, 28672, 8192)):
+            assert lib.dmm_gemv_kernel_name(m, n, k) == b"dmm::gemv_f16d_kernel", (m, n, k)
+        assert lib.dmm_gemv_kernel_name(9, 32784, K) == b"dmm::gemv_stream_kernel"    # more tiles
+        assert lib.dmm_gemv_kernel_name(9, 32784, 8192) == b"dmm::gemv_regx_kernel"   # ... and an x that does not fit the LDS
+        # seventeen to 32 rows: with two MFMAs per code on two to eight tiles per CU and K >= 2048
+        for m, n, k in ((17, N, 2048), (32, 28672, 8192), (24, 4112, 4096), (32, 32768, 28672)):
+            assert lib.dmm_gemv_kernel_name(m, n, k) == b"dmm::gemv_f16d_kernel", (m, n, k)
+        for m, n, k in ((32, N, K), (17, 4096, 8192), (32, 32784, 4096)):             # short K, one tile per CU, more than eight
+            assert lib.dmm_gemv_kernel_name(m, n, k) == b"dmm::gemv_regx_kernel", (m, n, k)
+        assert lib.dmm_gemv_kernel_name(33, N, 4096) == b""
         assert lib.dmm_gemv_kernel_name(2, 4096, K) == b"dmm::gemv_regx_kernel"       # one tile per CU, short x
         assert lib.dmm_gemv_kernel_name(2, 4096, 8192) == b"dmm::gemv_stream_kernel"
         assert lib.dmm_gemv_kernel_name(3, 4096, 28672) == b"dmm::gemv_regx_kernel"
-        assert lib.dmm_gemv_kernel_name(32, N, K) == b"dmm::gemv_regx_kernel"
         assert lib.dmm_gemv_kernel_name(M, N, 264) == b""
         y8 = c_matmul(dev(x), dev(codes), dev(grid), scale, "auto")
         assert torch.equal(y8, c_matmul(dev(x), dev(codes), dev(grid), scale, "gemv8"))
@@ -409,8 +417,8 @@ def test_integer_bridge_is_exact(path, M, N, K):
     yi = orc.decode_matmul_i32(x, codes, cb)
     scale = 2.0 ** -8
     want = (yi.astype(np.float64) / 4 * scale).astype(np.float16)
-    if path == "gemv" and M >= 12:   # x too large for the LDS, or more than 16 rows of it: the small-batch kernel and its passes
-        assert capi.lib().dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_regx_kernel"
+    if path == "gemv" and M >= 12:   # nine to sixteen rows: the kernel with resident sums; 32 on one tile per CU: the small-batch kernel's passes
+        assert capi.lib().dmm_gemv_kernel_name(M, N, K) == (b"dmm::gemv_f16d_kernel" if M <= 16 else b"dmm::gemv_regx_kernel")
     y = c_matmul(dev(x.astype(np.float16)), dev(codes), dev(orc.grid_from_codebook(cb)), scale, path)
     torch.cuda.synchronize()
     assert np.array_equal(bits(y), bits(want))
@@ -442,16 +450,23 @@ def test_gemv_8bit_every_share_of_tiles_is_exact(N, K):
 @pytest.mark.parametrize("M,N,K", [(2, 6000, 16384), (4, 4112, 8448), (4, 12272, 7168), (3, 16400, 11008), (4, 20000, 8192),
                                    (2, 24592, 16384), (4, 28672, 8192), (4, 32768, 7168), (2, 8192, 28672), (3, 4100, 28672),
                                    (8, 4112, 8192), (6, 20000, 4096), (8, 28672, 4096), (5, 8192, 28672), (8, 12272, 256),
-                                   (7, 32768, 512), (1, 16400, 4352), (5, 24592, 1280)])
+                                   (7, 32768, 512), (1, 16400, 4352), (5, 24592, 1280),
+                                   # nine to sixteen rows: eight waves with pieces of sixteen rows
+                                   (16, 8192, 8192), (9, 4112, 28672), (12, 12272, 2304), (16, 16400, 4096), (13, 20000, 1280),
+                                   (10, 24592, 768), (16, 28672, 8192), (11, 32768, 256), (15, 10240, 8192),
+                                   # seventeen to 32 rows: two groups of sixteen, one decode for both
+                                   (17, 8192, 8192), (32, 4112, 28672), (24, 12272, 2304), (32, 28672, 8192), (20, 16400, 256),
+                                   (31, 32768, 512), (32, 11008, 4096), (25, 20000, 1280), (18, 4096, 4096)])
 def test_chunked_16bit_kernel_is_exact(M, N, K):
-    """Up to eight rows of x on the 16-bit kernel with resident sums, exactly (the integer bridge): both widths
-    of the x slice (up to four and up to eight rows, full and with rows to spare), workgroups of one to eight row
+    """Up to 32 rows of x on the 16-bit kernel with resident sums, exactly (the integer bridge): all widths
+    of the x slice (up to four, eight and sixteen rows and two groups of sixteen, full and with rows to spare), workgroups of one to eight row
     tiles (launches of two to eight per workgroup at most), one to seven chunks with a last chunk that is not
     full, fewer k steps than waves, one row of x with the 8-bit kernels switched off.  Reference: the library's own decode
     (pinned bit for bit against the oracle above) times x in fp64 on the GPU, which is exact for these
     integers, plus the oracle's integer product on the first and last rows of W."""
     lib = capi.lib()
     was = lib.dmm_set_gemv_8bit(0 if M == 1 else 1)
+    was_choice = lib.dmm_set_choice(2, 1 if M > 16 else -1)   # more than sixteen rows: also where the operator would not
     try:
         assert lib.dmm_gemv_kernel_name(M, N, K) == b"dmm::gemv_f16d_kernel"
         rng = np.random.default_rng(M + N + K)
@@ -467,6 +482,7 @@ def test_chunked_16bit_kernel_is_exact(M, N, K):
         c_matmul(xd, codes, gd, scale, "gemv", out=y)
     finally:
         lib.dmm_set_gemv_8bit(was)
+        lib.dmm_set_choice(2, was_choice)
     W = c_decode(codes, gd)
     torch.cuda.synchronize()
     want = ((xd.double() @ W.double().T) * scale).to(torch.float16)
@@ -751,7 +767,7 @@ def test_matrix_matrix_with_y_only_2_byte_aligned(M, N, K):
 @pytest.mark.parametrize("M,K", [(8, 4096), (16, 4096), (3, 28672), (12, 1024 * 5), (2, 28672), (5, 16384), (9, 8192),
                                  (4, 4096), (4, 3328)])
 @pytest.mark.parametrize("share", [1, 2, 3, 4, 5, 7, 8, 9, 11])
-def test_small_batch_row_block_sizes(M, K, share):
+def test_small_batch_row_block_sizes(M, K, share, request):
     """The register-x kernel takes one to four row tiles per block, chosen from the most tiles
     a workgroup gets (`share`): every choice, with workgroups whose last block is partial and
     an N that is no multiple of 16; and every width of the x slice it moves through the LDS (up
@@ -764,6 +780,9 @@ def test_small_batch_row_block_sizes(M, K, share):
     # share of tiles it is instantiated for comes by here as well); everything else in this list to the
     # register-x kernel
     resident = M <= 8 and 2 <= share <= 8
+    if M > 8:   # nine to sixteen rows would take that kernel too (up to eight tiles per workgroup): kept off here
+        assert capi.lib().dmm_gemv_kernel_name(M, N, K) == (b"dmm::gemv_f16d_kernel" if share <= 8 else b"dmm::gemv_regx_kernel")
+        request.addfinalizer(lambda was=capi.lib().dmm_set_choice(2, 0): capi.lib().dmm_set_choice(2, was))
     assert capi.lib().dmm_gemv_kernel_name(M, N, K) == (b"dmm::gemv_f16d_kernel" if resident else b"dmm::gemv_regx_kernel")
     x, _, grid, scale = workload.make_inputs(M, 8, K, seed=share)
     g = torch.Generator(device=DEV)
@@ -786,11 +805,13 @@ def test_small_batch_row_block_sizes(M, K, share):
 @pytest.mark.parametrize("M,N,K", [(17, 4112, 8192), (24, 2052, 28672), (32, 8200, 4096), (31, 11008, 4096),
                                    (20, 500, 2304), (48, 1028, 4096), (64, 4096, 11008), (100, 2052, 8192),
                                    (128, 4112, 4096), (33, 16 * 300 - 4, 28672)])
-def test_more_than_16_rows_of_x_in_passes(M, N, K):
+def test_more_than_16_rows_of_x_in_passes(M, N, K, request):
     """More than 16 rows of x go through the small-batch kernel 16 at a time inside one launch
     (every workgroup walks its row blocks once per 16 rows); beyond 32 rows the operator takes
     that route where it beats the matrix-matrix kernel, as on these shapes.  Same tolerance, y
-    between guard bands, a last pass with rows to spare."""
+    between guard bands, a last pass with rows to spare.  (The kernel with resident sums, which
+    would serve some of these shapes up to 32 rows, is kept off.)"""
+    request.addfinalizer(lambda was=capi.lib().dmm_set_choice(2, 0): capi.lib().dmm_set_choice(2, was))
     x, _, grid, scale = workload.make_inputs(M, 8, K, seed=M)
     g = torch.Generator(device=DEV)
     g.manual_seed(M * 31 + 5)
@@ -971,11 +992,13 @@ def c_matmul_ws(x, codes, grid, scale, ws_bytes=None):
 
 @pytest.mark.parametrize("M,N,K", [(17, 512, 1088), (32, 1000, 2112), (24, 28672, 2560), (33, 514, 4096), (64, 256, 8192),
                                    (100, 771, 1088), (200, 2048, 2048), (48, 4096, 512)])
-def test_split_k_workspace_path(M, N, K):
+def test_split_k_workspace_path(M, N, K, request):
     """Short x with a workspace: K is split over several blocks per tile, fp32 partial sums
     are added in a fixed order.  Same tolerance as every other path, same bits run after run,
     also with a workspace too small for the preferred split, and the PyTorch operator (which
-    brings its own workspace) returns the same tensor."""
+    brings its own workspace) returns the same tensor.  The split is asked for: on the third shape
+    the operator's own choice is the matrix-vector kernel for up to 32 rows."""
+    request.addfinalizer(lambda was=capi.lib().dmm_set_choice(0, 2): capi.lib().dmm_set_choice(0, was))
     x, codes, grid, scale = workload.make_inputs(M, N, K, seed=M + N)
     xd, cd, gd = dev(x), dev(codes), dev(grid)
     ref = orc.matmul_f32(x.numpy(), orc.decode_f16(codes.numpy(), grid.numpy()), scale)

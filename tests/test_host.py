@@ -92,7 +92,8 @@ def test_argument_errors_are_status_codes_not_crashes():
     assert lib.dmm_workspace_bytes(48, 8192, 8192) % (48 * 8192 * 4) == 0
     assert lib.dmm_workspace_bytes(48, 8192, 8192) >= 2 * 48 * 8192 * 4
     assert lib.dmm_workspace_bytes(32, 11008, 4096) == 0          # up to 32 rows, 11 MB of codes: passes, no split
-    assert lib.dmm_workspace_bytes(32, 28672, 8192) >= 2 * 32 * 28672 * 4   # 59 MB of codes: the split pays
+    assert lib.dmm_workspace_bytes(32, 28672, 8192) == 0          # 59 MB of codes with K = 8192: one launch, every code decoded once
+    assert lib.dmm_workspace_bytes(32, 8192, 28672) >= 2 * 32 * 8192 * 4    # the same with K = 28672: the split pays
     assert lib.dmm_workspace_bytes(32, 11008, 4160) > 0           # K % 256 != 0: no small-batch kernel
     assert lib.dmm_workspace_bytes(32, 11008, 4100) == 0          # K % 64 != 0: no MFMA kernel
     assert lib.dmm_workspace_bytes(-1, 8, 64) == 0
