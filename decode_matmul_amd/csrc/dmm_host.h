@@ -449,7 +449,7 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
     const int64_t n_tiles = (N + 15) / 16, cus = cu_count();
     const int64_t share = n_tiles <= cus ? 1 : (n_tiles + cus - 1) / cus;   // most tiles a workgroup gets
     if (M == 1 && (n_tiles > cus || K >= 16384) && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
-    // Up to eight rows on launches of more than one and up to eight tiles per workgroup: the 16-bit kernel that keeps
+    // Two to sixteen rows on up to eight tiles per workgroup, and one row on two to eight: the 16-bit kernel that keeps
     // every tile's sums in registers and has each wave fetch the x of its own k steps.  It beats what served
     // before it at every such shape measured (graph launches, us, this kernel / before: M = 2 4096 -> 11008
     // 6.2 / 7.2, 8192 -> 8192 6.45 / 7.40, 8192 -> 10240 8.0 / 9.6, 8192 -> 28672 17.3 / 18.6, 28672 -> 8192 16.6 / 20.3,
@@ -457,7 +457,10 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
     // M = 8 8192 -> 10240 9.6 / 10.7, 8192 -> 28672 18.4 / 24.2, 4096 -> 22016 10.6 / 12.8; one row with the 8-bit
     // kernels off: 8192 -> 28672 16.6 / 18.0, 4096 -> 22016 9.3 / 11.3), the 8-bit kernel for two to four rows
     // included (M = 2 4096 -> 22016 9.5 / 10.4, 4096 -> 32000 10.1 / 11.75; M = 4 3072 -> 32768 9.7 / 11.8).  With
-    // one tile per workgroup it is level with them or behind (M = 1 11008 -> 4096 6.03 / 5.63, M = 4 6.31 / 6.71).
+    // one tile per workgroup it is behind for one row (11008 -> 4096 6.03 / 5.63) and 1 - 7 % ahead for two to eight
+    // (M = 2 4096 -> 4096 4.01 / 4.22, M = 4 11008 -> 4096 6.29 / 6.63, M = 8 7.95 / 8.34); nine to sixteen rows run it on
+    // eight waves with pieces of sixteen rows, ahead at every share (M = 16 4096 -> 4096 6.68 / 7.02, 4096 -> 11008
+    // 8.8 / 10.1, 8192 -> 28672 23.0 / 27.6).
     const int force = g_choice[2].load(std::memory_order_relaxed);
     // Seventeen to 32 rows: the same kernel with two MFMAs per code where a workgroup has two to eight tiles and
     // K is not short, else two passes of the small-batch kernel (graph launches, us, this kernel / passes, M = 32:
@@ -469,7 +472,7 @@ GemvKind pick_gemv(int64_t M, int64_t N, int64_t K)
         return force != 0 && rows32_resident(N, K, cus) && gemv_f16d_ok(M, N, K) ? kGemvF16d : kGemvRegx;
     }
     if (force == 1 && gemv_f16d_ok(M, N, K)) return kGemvF16d;
-    if (force != 0 && (share >= 2 || M > 8) && gemv_f16d_ok(M, N, K)) return kGemvF16d;
+    if (force != 0 && (share >= 2 || M >= 2) && gemv_f16d_ok(M, N, K)) return kGemvF16d;
     // Beyond eight tiles per workgroup: two to four rows on 8-bit operands where their x fits the LDS
     if (M >= 2 && n_tiles > 4 * cus && gemv_q8_enabled() && gemv_8bit_ok(M, N, K)) return kGemvQ8;
     // Otherwise the 16-bit streaming kernel, one tile at a time, or the small-batch kernel when x does not fit the

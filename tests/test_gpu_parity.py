@@ -329,9 +329,15 @@ def test_gemv_8bit_switch_and_kernel_name():
         for m, n, k in ((32, N, K), (17, 4096, 8192), (32, 32784, 4096)):             # short K, one tile per CU, more than eight
             assert lib.dmm_gemv_kernel_name(m, n, k) == b"dmm::gemv_regx_kernel", (m, n, k)
         assert lib.dmm_gemv_kernel_name(33, N, 4096) == b""
+        for m, n, k in ((2, 4096, K), (2, 4096, 8192), (3, 4096, 28672), (8, 16, 256)):  # two rows or more: one tile per CU too
+            assert lib.dmm_gemv_kernel_name(m, n, k) == b"dmm::gemv_f16d_kernel", (m, n, k)
+        was_choice = lib.dmm_set_choice(2, 0)                                           # ... and what serves with that kernel off
         assert lib.dmm_gemv_kernel_name(2, 4096, K) == b"dmm::gemv_regx_kernel"       # one tile per CU, short x
         assert lib.dmm_gemv_kernel_name(2, 4096, 8192) == b"dmm::gemv_stream_kernel"
         assert lib.dmm_gemv_kernel_name(3, 4096, 28672) == b"dmm::gemv_regx_kernel"
+        assert lib.dmm_gemv_kernel_name(9, N, K) == b"dmm::gemv_stream_kernel"
+        assert lib.dmm_gemv_kernel_name(32, 28672, 8192) == b"dmm::gemv_regx_kernel"
+        lib.dmm_set_choice(2, was_choice)
         assert lib.dmm_gemv_kernel_name(M, N, 264) == b""
         y8 = c_matmul(dev(x), dev(codes), dev(grid), scale, "auto")
         assert torch.equal(y8, c_matmul(dev(x), dev(codes), dev(grid), scale, "gemv8"))
@@ -779,7 +785,7 @@ def test_small_batch_row_block_sizes(M, K, share, request):
     # up to eight rows of x on two to eight tiles per workgroup go to the 16-bit kernel with resident sums (every
     # share of tiles it is instantiated for comes by here as well); everything else in this list to the
     # register-x kernel
-    resident = M <= 8 and 2 <= share <= 8
+    resident = M <= 8 and share <= 8
     if M > 8:   # nine to sixteen rows would take that kernel too (up to eight tiles per workgroup): kept off here
         assert capi.lib().dmm_gemv_kernel_name(M, N, K) == (b"dmm::gemv_f16d_kernel" if share <= 8 else b"dmm::gemv_regx_kernel")
         request.addfinalizer(lambda was=capi.lib().dmm_set_choice(2, 0): capi.lib().dmm_set_choice(2, was))
