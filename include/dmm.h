@@ -179,8 +179,8 @@ int dmm_set_gemv_8bit(int enabled);
 /* Which matrix-vector kernel the operator runs for a shape with aligned pointers, as a profiler's
  * kernel trace names it without the template arguments ("dmm::gemv_q8d_kernel" - one row of x on
  * 8-bit operands, up to eight row tiles per compute unit -, "dmm::gemv_q8c_kernel" - the same for
- * more tiles -, "dmm::gemv_q8_kernel", "dmm::gemv_stream_kernel", "dmm::gemv_f16d_kernel" - up to eight
- * rows on 16-bit operands, two to eight row tiles per compute unit -, "dmm::gemv_regx_kernel"; ""
+ * more tiles -, "dmm::gemv_q8_kernel", "dmm::gemv_stream_kernel", "dmm::gemv_f16d_kernel" - up to 32
+ * rows on 16-bit operands, up to eight row tiles per compute unit -, "dmm::gemv_regx_kernel"; ""
  * outside dmm_gemv_f16's domain).  For
  * benchmarks that report per kernel.  Static storage.  No counterpart in the reference. */
 const char *dmm_gemv_kernel_name(int64_t M, int64_t N, int64_t K);
