@@ -134,6 +134,36 @@ def test_argument_errors_are_status_codes_not_crashes():
         lib.dmm_set_choice(0, -1)
 
 
+def test_kernel_choice_queries_answer_without_a_device():
+    """dmm_gemv_kernel_name and dmm_integer_kernel_name are pure: with no device set up they answer for the
+    MI355X's 256 compute units.  The rules as documented: one row on 8-bit operands from two row tiles per
+    compute unit on; two to sixteen rows on up to eight tiles, and 17 to 32 on two to eight with K >= 2048,
+    on the 16-bit kernel with resident sums; the integer operator's kernel with resident sums for up to 8
+    rows on two to eight tiles; and the overrides of dmm_set_choice."""
+    lib = capi.lib()
+    name, iname = lib.dmm_gemv_kernel_name, lib.dmm_integer_kernel_name
+    assert name(1, 28672, 8192) == b"dmm::gemv_q8d_kernel" and name(1, 4096, 4096) == b"dmm::gemv_stream_kernel"
+    assert name(1, 32784, 4096) == b"dmm::gemv_q8c_kernel"
+    for m, n, k in ((2, 4096, 4096), (8, 28672, 8192), (9, 4096, 11008), (16, 32768, 256), (17, 11008, 4096), (32, 28672, 8192)):
+        assert name(m, n, k) == b"dmm::gemv_f16d_kernel", (m, n, k)
+    for m, n, k in ((32, 4096, 11008), (24, 16384, 1024), (16, 32784, 8192), (32, 32784, 4096)):
+        assert name(m, n, k) == b"dmm::gemv_regx_kernel", (m, n, k)
+    assert name(33, 4096, 4096) == b"" and name(1, 4096, 264) == b"" and name(1, 4098, 4096) == b""
+    assert iname(8, 28672, 8192) == b"dmm::int8d_kernel" and iname(1, 4112, 256) == b"dmm::int8d_kernel"
+    assert iname(8, 4096, 4096) == b"dmm::int8x_kernel" and iname(9, 28672, 8192) == b"dmm::int8x_kernel"
+    assert iname(2048, 4096, 4096) == b"dmm::int8g_kernel" and iname(8, 4096, 264) == b"dmm::int8_kernel"
+    try:
+        assert lib.dmm_set_choice(2, 0) == -1
+        assert name(8, 28672, 8192) == b"dmm::gemv_regx_kernel" and name(32, 28672, 8192) == b"dmm::gemv_regx_kernel"
+        assert lib.dmm_set_choice(2, 1) == 0
+        assert name(32, 4096, 11008) == b"dmm::gemv_f16d_kernel"
+        assert lib.dmm_set_choice(1, 1) == -1
+        assert iname(8, 28672, 8192) == b"dmm::int8x_kernel"
+    finally:
+        lib.dmm_set_choice(2, -1)
+        lib.dmm_set_choice(1, -1)
+
+
 def test_operator_rejects_bad_inputs_with_runtime_error():
     x = torch.zeros(1, 64, dtype=torch.float16)
     codes = torch.zeros(4, 8, dtype=torch.int16)
