@@ -49,7 +49,7 @@ MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 # WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain 256 MiB device copy
 # (x2.000 and x1.000).  39.19 MB per launch against 38,855,680 algorithmic bytes (codes, x, grid, y): 1.009.
 # The many-tile 8-bit kernel (more than eight row tiles per compute unit) runs in no leg of this file.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8d_kernel": 39192105, "dmm::gemv_f16d_kernel": 39175971,
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = {"dmm::gemv_q8d_kernel": 39186492, "dmm::gemv_f16d_kernel": 39173941,
                                  "dmm::gemv_stream_kernel": 39189916}
 GEMV_TRAFFIC_SOURCE = {k: "constant from an earlier rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command, summarised in "
                           "profiles/gemv_kernels_llama70b_batch1.md; not measured by this run (a counter run cannot share a "
