@@ -1008,8 +1008,8 @@ def dispatch_check(torch, lib, capi, workload, dev):
             extra = {"chosen_no_workspace_us": round(t0, 3), "slower_by_no_workspace": round(t0 / best2 - 1.0, 4)}
         add(check, M, K, N, times, extra)
 
-    # ---- the integer operator on up to 8 rows: the kernel with resident sums against the row-block kernel
-    for M in (1, 4, 8):
+    # ---- the integer operator on up to 16 rows: the kernel with resident sums against the row-block kernel
+    for M in (1, 4, 8, 12, 16):
         for K, N in ((4096, 11008), (8192, 8192), (8192, 10240), (8192, 28672), (28672, 8192)):
             gi = torch.Generator(device=dev)
             gi.manual_seed(5)
@@ -1027,7 +1027,7 @@ def dispatch_check(torch, lib, capi, workload, dev):
                 lib.dmm_set_choice(1, was)
             if kernel == "dmm::int8d_kernel":
                 times["resident sums"] = times["operator"]
-            add("int8, up to 8 rows", M, K, N, times, {"kernel": kernel})
+            add("int8, up to 16 rows", M, K, N, times, {"kernel": kernel})
 
     # ---- the integer operator on more than 16 rows: passes against the matrix-matrix kernel (pick_int8)
     for M in (32, 64, 128, 192, 256, 384):

@@ -103,10 +103,15 @@ const std::vector<KernelInfo> &kernel_table()
     kinfo(int8d_kernel<2, 1, 2, T>, kLdsMax, true), kinfo(int8d_kernel<3, 1, 3, T>, kLdsMax, true),                \
         kinfo(int8d_kernel<4, 1, 2, T>, kLdsMax, true), kinfo(int8d_kernel<6, 1, 3, T>, kLdsMax, true),            \
         kinfo(int8d_kernel<8, 1, 2, T>, kLdsMax, true)
-#define DMM_K_I8X(T) DMM_K_I8X_S(T, false), DMM_K_I8X_S(T, true), DMM_K_I8D(T), kinfo(int8g_kernel<T>, kI8gSmem, true)
+#define DMM_K_I8D8(T)                                                                                        \
+    kinfo(int8d_kernel<2, 1, 2, T, 8>, kLdsMax, true), kinfo(int8d_kernel<3, 1, 3, T, 8>, kLdsMax, true),          \
+        kinfo(int8d_kernel<4, 1, 2, T, 8>, kLdsMax, true), kinfo(int8d_kernel<6, 1, 3, T, 8>, kLdsMax, true),      \
+        kinfo(int8d_kernel<8, 1, 2, T, 8>, kLdsMax, true)
+#define DMM_K_I8X(T) DMM_K_I8X_S(T, false), DMM_K_I8X_S(T, true), DMM_K_I8D(T), DMM_K_I8D8(T), kinfo(int8g_kernel<T>, kI8gSmem, true)
         DMM_BOTH_LAYOUTS(DMM_K_I8X),
 #undef DMM_K_I8X
 #undef DMM_K_I8D
+#undef DMM_K_I8D8
 #undef DMM_K_I8X_S
 #undef DMM_K_GREG
 #undef DMM_K_REGX
@@ -744,23 +749,28 @@ int launch_int8g(const void *x, const void *codes, const void *cb, void *out, in
                   (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
 }
 
-// Up to 8 rows of x with two to eight row tiles per compute unit: the kernel with resident sums (graph
+// Up to 16 rows of x with two to eight row tiles per compute unit: the kernel with resident sums (graph
 // launches, us, row-block kernel / this one: M = 1 4096 -> 11008 6.9 / 5.6, 8192 -> 8192 7.5 / 6.4, 8192 -> 28672
-// 18.3 / 16.2, 28672 -> 8192 17.1 / 15.2; M = 8 7.1 / 6.0, 8.1 / 6.6, 19.2 / 18.3, 18.6 / 17.7)
+// 18.3 / 16.2, 28672 -> 8192 17.1 / 15.2; M = 8 7.1 / 6.0, 8.1 / 6.6, 19.2 / 18.3, 18.6 / 17.7; M = 16 7.7 / 6.7, 8.7 / 8.1,
+// 20.4 / 20.0, 20.0 / 19.0)
 inline bool int8d_ok(int64_t M, int64_t N, int cus)
 {
     const int64_t n_tiles = (N + 15) / 16;
-    return M >= 1 && M <= 8 && n_tiles > cus && n_tiles <= 8 * (int64_t)cus;
+    return M >= 1 && M <= 16 && n_tiles > cus && n_tiles <= 8 * (int64_t)cus;
 }
 
 template <int NT, int U, int D, bool kTiled>
 int launch_int8d_inst(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
                       hipStream_t stream)
 {
-    const size_t shmem = (size_t)2 * kI8TableBytes + 16 * kI8dPiece;
+    const size_t shmem = (size_t)2 * kI8TableBytes + 16 * i8d_piece_bytes(16);   // = 8 * i8d_piece_bytes(8)
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = cu_count();   // int8d_ok: more tiles than that, and at most NT each
-    return launch(int8d_kernel<NT, U, D, kTiled>, dim3((unsigned)wgs), dim3(1024), shmem, stream, (const int8_t *)x,
+    if (M > 8)
+        return launch(int8d_kernel<NT, U, D, kTiled, 8>, dim3((unsigned)wgs), dim3(512), shmem, stream, (const int8_t *)x,
+                      (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K,
+                      (int)(n_tiles / wgs), (int)(n_tiles % wgs));
+    return launch(int8d_kernel<NT, U, D, kTiled, 16>, dim3((unsigned)wgs), dim3(1024), shmem, stream, (const int8_t *)x,
                   (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K,
                   (int)(n_tiles / wgs), (int)(n_tiles % wgs));
 }

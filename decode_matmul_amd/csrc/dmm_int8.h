@@ -385,8 +385,9 @@ __global__ __launch_bounds__(64 * W) void int8x_kernel(const int8_t *__restrict_
 // that is its own (pieces of row m exchanged by m: no bank conflicts) into the four B operands of a tile
 // step, and keeps them for every tile; the slice of the next chunk is asked for before the tile steps of
 // this one.  No barrier between the one after the tables and the end, where the sums go through the same
-// pieces, four tiles at a time (the 128 KB of tables leave 32 KB).  Exact like int8x_kernel; a table with
-// a byte that is not 2 mod 4 goes to the scalar decode.
+// pieces, four tiles at a time (the 128 KB of tables leave 32 KB).  Nine to sixteen rows of x: eight waves with
+// pieces of sixteen rows (four load instructions per slice), a chunk of 8 k steps.  Exact like int8x_kernel; a
+// table with a byte that is not 2 mod 4 goes to the scalar decode.
 template <int kCtrl>
 __device__ __forceinline__ int dpp_shr_add_i(int v)
 {
@@ -401,15 +402,19 @@ __device__ __forceinline__ int row_sum16_i(int v)
     return dpp_shr_add_i<0x111>(v);
 }
 
-constexpr int kI8dPiece = 2048;   // LDS bytes of a wave's own piece: 8 rows x 256 bytes
+// W = 16 waves with pieces of 8 rows of x (2 KB), or 8 waves with pieces of 16 rows (4 KB): 32 KB either way
+__host__ __device__ constexpr int i8d_piece_bytes(int W) { return W == 16 ? 2048 : 4096; }
 
-template <int NT, int U, int D, bool kTiled>
-__global__ __launch_bounds__(1024) void int8d_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
+template <int NT, int U, int D, bool kTiled, int W = 16>
+__global__ __launch_bounds__(64 * W) void int8d_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
                                                      const int64_t *__restrict__ codebook_abs,
                                                      int32_t *__restrict__ out, int M, int N, int K, int tiles_q,
                                                      int tiles_r)
 {
-    constexpr int W = 16;
+    static_assert(W == 16 || W == 8, "sixteen waves for up to 8 rows of x, eight for up to 16");
+    constexpr int kPiece = i8d_piece_bytes(W);
+    constexpr int XR = kPiece / 256;   // rows of x a piece holds = columns of the product that are stored
+    constexpr int XL = XR / 4;         // load instructions per slice, four rows each
     static_assert((U * NT) % D == 0, "the ring has to divide the unrolled loop");
     static_assert(NT <= 8, "the sums of the end go through the pieces four tiles at a time, twice at most");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem_raw[];
@@ -434,15 +439,15 @@ __global__ __launch_bounds__(1024) void int8d_kernel(const int8_t *__restrict__ 
     constexpr int kOut = (int)0x80000000;
     const int xcoff = q * K + c16 * 16;
     auto x_soff = [&](int c, int i) { return c * W + wave < n_steps ? (c * W + wave) * 256 + i * 4 * K : kOut; };
-    u4_t xv[2];
+    u4_t xv[XL];
 #pragma unroll
-    for (int i = 0; i < 2; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(0, i), 0);
+    for (int i = 0; i < XL; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(0, i), 0);
     // the wave's piece: row m at m * 256, its piece p in slot p ^ m.  Writes: row 4 i + h, piece lane % 16,
-    // h = lane / 16, i.e. (xs_w ^ 64 i) + 1024 i.  Reads: row c16 % 8, piece 4 q + t, i.e. xs_r ^ 16 t (columns
-    // 8 .. 15 of the product repeat 0 .. 7 and are not stored).
-    const uint32_t piece = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + wave * kI8dPiece);
+    // h = lane / 16, i.e. (xs_w ^ 64 i) + 1024 i.  Reads: row c16 % XR, piece 4 q + t, i.e. xs_r ^ 16 t (with 8-row
+    // pieces columns 8 .. 15 of the product repeat 0 .. 7 and are not stored).
+    const uint32_t piece = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + wave * kPiece);
     const uint32_t xs_w = piece + (uint32_t)(q * 256 + ((c16 ^ q) << 4));
-    const int xr_row = c16 & 7;
+    const int xr_row = c16 & (XR - 1);
     const uint32_t xs_r = piece + (uint32_t)(xr_row * 256 + (((4 * q) ^ xr_row) << 4));
 
     const int t0 = (int)blockIdx.x * tiles_q + ((int)blockIdx.x < tiles_r ? (int)blockIdx.x : tiles_r);
@@ -520,12 +525,12 @@ __global__ __launch_bounds__(1024) void int8d_kernel(const int8_t *__restrict__ 
             const bool step_ok = (U == 1 || c < n_chunks) && c * W + wave < n_steps;
             // the slice through the wave's piece: in as loaded, out as the B operands of the four MFMAs
 #pragma unroll
-            for (int i = 0; i < 2; i++) lds_write16((xs_w ^ (uint32_t)(64 * i)) + (uint32_t)(1024 * i), xv[i]);
+            for (int i = 0; i < XL; i++) lds_write16((xs_w ^ (uint32_t)(64 * i)) + (uint32_t)(1024 * i), xv[i]);
             u4_t xb[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) xb[t] = lds_read16(xs_r ^ (uint32_t)(16 * t));
 #pragma unroll
-            for (int i = 0; i < 2; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(c + 1, i), 0);
+            for (int i = 0; i < XL; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(c + 1, i), 0);
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const int slot = (u * NT + t) % D;
@@ -560,7 +565,7 @@ __global__ __launch_bounds__(1024) void int8d_kernel(const int8_t *__restrict__ 
     }
     // the sums, four tiles at a time, through the wave's own piece: cell (tile % 4, quarter, column) at slot
     // cell ^ wave, so that the 16 lanes of a reader, one per wave, meet no bank conflict; wave w adds up
-    // columns 2 (w / 4) and 2 (w / 4) + 1 of tile w % 4 of the four
+    // XR / (W / 4) columns of tile w % 4 of the four (lanes of waves that do not exist add nothing)
 #pragma unroll
     for (int r0 = 0; r0 < NT; r0 += 4) {
         if (r0 > 0) {
@@ -569,17 +574,20 @@ __global__ __launch_bounds__(1024) void int8d_kernel(const int8_t *__restrict__ 
         }
 #pragma unroll
         for (int t = r0; t < r0 + 4 && t < NT; t++)
-            if (t < nt && c16 < 8)
-                lds_write16(piece + (uint32_t)((((((t & 3) * 4 + q) * 8 + c16) ^ wave)) << 4), __builtin_bit_cast(u4_t, acc[t]));
+            if (t < nt && c16 < XR)
+                lds_write16(piece + (uint32_t)((((((t & 3) * 4 + q) * XR + c16) ^ wave)) << 4), __builtin_bit_cast(u4_t, acc[t]));
         __syncthreads();
         const int tw = wave & 3;
         if (r0 + tw < nt) {
-            const uint32_t src = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + c16 * kI8dPiece);
+            constexpr int kCols = XR / (W / 4);   // 2 with sixteen waves, 8 with eight
+            const int sw = c16 & (W - 1);
+            const uint32_t src = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + sw * kPiece);
             const int n = (t0 + r0 + tw) * 16 + 4 * q;
 #pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const int m = 2 * (wave >> 2) + j;
-                i4_t v = __builtin_bit_cast(i4_t, lds_read16(src + (uint32_t)(((((tw * 4 + q) * 8 + m) ^ c16)) << 4)));
+            for (int j = 0; j < kCols; j++) {
+                const int m = kCols * (wave >> 2) + j;
+                i4_t v = __builtin_bit_cast(i4_t, lds_read16(src + (uint32_t)(((((tw * 4 + q) * XR + m) ^ sw)) << 4)));
+                if (W < 16 && c16 >= W) v = i4_t{0, 0, 0, 0};
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = row_sum16_i(v[e]);
                 if (c16 == 15 && m < M && n < N)   // N % 4 == 0, so the four rows are in range together

@@ -590,7 +590,7 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     with the scalar decode.  Exact against the oracle's restatement of
     /root/reference/test_decode_matmul.py:58-71."""
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    resident = M <= 8 and 2 <= -(-((N + 15) // 16) // cus) <= 8   # two to eight row tiles per compute unit
+    resident = M <= 16 and 2 <= -(-((N + 15) // 16) // cus) <= 8   # two to eight row tiles per compute unit
     assert capi.lib().dmm_integer_kernel_name(M, N, K) == (b"dmm::int8d_kernel" if resident else b"dmm::int8x_kernel")
     rng = np.random.default_rng(M * 977 + N + K)
     if table == "e8p":
@@ -616,9 +616,13 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     (4, 16 * (256 * 3 - 10), 4352, False, "e8p"), (5, 8192 + 16, 1024, True, "any"), (6, 16384, 2048, True, "e8p"),
     (7, 16 * (256 * 5 - 1), 512, False, "mod4"), (8, 16 * (256 * 6 - 100), 1280, True, "e8p"),
     (8, 28672, 256, True, "e8p"), (1, 28672, 8448, True, "e8p"), (8, 32768, 768, False, "mod4"),
-    (3, 16 * (256 * 7 + 1) - 12, 512, False, "any"), (8, 10240, 8192, True, "e8p"), (1, 16 * (256 * 4), 4096, False, "e8p")])
+    (3, 16 * (256 * 7 + 1) - 12, 512, False, "any"), (8, 10240, 8192, True, "e8p"), (1, 16 * (256 * 4), 4096, False, "e8p"),
+    # nine to sixteen rows: eight waves with pieces of sixteen rows
+    (16, 8192, 8192, True, "e8p"), (9, 4100, 2304, False, "mod4"), (12, 16 * (256 * 3 - 10), 256, True, "e8p"),
+    (16, 28672, 1280, True, "any"), (13, 16 * (256 * 5 - 1), 768, False, "e8p"), (10, 16 * (256 * 6 - 100), 512, True, "mod4"),
+    (16, 32768, 512, False, "e8p"), (15, 16384, 4352, True, "e8p")])
 def test_integer_operator_resident_sums(M, N, K, tiled, table):
-    """Up to eight rows of x with two to eight row tiles per compute unit run on the kernel that keeps the
+    """Up to sixteen rows of x with two to eight row tiles per compute unit run on the kernel that keeps the
     sums of its whole share in registers.  Exact against the oracle's decode times x in float64 (every sum
     is far below 2^53, so that product is the integer one) and, on the first and last rows of W, against
     the integer oracle itself (/root/reference/test_decode_matmul.py:58-71 restated); the row-block kernel,

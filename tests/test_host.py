@@ -138,7 +138,7 @@ def test_kernel_choice_queries_answer_without_a_device():
     """dmm_gemv_kernel_name and dmm_integer_kernel_name are pure: with no device set up they answer for the
     MI355X's 256 compute units.  The rules as documented: one row on 8-bit operands from two row tiles per
     compute unit on; two to sixteen rows on up to eight tiles, and 17 to 32 on two to eight with K >= 2048,
-    on the 16-bit kernel with resident sums; the integer operator's kernel with resident sums for up to 8
+    on the 16-bit kernel with resident sums; the integer operator's kernel with resident sums for up to 16
     rows on two to eight tiles; and the overrides of dmm_set_choice."""
     lib = capi.lib()
     name, iname = lib.dmm_gemv_kernel_name, lib.dmm_integer_kernel_name
@@ -150,7 +150,8 @@ def test_kernel_choice_queries_answer_without_a_device():
         assert name(m, n, k) == b"dmm::gemv_regx_kernel", (m, n, k)
     assert name(33, 4096, 4096) == b"" and name(1, 4096, 264) == b"" and name(1, 4098, 4096) == b""
     assert iname(8, 28672, 8192) == b"dmm::int8d_kernel" and iname(1, 4112, 256) == b"dmm::int8d_kernel"
-    assert iname(8, 4096, 4096) == b"dmm::int8x_kernel" and iname(9, 28672, 8192) == b"dmm::int8x_kernel"
+    assert iname(8, 4096, 4096) == b"dmm::int8x_kernel" and iname(17, 28672, 8192) == b"dmm::int8x_kernel"
+    assert iname(16, 28672, 8192) == b"dmm::int8d_kernel"
     assert iname(2048, 4096, 4096) == b"dmm::int8g_kernel" and iname(8, 4096, 264) == b"dmm::int8_kernel"
     try:
         assert lib.dmm_set_choice(2, 0) == -1
