@@ -1008,9 +1008,10 @@ def dispatch_check(torch, lib, capi, workload, dev):
             extra = {"chosen_no_workspace_us": round(t0, 3), "slower_by_no_workspace": round(t0 / best2 - 1.0, 4)}
         add(check, M, K, N, times, extra)
 
-    # ---- the integer operator on up to 16 rows: the kernel with resident sums against the row-block kernel
-    for M in (1, 4, 8, 12, 16):
-        for K, N in ((4096, 11008), (8192, 8192), (8192, 10240), (8192, 28672), (28672, 8192)):
+    # ---- the integer operator on up to 32 rows: the kernel with resident sums against the row-block kernel
+    for M in (1, 4, 8, 12, 16, 32):
+        for K, N in ((4096, 11008), (8192, 8192), (8192, 10240), (8192, 28672), (28672, 8192), (512, 16384), (1024, 16384),
+                     (2048, 8192)):
             gi = torch.Generator(device=dev)
             gi.manual_seed(5)
             x = torch.randint(-128, 128, (M, K), generator=gi, dtype=torch.int8, device=dev)
@@ -1020,14 +1021,13 @@ def dispatch_check(torch, lib, capi, workload, dev):
                 return lib.dmm_decode_matmul_i8(x.data_ptr(), c, cb.data_ptr(), out.data_ptr(), M, N, K, 1, s)
             times = {"operator": graph_us(i8_small, workload.code_bytes(N, K))}
             kernel = lib.dmm_integer_kernel_name(M, N, K).decode()
-            was = lib.dmm_set_choice(1, 1)
-            try:
-                times["row blocks"] = graph_us(i8_small, workload.code_bytes(N, K))
-            finally:
-                lib.dmm_set_choice(1, was)
-            if kernel == "dmm::int8d_kernel":
-                times["resident sums"] = times["operator"]
-            add("int8, up to 16 rows", M, K, N, times, {"kernel": kernel})
+            for name, value in (("row blocks", 0), ("resident sums", 1)):
+                was = lib.dmm_set_choice(3, value)
+                try:
+                    times[name] = graph_us(i8_small, workload.code_bytes(N, K))
+                finally:
+                    lib.dmm_set_choice(3, was)
+            add("int8, up to 32 rows", M, K, N, times, {"kernel": kernel})
 
     # ---- the integer operator on more than 16 rows: passes against the matrix-matrix kernel (pick_int8)
     for M in (32, 64, 128, 192, 256, 384):

@@ -163,7 +163,7 @@ int dmm_set_gemv_8bit(int enabled)
 
 int dmm_set_choice(int which, int value)
 {
-    if (which < 0 || which > 2 || value < -1 || value > 2) return DMM_ERR_BAD_SHAPE;
+    if (which < 0 || which > 3 || value < -1 || value > 2) return DMM_ERR_BAD_SHAPE;
     return g_choice[which].exchange(value, std::memory_order_relaxed);
 }
 
@@ -171,7 +171,7 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K)
 {
     switch (pick_int8(M, N, K, cu_count_or_default())) {
         case kInt8Gemm: return "dmm::int8g_kernel";
-        case kInt8Gemv: return int8_takes_resident(M, N, cu_count_or_default()) ? "dmm::int8d_kernel" : "dmm::int8x_kernel";
+        case kInt8Gemv: return int8_takes_resident(M, N, K, cu_count_or_default()) ? "dmm::int8d_kernel" : "dmm::int8x_kernel";
         default: return "dmm::int8_kernel";
     }
 }

@@ -107,11 +107,16 @@ const std::vector<KernelInfo> &kernel_table()
     kinfo(int8d_kernel<2, 1, 2, T, 8>, kLdsMax, true), kinfo(int8d_kernel<3, 1, 3, T, 8>, kLdsMax, true),          \
         kinfo(int8d_kernel<4, 1, 2, T, 8>, kLdsMax, true), kinfo(int8d_kernel<6, 1, 3, T, 8>, kLdsMax, true),      \
         kinfo(int8d_kernel<8, 1, 2, T, 8>, kLdsMax, true)
-#define DMM_K_I8X(T) DMM_K_I8X_S(T, false), DMM_K_I8X_S(T, true), DMM_K_I8D(T), DMM_K_I8D8(T), kinfo(int8g_kernel<T>, kI8gSmem, true)
+#define DMM_K_I8D8G2(T)                                                                                      \
+    kinfo(int8d_kernel<2, 1, 2, T, 8, 2>, kLdsMax, true), kinfo(int8d_kernel<3, 1, 3, T, 8, 2>, kLdsMax, true),    \
+        kinfo(int8d_kernel<4, 1, 2, T, 8, 2>, kLdsMax, true), kinfo(int8d_kernel<6, 1, 3, T, 8, 2>, kLdsMax, true), \
+        kinfo(int8d_kernel<8, 1, 2, T, 8, 2>, kLdsMax, true)
+#define DMM_K_I8X(T) DMM_K_I8X_S(T, false), DMM_K_I8X_S(T, true), DMM_K_I8D(T), DMM_K_I8D8(T), DMM_K_I8D8G2(T), kinfo(int8g_kernel<T>, kI8gSmem, true)
         DMM_BOTH_LAYOUTS(DMM_K_I8X),
 #undef DMM_K_I8X
 #undef DMM_K_I8D
 #undef DMM_K_I8D8
+#undef DMM_K_I8D8G2
 #undef DMM_K_I8X_S
 #undef DMM_K_GREG
 #undef DMM_K_REGX
@@ -394,7 +399,7 @@ int launch_gemv_regx(const void *x, const void *codes, const void *grid, float s
 // [1]: the integer operator on more than 16 rows (1 passes of the matrix-vector kernel, 2 matrix-matrix);
 // [2]: up to eight rows of x (0 never the 16-bit kernel with resident sums, 1 wherever it can run).
 // A forced kernel that cannot take the call leaves the choice to the library.
-std::atomic<int> g_choice[3] = {{-1}, {-1}, {-1}};
+std::atomic<int> g_choice[4] = {{-1}, {-1}, {-1}, {-1}};
 
 // Whether the operator may pick the 8-bit kernel: dmm_set_gemv_8bit, or DMM_GEMV_8BIT=0 in the
 // environment (read once, at the first call that needs it) for hosts that cannot call it.
@@ -749,14 +754,14 @@ int launch_int8g(const void *x, const void *codes, const void *cb, void *out, in
                   (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K);
 }
 
-// Up to 16 rows of x with two to eight row tiles per compute unit: the kernel with resident sums (graph
+// Up to 32 rows of x with two to eight row tiles per compute unit: the kernel with resident sums (graph
 // launches, us, row-block kernel / this one: M = 1 4096 -> 11008 6.9 / 5.6, 8192 -> 8192 7.5 / 6.4, 8192 -> 28672
 // 18.3 / 16.2, 28672 -> 8192 17.1 / 15.2; M = 8 7.1 / 6.0, 8.1 / 6.6, 19.2 / 18.3, 18.6 / 17.7; M = 16 7.7 / 6.7, 8.7 / 8.1,
-// 20.4 / 20.0, 20.0 / 19.0)
+// 20.4 / 20.0, 20.0 / 19.0; M = 32 10.4 / 9.3, 12.3 / 11.3, 30.4 / 24.6, 32.1 / 26.8)
 inline bool int8d_ok(int64_t M, int64_t N, int cus)
 {
     const int64_t n_tiles = (N + 15) / 16;
-    return M >= 1 && M <= 16 && n_tiles > cus && n_tiles <= 8 * (int64_t)cus;
+    return M >= 1 && M <= 32 && n_tiles > cus && n_tiles <= 8 * (int64_t)cus;
 }
 
 template <int NT, int U, int D, bool kTiled>
@@ -766,6 +771,10 @@ int launch_int8d_inst(const void *x, const void *codes, const void *cb, void *ou
     const size_t shmem = (size_t)2 * kI8TableBytes + 16 * i8d_piece_bytes(16);   // = 8 * i8d_piece_bytes(8)
     const int64_t n_tiles = (N + 15) / 16;
     const int64_t wgs = cu_count();   // int8d_ok: more tiles than that, and at most NT each
+    if (M > 16)
+        return launch(int8d_kernel<NT, U, D, kTiled, 8, 2>, dim3((unsigned)wgs), dim3(512), shmem, stream, (const int8_t *)x,
+                      (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K,
+                      (int)(n_tiles / wgs), (int)(n_tiles % wgs));
     if (M > 8)
         return launch(int8d_kernel<NT, U, D, kTiled, 8>, dim3((unsigned)wgs), dim3(512), shmem, stream, (const int8_t *)x,
                       (const uint16_t *)codes, (const int64_t *)cb, (int32_t *)out, (int)M, (int)N, (int)K,
@@ -791,11 +800,18 @@ int launch_int8d(const void *x, const void *codes, const void *cb, void *out, in
     }
 }
 
-// does the matrix-vector route of the integer operator take the kernel with resident sums?  g_choice[1] = 1
-// keeps the row-block kernel
-inline bool int8_takes_resident(int64_t M, int64_t N, int cus)
+// does the matrix-vector route of the integer operator take the kernel with resident sums?  g_choice[3]: 0 never,
+// 1 wherever it can run
+// ... from K = 1024 on for up to 16 rows (from 512 on for up to 8 rows on at most four tiles per compute unit) and
+// from K = 4096 on for 17 to 32: with fewer k steps than waves the row-block kernel is ahead (us, row blocks / this
+// kernel: M = 16 32768 x 512 6.8 / 8.0, M = 8 32768 x 512 6.6 / 7.1, M = 32 8192 x 512 5.1 / 6.6, 8192 x 2048 6.6 / 7.1;
+// but M = 8 16384 x 512 5.1 / 4.7, M = 16 16384 x 1024 6.3 / 5.8, M = 32 11008 x 4096 10.1 / 9.3, 28672 x 8192 30.8 / 24.9)
+inline bool int8_takes_resident(int64_t M, int64_t N, int64_t K, int cus)
 {
-    return int8d_ok(M, N, cus) && g_choice[1].load(std::memory_order_relaxed) != 1;
+    const int force = g_choice[3].load(std::memory_order_relaxed);
+    const int64_t share = ((N + 15) / 16 + cus - 1) / cus;
+    const int64_t k_min = M > 16 ? 4096 : M <= 8 && share <= 4 ? 512 : 1024;
+    return int8d_ok(M, N, cus) && force != 0 && (force == 1 || K >= k_min);
 }
 
 // any number of rows of x, 16 per pass
@@ -803,7 +819,7 @@ template <bool kTiled>
 int run_int8x(const void *x, const void *codes, const void *cb, void *out, int64_t M, int64_t N, int64_t K,
               hipStream_t stream)
 {
-    if (int8_takes_resident(M, N, cu_count())) return launch_int8d<kTiled>(x, codes, cb, out, M, N, K, stream);
+    if (int8_takes_resident(M, N, K, cu_count())) return launch_int8d<kTiled>(x, codes, cb, out, M, N, K, stream);
     switch (small_batch_row_block((N + 15) / 16, cu_count())) {
         case 1: return launch_int8x<1, kTiled>(x, codes, cb, out, M, N, K, stream);
         case 2: return launch_int8x<2, kTiled>(x, codes, cb, out, M, N, K, stream);

@@ -405,13 +405,16 @@ __device__ __forceinline__ int row_sum16_i(int v)
 // W = 16 waves with pieces of 8 rows of x (2 KB), or 8 waves with pieces of 16 rows (4 KB): 32 KB either way
 __host__ __device__ constexpr int i8d_piece_bytes(int W) { return W == 16 ? 2048 : 4096; }
 
-template <int NT, int U, int D, bool kTiled, int W = 16>
+// CG: groups of sixteen rows of x (1, or 2 for 17 to 32 rows on eight waves): one decode of a code feeds an MFMA per
+// group, the slices of the groups go through the wave's piece one after the other, and so do the sums at the end.
+template <int NT, int U, int D, bool kTiled, int W = 16, int CG = 1>
 __global__ __launch_bounds__(64 * W) void int8d_kernel(const int8_t *__restrict__ x, const uint16_t *__restrict__ codes,
                                                      const int64_t *__restrict__ codebook_abs,
                                                      int32_t *__restrict__ out, int M, int N, int K, int tiles_q,
                                                      int tiles_r)
 {
     static_assert(W == 16 || W == 8, "sixteen waves for up to 8 rows of x, eight for up to 16");
+    static_assert(CG == 1 || (CG == 2 && W == 8), "a second group of rows only beside a full first one");
     constexpr int kPiece = i8d_piece_bytes(W);
     constexpr int XR = kPiece / 256;   // rows of x a piece holds = columns of the product that are stored
     constexpr int XL = XR / 4;         // load instructions per slice, four rows each
@@ -439,9 +442,11 @@ __global__ __launch_bounds__(64 * W) void int8d_kernel(const int8_t *__restrict_
     constexpr int kOut = (int)0x80000000;
     const int xcoff = q * K + c16 * 16;
     auto x_soff = [&](int c, int i) { return c * W + wave < n_steps ? (c * W + wave) * 256 + i * 4 * K : kOut; };
-    u4_t xv[XL];
+    u4_t xv[CG][XL];   // load i of group g: rows 16 g + 4 i ..
 #pragma unroll
-    for (int i = 0; i < XL; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(0, i), 0);
+    for (int g = 0; g < CG; g++)
+#pragma unroll
+        for (int i = 0; i < XL; i++) xv[g][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(0, 4 * g + i), 0);
     // the wave's piece: row m at m * 256, its piece p in slot p ^ m.  Writes: row 4 i + h, piece lane % 16,
     // h = lane / 16, i.e. (xs_w ^ 64 i) + 1024 i.  Reads: row c16 % XR, piece 4 q + t, i.e. xs_r ^ 16 t (with 8-row
     // pieces columns 8 .. 15 of the product repeat 0 .. 7 and are not stored).
@@ -514,9 +519,11 @@ __global__ __launch_bounds__(64 * W) void int8d_kernel(const int8_t *__restrict_
         return;
     }
 
-    i4_t acc[NT];
+    i4_t acc[NT][CG];
 #pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = i4_t{0, 0, 0, 0};
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int g = 0; g < CG; g++) acc[t][g] = i4_t{0, 0, 0, 0};
 
     for (int c0 = 0; c0 < n_chunks; c0 += U) {
 #pragma unroll
@@ -524,13 +531,18 @@ __global__ __launch_bounds__(64 * W) void int8d_kernel(const int8_t *__restrict_
             const int c = c0 + u;
             const bool step_ok = (U == 1 || c < n_chunks) && c * W + wave < n_steps;
             // the slice through the wave's piece: in as loaded, out as the B operands of the four MFMAs
+            // (the LDS serves a wave's instructions in order: the second group's slice may follow the first one's reads)
+            u4_t xb[CG][4];
 #pragma unroll
-            for (int i = 0; i < XL; i++) lds_write16((xs_w ^ (uint32_t)(64 * i)) + (uint32_t)(1024 * i), xv[i]);
-            u4_t xb[4];
+            for (int g = 0; g < CG; g++) {
 #pragma unroll
-            for (int t = 0; t < 4; t++) xb[t] = lds_read16(xs_r ^ (uint32_t)(16 * t));
+                for (int i = 0; i < XL; i++) lds_write16((xs_w ^ (uint32_t)(64 * i)) + (uint32_t)(1024 * i), xv[g][i]);
 #pragma unroll
-            for (int i = 0; i < XL; i++) xv[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(c + 1, i), 0);
+                for (int t = 0; t < 4; t++) xb[g][t] = lds_read16(xs_r ^ (uint32_t)(16 * t));
+#pragma unroll
+                for (int i = 0; i < XL; i++)
+                    xv[g][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xcoff, x_soff(c + 1, 4 * g + i), 0);
+            }
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const int slot = (u * NT + t) % D;
@@ -556,7 +568,9 @@ __global__ __launch_bounds__(64 * W) void int8d_kernel(const int8_t *__restrict_
                     for (int i = 0; i < 4; i++) {
                         const i4_t a = i4_t{(int)(g[2 * i][0] ^ m[2 * i][0]), (int)(g[2 * i][1] ^ m[2 * i][1]),
                                             (int)(g[2 * i + 1][0] ^ m[2 * i + 1][0]), (int)(g[2 * i + 1][1] ^ m[2 * i + 1][1])};
-                        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, __builtin_bit_cast(i4_t, xb[i]), acc[t], 0, 0, 0);
+#pragma unroll
+                        for (int g2 = 0; g2 < CG; g2++)
+                            acc[t][g2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, __builtin_bit_cast(i4_t, xb[g2][i]), acc[t][g2], 0, 0, 0);
                     }
                 }
                 issue(cw[slot], c + (t + D) / NT, (t + D) % NT);   // the item D further on
@@ -567,31 +581,32 @@ __global__ __launch_bounds__(64 * W) void int8d_kernel(const int8_t *__restrict_
     // cell ^ wave, so that the 16 lanes of a reader, one per wave, meet no bank conflict; wave w adds up
     // XR / (W / 4) columns of tile w % 4 of the four (lanes of waves that do not exist add nothing)
 #pragma unroll
-    for (int r0 = 0; r0 < NT; r0 += 4) {
-        if (r0 > 0) {
-            if (r0 >= nt) break;        // uniform
-            __syncthreads();            // the readers of the round before are done with the pieces
-        }
+    for (int g = 0; g < CG; g++) {
 #pragma unroll
-        for (int t = r0; t < r0 + 4 && t < NT; t++)
-            if (t < nt && c16 < XR)
-                lds_write16(piece + (uint32_t)((((((t & 3) * 4 + q) * XR + c16) ^ wave)) << 4), __builtin_bit_cast(u4_t, acc[t]));
-        __syncthreads();
-        const int tw = wave & 3;
-        if (r0 + tw < nt) {
-            constexpr int kCols = XR / (W / 4);   // 2 with sixteen waves, 8 with eight
-            const int sw = c16 & (W - 1);
-            const uint32_t src = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + sw * kPiece);
-            const int n = (t0 + r0 + tw) * 16 + 4 * q;
+        for (int r0 = 0; r0 < NT; r0 += 4) {
+            if (r0 > 0 && r0 >= nt) break;          // uniform
+            if (g > 0 || r0 > 0) __syncthreads();   // the readers of the round before are done with the pieces
 #pragma unroll
-            for (int j = 0; j < kCols; j++) {
-                const int m = kCols * (wave >> 2) + j;
-                i4_t v = __builtin_bit_cast(i4_t, lds_read16(src + (uint32_t)(((((tw * 4 + q) * XR + m) ^ sw)) << 4)));
-                if (W < 16 && c16 >= W) v = i4_t{0, 0, 0, 0};
+            for (int t = r0; t < r0 + 4 && t < NT; t++)
+                if (t < nt && c16 < XR)
+                    lds_write16(piece + (uint32_t)((((((t & 3) * 4 + q) * XR + c16) ^ wave)) << 4), __builtin_bit_cast(u4_t, acc[t][g]));
+            __syncthreads();
+            const int tw = wave & 3;
+            if (r0 + tw < nt) {
+                constexpr int kCols = XR / (W / 4);   // 2 with sixteen waves, 8 with eight
+                const int sw = c16 & (W - 1);
+                const uint32_t src = lds_addr(smem_raw) + (uint32_t)(2 * kI8TableBytes + sw * kPiece);
+                const int n = (t0 + r0 + tw) * 16 + 4 * q;
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = row_sum16_i(v[e]);
-                if (c16 == 15 && m < M && n < N)   // N % 4 == 0, so the four rows are in range together
-                    *reinterpret_cast<i4_t *>(out + (int64_t)m * N + n) = v;
+                for (int j = 0; j < kCols; j++) {
+                    const int m = kCols * (wave >> 2) + j;
+                    i4_t v = __builtin_bit_cast(i4_t, lds_read16(src + (uint32_t)(((((tw * 4 + q) * XR + m) ^ sw)) << 4)));
+                    if (W < 16 && c16 >= W) v = i4_t{0, 0, 0, 0};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = row_sum16_i(v[e]);
+                    if (c16 == 15 && 16 * g + m < M && n < N)   // N % 4 == 0, so the four rows are in range together
+                        *reinterpret_cast<i4_t *>(out + (int64_t)(16 * g + m) * N + n) = v;
+                }
             }
         }
     }

@@ -237,7 +237,7 @@ int dmm_decode_matmul_i8(const void *x, const void *codes, const void *codebook_
 
 /* Which kernel dmm_decode_matmul_i8 takes for this shape when x, codes and out are 16-byte
  * aligned: "dmm::int8g_kernel" (matrix-matrix, many rows of x), "dmm::int8x_kernel"
- * (matrix-vector, 16 rows of x per pass), "dmm::int8d_kernel" (matrix-vector, up to 16 rows of x
+ * (matrix-vector, 16 rows of x per pass), "dmm::int8d_kernel" (matrix-vector, up to 32 rows of x
  * with two to eight 16-row tiles of W per compute unit, every tile's sums in registers) or
  * "dmm::int8_kernel" (scalar).  For tests and
  * benchmarks; no counterpart in the reference. */
@@ -249,12 +249,12 @@ const char *dmm_integer_kernel_name(int64_t M, int64_t N, int64_t K);
  * small-batch kernel, 16 rows each; 1: the matrix-matrix kernel; 2: split K, where a workspace is
  * given - dmm_workspace_bytes then answers for the split as well).  which = 1: the integer
  * operator on more than 16 rows (1: passes of the matrix-vector kernel, 2: the matrix-matrix
- * kernel) and on up to 16 rows (1: the row-block kernel where the library would take the one that
- * keeps every tile's sums in registers).  which = 2: up to 32 rows of x (0: never the 16-bit kernel that keeps every tile's
- * sums in registers, 1: wherever it can run).  value -1: the library's own choice (the default).
- * A forced kernel that cannot take a call (shape, alignment) leaves that call to the library's choice; results do not depend on
- * the setting beyond what the kernels' own summation orders differ by (the integer operator:
- * not at all).  Returns the previous value (>= -1), or DMM_ERR_BAD_SHAPE for arguments out of
+ * kernel).  which = 2: up to 32 rows of x (0: never the 16-bit kernel that keeps every tile's
+ * sums in registers, 1: wherever it can run).  which = 3: the same for the integer operator's kernel
+ * of that kind (up to 32 rows).  value -1: the library's own choice (the default).  A forced
+ * kernel that cannot take a call (shape, alignment) leaves that call to the library's choice;
+ * results do not depend on the setting beyond what the kernels' own summation orders differ by
+ * (the integer operator: not at all).  Returns the previous value (>= -1), or DMM_ERR_BAD_SHAPE for arguments out of
  * range.  No counterpart in the reference. */
 int dmm_set_choice(int which, int value);
 

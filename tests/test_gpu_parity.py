@@ -590,7 +590,8 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     with the scalar decode.  Exact against the oracle's restatement of
     /root/reference/test_decode_matmul.py:58-71."""
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    resident = M <= 16 and 2 <= -(-((N + 15) // 16) // cus) <= 8   # two to eight row tiles per compute unit
+    share = -(-((N + 15) // 16) // cus)
+    resident = M <= 32 and 2 <= share <= 8 and K >= (4096 if M > 16 else 512 if M <= 8 and share <= 4 else 1024)   # two to eight row tiles per compute unit, K not short
     assert capi.lib().dmm_integer_kernel_name(M, N, K) == (b"dmm::int8d_kernel" if resident else b"dmm::int8x_kernel")
     rng = np.random.default_rng(M * 977 + N + K)
     if table == "e8p":
@@ -620,14 +621,22 @@ def test_integer_operator_matrix_unit(M, N, K, tiled, table):
     # nine to sixteen rows: eight waves with pieces of sixteen rows
     (16, 8192, 8192, True, "e8p"), (9, 4100, 2304, False, "mod4"), (12, 16 * (256 * 3 - 10), 256, True, "e8p"),
     (16, 28672, 1280, True, "any"), (13, 16 * (256 * 5 - 1), 768, False, "e8p"), (10, 16 * (256 * 6 - 100), 512, True, "mod4"),
-    (16, 32768, 512, False, "e8p"), (15, 16384, 4352, True, "e8p")])
+    (16, 32768, 512, False, "e8p"), (15, 16384, 4352, True, "e8p"),
+    # seventeen to 32 rows: two groups of sixteen, one decode for both
+    (17, 8192, 8192, True, "e8p"), (32, 4100, 2304, False, "mod4"), (24, 16 * (256 * 3 - 10), 256, True, "e8p"),
+    (32, 28672, 1280, True, "any"), (25, 16 * (256 * 5 - 1), 768, False, "e8p"), (31, 16 * (256 * 6 - 100), 512, True, "mod4"),
+    (32, 32768, 512, False, "e8p"), (20, 16384, 4352, True, "e8p")])
 def test_integer_operator_resident_sums(M, N, K, tiled, table):
-    """Up to sixteen rows of x with two to eight row tiles per compute unit run on the kernel that keeps the
+    """Up to 32 rows of x with two to eight row tiles per compute unit run on the kernel that keeps the
     sums of its whole share in registers.  Exact against the oracle's decode times x in float64 (every sum
     is far below 2^53, so that product is the integer one) and, on the first and last rows of W, against
     the integer oracle itself (/root/reference/test_decode_matmul.py:58-71 restated); the row-block kernel,
     forced, gives the same tensor."""
-    assert capi.lib().dmm_integer_kernel_name(M, N, K) == b"dmm::int8d_kernel"
+    lib = capi.lib()
+    # the operator's own rule takes this kernel from some K on; here it is tried on the shorter K as well
+    share = -(-((N + 15) // 16) // torch.cuda.get_device_properties(0).multi_processor_count)
+    takes = K >= (4096 if M > 16 else 512 if M <= 8 and share <= 4 else 1024)
+    assert (lib.dmm_integer_kernel_name(M, N, K) == b"dmm::int8d_kernel") == takes
     rng = np.random.default_rng(M * 613 + N + K)
     if table == "e8p":
         cb = orc.build_codebook_abs()
@@ -638,8 +647,14 @@ def test_integer_operator_resident_sums(M, N, K, tiled, table):
     x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
     codes = rng.integers(-32768, 32768, size=(N, K // 8)).astype(np.int16)
     cd = dev(orc.transpose_tile(codes)) if tiled else dev(codes)
-    out = c_matmul_i8(dev(x), cd, dev(cb), tiled)
-    torch.cuda.synchronize()
+    before, before_mm = lib.dmm_set_choice(3, 1), lib.dmm_set_choice(1, 1)   # ... and not the matrix-matrix kernel
+    try:
+        assert lib.dmm_integer_kernel_name(M, N, K) in (b"dmm::int8d_kernel", b"dmm::int8g_kernel")   # (the name does not see the second override)
+        out = c_matmul_i8(dev(x), cd, dev(cb), tiled)
+        torch.cuda.synchronize()
+    finally:
+        lib.dmm_set_choice(3, before)
+        lib.dmm_set_choice(1, before_mm)
     got = out.cpu().numpy()
     rows = np.r_[0:40, N - 40:N]
     assert np.array_equal(got[:, rows], orc.decode_matmul_i32(x, codes[rows], cb))
@@ -647,13 +662,14 @@ def test_integer_operator_resident_sums(M, N, K, tiled, table):
     want = (dev(x).double() @ W.T).cpu().numpy().astype(np.int64).astype(np.int32)
     del W
     assert np.array_equal(got, want)
-    before = capi.lib().dmm_set_choice(1, 1)
+    before, before_mm = lib.dmm_set_choice(3, 0), lib.dmm_set_choice(1, 1)
     try:
-        assert capi.lib().dmm_integer_kernel_name(M, N, K) == b"dmm::int8x_kernel"
+        assert lib.dmm_integer_kernel_name(M, N, K) in (b"dmm::int8x_kernel", b"dmm::int8g_kernel")
         out2 = c_matmul_i8(dev(x), cd, dev(cb), tiled)
         torch.cuda.synchronize()
     finally:
-        capi.lib().dmm_set_choice(1, before)
+        lib.dmm_set_choice(3, before)
+        lib.dmm_set_choice(1, before_mm)
     assert torch.equal(out, out2)
 
 
