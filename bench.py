@@ -463,6 +463,34 @@ def timed_kernel(torch, lib, fn, reps):
     return sum(t) / len(t)
 
 
+GRAPH_LAUNCHES, GRAPH_WARM_REPLAYS, GRAPH_REGIONS, GRAPH_REPLAYS_PER_REGION = 24, 20, 5, 4
+
+
+def graph_launch_us(torch, launch, copies):
+    """us per launch of launch(i, stream) as replays of one HIP graph of 24 dependent launches over the rotating
+    code buffers (what a serving loop sees: the time from the end of one kernel to the end of the next, the
+    ~1.7 us between dependent launches included).  Events around regions of 4 replays (96 launches: the ~17 us a
+    region costs beyond its kernels are 0.2 us per launch), median of 5 regions after 20 replays."""
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        cap = torch.cuda.current_stream().cuda_stream
+        for i in range(GRAPH_LAUNCHES):
+            launch(i, cap)
+    for _ in range(GRAPH_WARM_REPLAYS):
+        g.replay()
+    torch.cuda.synchronize()
+    t = []
+    for _ in range(GRAPH_REGIONS):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(GRAPH_REPLAYS_PER_REGION):
+            g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        t.append(a.elapsed_time(b) * 1e3 / (GRAPH_REPLAYS_PER_REGION * GRAPH_LAUNCHES))
+    return sorted(t)[len(t) // 2]
+
+
 def hbm_read_probe(torch, lib, probs, copies, stream, steps):
     """What a kernel that only reads gets out of the memory system at the headline shapes: the
     library's read probe (same launch shape and access pattern as the batch-1 kernels, no decode)
@@ -729,8 +757,10 @@ def gemv_7b(torch, lib, capi, workload, dev, stream, rand_codes):
 
 def small_batch(torch, lib, capi, workload, dev, stream, rand_codes, shapes=None, batches=(4, 8, 16, 32)):
     """A few rows of x (the small-batch configuration's shapes by default; the headline's shapes
-    as a second leg): kernel durations by events, every launch on the next of enough code
-    buffers to stay out of the Infinity Cache."""
+    as a second leg), every launch on the next of enough code buffers to stay out of the Infinity
+    Cache: `kernel_us` is the kernel's duration by events around eager launches (box and launch
+    conditions move it by a microsecond or two), `graph_us` the time per launch of the same calls as
+    one HIP graph, which the rates are computed from."""
     rows = []
     for K, N in (workload.SMALL_BATCH if shapes is None else shapes):
         copies = max(2, -(-320 * 1000000 // workload.code_bytes(N, K)))
@@ -743,24 +773,27 @@ def small_batch(torch, lib, capi, workload, dev, stream, rand_codes, shapes=None
             ws_bytes = lib.dmm_workspace_bytes(M, N, K)
             ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
 
-            def fn(i):
+            def fn(i, s=stream):
                 st = lib.dmm_decode_matmul_ws_f16(x.data_ptr(), codes[i % copies].data_ptr(), grid.data_ptr(), scale,
-                                                  y.data_ptr(), M, N, K, ws.data_ptr(), ws_bytes, stream)
+                                                  y.data_ptr(), M, N, K, ws.data_ptr(), ws_bytes, s)
                 assert st == 0, st
             for i in range(WARM_LAUNCHES):
                 fn(i)
             t = timed_kernel(torch, lib, fn, 48)     # spans both kernels when the call splits K
-            rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3), "workspace_MB": round(ws_bytes / 1e6, 1),
-                         "GBps_code": round(workload.code_bytes(N, K) / t / 1e9, 1),
-                         "TFLOPs": round(workload.flops(M, N, K) / t / 1e12, 2)})
+            tg = graph_launch_us(torch, fn, copies) * 1e-6
+            rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3), "graph_us": round(tg * 1e6, 3),
+                         "workspace_MB": round(ws_bytes / 1e6, 1),
+                         "GBps_code": round(workload.code_bytes(N, K) / tg / 1e9, 1),
+                         "TFLOPs": round(workload.flops(M, N, K) / tg / 1e12, 2)})
     return rows
 
 
 def integer_operator(torch, lib, capi, workload, dev, stream, rand_codes):
     """The reference's own operator (int8 x, int16 codes in its tile order, int64 table -> int32,
     dmm_decode_matmul_i8) at the headline shapes, M = 1 and M = 8 (the reference asks for M % 8
-    == 0).  Kernel durations by events; every launch reads the next of enough code buffers to
-    stay out of the Infinity Cache.  Random 16-bit codes are equally random in either layout."""
+    == 0).  `kernel_us`: kernel durations by events around eager launches; `graph_us`: per launch of
+    the same calls as one HIP graph (the rates are computed from it); every launch reads the next of
+    enough code buffers to stay out of the Infinity Cache.  Random 16-bit codes are equally random in either layout."""
     from decode_matmul_amd import codebook
     cb = codebook.build_codebook_abs().to(dev)
     rows = []
@@ -773,16 +806,17 @@ def integer_operator(torch, lib, capi, workload, dev, stream, rand_codes):
             x = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8, device=dev)
             out = torch.empty(M, N, dtype=torch.int32, device=dev)
 
-            def fn(i):
+            def fn(i, s=stream):
                 st = lib.dmm_decode_matmul_i8(x.data_ptr(), codes[i % copies].data_ptr(), cb.data_ptr(), out.data_ptr(),
-                                              M, N, K, 1, stream)
+                                              M, N, K, 1, s)
                 assert st == 0, st
             for i in range(WARM_LAUNCHES):
                 fn(i)
             t = timed_kernel(torch, lib, fn, 40)
-            rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3),
-                         "GBps_code": round(workload.code_bytes(N, K) / t / 1e9, 1),
-                         "frac_hbm": round(workload.code_bytes(N, K) / t / 1e9 / HBM_PEAK_GBS, 4),
+            tg = graph_launch_us(torch, fn, copies) * 1e-6
+            rows.append({"M": M, "K": K, "N": N, "kernel_us": round(t * 1e6, 3), "graph_us": round(tg * 1e6, 3),
+                         "GBps_code": round(workload.code_bytes(N, K) / tg / 1e9, 1),
+                         "frac_hbm": round(workload.code_bytes(N, K) / tg / 1e9 / HBM_PEAK_GBS, 4),
                          "kernel": lib.dmm_integer_kernel_name(M, N, K).decode()})
         del codes
     # M = 2048 at the prefill shapes: the int8 matrix-matrix kernel (2 M N K integer operations)
